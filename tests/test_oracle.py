@@ -1,0 +1,318 @@
+"""Pins the CPU oracle (oracle/hyper_oracle.py) with checks that do not re-type its formulas:
+closed forms, library routines, brute-force per-row loops on tiny inputs, and invariants."""
+import math
+from fractions import Fraction
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import hyper_oracle as O
+
+
+def _rand(shape, seed, dtype=torch.float16):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randn(shape, generator=g).to(dtype)
+
+
+# ------------------------------------------------------------------------------ gray LUT
+@pytest.mark.parametrize("r", range(1, 11))
+def test_gray_lut_closed_form(r):
+    lut = O.gray_lut(r)
+    i = np.arange(1 << r)
+    assert lut.dtype == np.int32
+    assert np.array_equal(lut, i ^ (i >> 1))
+    # neighbours differ in exactly one bit (unit Hamming distance), and it is a permutation
+    diff = lut[1:] ^ lut[:-1]
+    assert all(bin(int(x)).count("1") == 1 for x in diff)
+    assert sorted(lut.tolist()) == list(range(1 << r))
+
+
+def test_gray_lut_rejects_non_positive():
+    with pytest.raises(ValueError):
+        O.gray_lut(0)
+
+
+# ---------------------------------------------------------------------------------- hash
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_hash_against_exact_rationals(dtype):
+    x = _rand((1, 2, 40, 16), 1, dtype)
+    p = _rand((16, 5), 2, dtype)
+    got = O.lsh_hash(x, p)
+    assert got.shape == (1, 2, 40) and got.dtype == np.int32
+    xf = x.double().numpy()
+    pf = p.double().numpy()
+    for h in range(2):
+        for i in range(40):
+            bin_id = 0
+            for j in range(5):
+                acc = sum(Fraction(float(a)) * Fraction(float(b)) for a, b in zip(xf[0, h, i], pf[:, j]))
+                if acc > 0:
+                    bin_id |= 1 << j
+            assert got[0, h, i] == bin_id ^ (bin_id >> 1)
+
+
+def test_hash_zero_and_cancelling_rows():
+    # an all-zero row and a row whose projection cancels exactly give bit 0 ("> 0" is strict)
+    p = torch.tensor([[1.0, 1.0], [1.0, -1.0]], dtype=torch.float16)
+    x = torch.tensor([[0.0, 0.0], [1.0, -1.0], [1.0, 1.0], [-1.0, -1.0]], dtype=torch.float16).view(1, 1, 4, 2)
+    # dots: row0 (0,0) -> bin 0; row1 (0,2) -> bin 2; row2 (2,0) -> bin 1; row3 (-2,0) -> bin 0
+    assert O.lsh_hash(x, p).ravel().tolist() == [0, 3, 1, 0]
+
+
+def test_hash_near_cancellation_uses_exact_sign():
+    # 1 + 2^-11 is not representable in fp16 but the fp64 products here cancel to +-2^-24;
+    # build a row where the float64 sum of 3 terms is tiny compared with the terms
+    big = 2.0 ** 15
+    x = np.array([[big, -big, 2.0 ** -24]], dtype=np.float64).reshape(1, 1, 1, 3)
+    p = np.array([[big], [big], [2.0 ** -24]], dtype=np.float64)
+    assert O.lsh_hash(x, p).ravel().tolist() == [1]
+    p2 = np.array([[big], [big], [-(2.0 ** -24)]], dtype=np.float64)
+    assert O.lsh_hash(x, p2).ravel().tolist() == [0]
+
+
+def test_hash_invariants():
+    x = _rand((2, 3, 257, 64), 3)
+    p = _rand((64, 8), 4)
+    h0 = O.lsh_hash(x, p)
+    assert h0.min() >= 0 and h0.max() < 256
+    # positive scaling by a power of two is exact in fp16 and keeps every sign
+    assert np.array_equal(O.lsh_hash(x * 4, p), h0)
+    # negation flips every bit when no projection is exactly zero: bin -> 255 - bin
+    inv = np.argsort(O.gray_lut(8))
+    bins = inv[h0]
+    bins_neg = inv[O.lsh_hash(-x, p)]
+    assert np.array_equal(bins + bins_neg, np.full_like(bins, 255))
+
+
+def test_hash_per_head_projection():
+    x = _rand((2, 2, 33, 8), 5)
+    p = _rand((2, 2, 8, 4), 6)
+    got = O.lsh_hash(x, p)
+    for b in range(2):
+        for h in range(2):
+            assert np.array_equal(got[b, h], O.lsh_hash(x[b:b + 1, h:h + 1], p[b, h])[0, 0])
+
+
+# ---------------------------------------------------------------------------------- sort
+def test_stable_argsort_bruteforce():
+    rng = np.random.default_rng(0)
+    buckets = rng.integers(0, 7, size=(2, 3, 200)).astype(np.int32)
+    got = O.stable_bucket_argsort(buckets)
+    for b in range(2):
+        for h in range(3):
+            row = buckets[b, h]
+            rank = [sum(1 for j in range(200) if (row[j], j) < (row[i], i)) for i in range(200)]
+            want = np.empty(200, dtype=np.int64)
+            want[rank] = np.arange(200)
+            assert np.array_equal(got[b, h], want)
+    ref = torch.sort(torch.from_numpy(buckets), dim=2, stable=True)[1].numpy()
+    assert np.array_equal(got, ref)
+
+
+# -------------------------------------------------------------------------------- gather
+def test_gather_rows_loop_and_padding():
+    x = _rand((2, 2, 10, 4), 7, torch.float32)
+    idx = torch.randint(0, 10, (2, 2, 6), generator=torch.Generator().manual_seed(8))
+    got = O.gather_rows(x, idx)
+    for b in range(2):
+        for h in range(2):
+            for s in range(6):
+                assert torch.equal(got[b, h, s], x[b, h, idx[b, h, s]])
+    padded = O.gather_rows(x, idx, chunk_size=4)  # 10 % 4 != 0 -> rows padded 6 -> 8
+    assert padded.shape == (2, 2, 8, 4)
+    assert torch.equal(padded[:, :, :6], got) and padded[:, :, 6:].abs().sum() == 0
+
+
+# ----------------------------------------------------------------------- exact attention
+@pytest.mark.parametrize("causal", [False, True])
+def test_exact_attention_vs_sdpa(causal):
+    q, k, v = (_rand((2, 3, 200, 32), s, torch.float32).double() for s in (10, 11, 12))
+    out, lse = O.exact_attention(q, k, v, None, causal, q_chunk=64)
+    ref = torch.nn.functional.scaled_dot_product_attention(q, k, v, is_causal=causal)
+    assert torch.allclose(out, ref, atol=1e-12, rtol=1e-10)
+    # lse by a per-row loop
+    sc = 1 / math.sqrt(32)
+    for i in (0, 1, 77, 199):
+        kk = k[0, 1, : i + 1] if causal else k[0, 1]
+        want = torch.logsumexp((kk @ q[0, 1, i]) * sc, 0)
+        assert abs(lse[0, 1, i] - want) < 1e-12
+
+
+# -------------------------------------------------------------- block + sampled attention
+def _brute_block_sampled(q, k, v, qi, ki, block_size, sampled, scale, smooth):
+    """Row-by-row definition: the column multiset of sorted position i."""
+    nq, d = q.shape
+    nk = k.shape[0]
+    T = -(-block_size // 128)
+    out = torch.zeros(nq, v.shape[1], dtype=torch.float64)
+    lse = torch.zeros(nq, dtype=torch.float64)
+    for i in range(nq):
+        t = i // 128
+        if smooth:
+            first = t * 128 + 64 - T * 64
+            width = min(((t // T) + 1) * T * 128, nk) - (t // T) * T * 128
+            cols = [int(ki[(first + u) % nk]) for u in range(width)]
+        else:
+            lo = (t // T) * T * 128
+            cols = [int(ki[p]) for p in range(lo, min(lo + T * 128, nk))]
+        cols = cols + [int(s) for s in sampled]
+        kk = k[cols]
+        s = (kk @ q[qi[i]]) * scale
+        m = s.max()
+        w = torch.exp(s - m)
+        lse[qi[i]] = m + torch.log(w.sum())
+        out[qi[i]] = (w[:, None] * v[cols]).sum(0) / w.sum()
+    return out, lse
+
+
+@pytest.mark.parametrize("smooth", [False, True])
+@pytest.mark.parametrize("block_size,sample_size,n", [(128, 0, 256), (256, 128, 512), (256, 128, 384)])
+def test_block_sampled_bruteforce(smooth, block_size, sample_size, n):
+    q, k, v = (_rand((1, 2, n, 16), s, torch.float32).double() for s in (20, 21, 22))
+    g = torch.Generator().manual_seed(23)
+    qi = torch.stack([torch.randperm(n, generator=g) for _ in range(2)]).view(1, 2, n)
+    ki = torch.stack([torch.randperm(n, generator=g) for _ in range(2)]).view(1, 2, n)
+    sampled = torch.randint(0, n, (sample_size,), generator=g)
+    out, lse = O.block_sampled_attention(q, k, v, qi, ki, block_size, sample_size, 0.3, smooth, sampled)
+    for h in range(2):
+        bo, bl = _brute_block_sampled(q[0, h], k[0, h], v[0, h], qi[0, h], ki[0, h], block_size, sampled, 0.3, smooth)
+        assert torch.allclose(out[0, h], bo, atol=1e-11)
+        assert torch.allclose(lse[0, h], bl, atol=1e-11)
+
+
+def test_block_sampled_default_sample_is_first_rows():
+    n = 256
+    q, k, v = (_rand((1, 1, n, 8), s, torch.float32).double() for s in (30, 31, 32))
+    idn = torch.arange(n).view(1, 1, n)
+    a = O.block_sampled_attention(q, k, v, idn, idn, 128, 128)
+    b = O.block_sampled_attention(q, k, v, idn, idn, 128, 128, sampled_idx=np.arange(128))
+    assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+
+
+def test_block_sampled_reduces_to_exact():
+    n = 256
+    q, k, v = (_rand((2, 2, n, 32), s, torch.float32).double() for s in (40, 41, 42))
+    g = torch.Generator().manual_seed(43)
+    qi = torch.stack([torch.randperm(n, generator=g) for _ in range(4)]).view(2, 2, n)
+    ki = torch.stack([torch.randperm(n, generator=g) for _ in range(4)]).view(2, 2, n)
+    out, lse = O.block_sampled_attention(q, k, v, qi, ki, n, 0)
+    ref = torch.nn.functional.scaled_dot_product_attention(q, k, v)
+    assert torch.allclose(out, ref, atol=1e-12)
+    assert torch.allclose(lse, O.exact_attention(q, k, v)[1], atol=1e-12)
+
+
+def test_block_sampled_equals_merge_of_parts():
+    n = 512
+    q, k, v = (_rand((1, 2, n, 16), s, torch.float32).double() for s in (50, 51, 52))
+    g = torch.Generator().manual_seed(53)
+    qi = torch.stack([torch.randperm(n, generator=g) for _ in range(2)]).view(1, 2, n)
+    ki = torch.stack([torch.randperm(n, generator=g) for _ in range(2)]).view(1, 2, n)
+    fused, lse = O.block_sampled_attention(q, k, v, qi, ki, 256, 128)
+    blk, lse_b = O.block_sampled_attention(q, k, v, qi, ki, 256, 0)
+    smp, lse_s = O.exact_attention(q, k[:, :, :128], v[:, :, :128])
+    # exact two-way softmax merge written directly (not through the oracle's merge)
+    w = torch.exp(lse_b - torch.maximum(lse_b, lse_s)), torch.exp(lse_s - torch.maximum(lse_b, lse_s))
+    want = (blk * w[0][..., None] + smp * w[1][..., None]) / (w[0] + w[1])[..., None]
+    assert torch.allclose(fused, want, atol=1e-12)
+    assert torch.allclose(lse, torch.logaddexp(lse_b, lse_s), atol=1e-12)
+
+
+def test_block_sampled_value_dim_may_differ():
+    n = 256
+    q, k = (_rand((1, 1, n, 16), s, torch.float32).double() for s in (60, 61))
+    v = _rand((1, 1, n, 8), 62, torch.float32).double()
+    idn = torch.arange(n).view(1, 1, n)
+    out, _ = O.block_sampled_attention(q, k, v, idn, idn, 128, 128)
+    assert out.shape == (1, 1, n, 8)
+
+
+# ----------------------------------------------------------------------------- lse merge
+def test_merge_of_disjoint_key_sets_is_attention_over_union():
+    q, k, v = (_rand((1, 2, 64, 16), s, torch.float32).double() for s in (70, 71, 72))
+    a1, l1 = O.exact_attention(q, k[:, :, :40], v[:, :, :40])
+    a2, l2 = O.exact_attention(q, k[:, :, 40:], v[:, :, 40:])
+    attn, lse = O.add_self_attentions(a1, l1.unsqueeze(-1), a2, l2.unsqueeze(-1))
+    ref, lref = O.exact_attention(q, k, v)
+    assert torch.allclose(attn, ref, atol=1e-12)
+    assert torch.allclose(lse.squeeze(-1), lref, atol=1e-12)
+
+
+def test_merge_low_precision_matches_high_precision_within_bound():
+    # c is rounded to the attention dtype (src/attn_utils.py:21): stays within the 2e-3 band
+    q, k, v = (_rand((1, 2, 128, 64), s, torch.float16) for s in (73, 74, 75))
+    a1, l1 = O.exact_attention(q, k[:, :, :64], v[:, :, :64])
+    a2, l2 = O.exact_attention(q, k[:, :, 64:], v[:, :, 64:])
+    hi, lhi = O.add_self_attentions(a1, l1.unsqueeze(-1), a2, l2.unsqueeze(-1))
+    lo, llo = O.add_self_attentions(a1.half(), l1.float().unsqueeze(-1), a2.half(), l2.float().unsqueeze(-1))
+    assert (lo.double() - hi).norm() / hi.norm() < 2e-3
+    assert (llo.double() - lhi).abs().max() < 2e-3 * lhi.abs().max().clamp(min=1)
+
+
+# --------------------------------------------------------------------- causal recursion
+def _p(seed, d=16, r=4):
+    return _rand((d, r), seed, torch.float32).double()
+
+
+def test_forward_small_n_is_exact_causal():
+    q, k, v = (_rand((1, 2, 200, 16), s, torch.float32).double() for s in (80, 81, 82))
+    attn, lse = O.hyper_forward(q, k, v, _p(83), causal=True, min_seq_len=256)
+    ref = torch.nn.functional.scaled_dot_product_attention(q, k, v, is_causal=True)
+    assert torch.allclose(attn, ref, atol=1e-12) and lse.shape == (1, 2, 200, 1)
+
+
+@pytest.mark.parametrize("n", [512, 511, 300])
+def test_forward_one_level_full_block_is_exact_causal(n):
+    # one split; the un-masked part sees every first-half key (block = half or exact branch)
+    q, k, v = (_rand((1, 2, n, 16), s, torch.float32).double() for s in (84, 85, 86))
+    half = (n + 1) // 2
+    hyper = half % 128 == 0
+    attn, lse = O.hyper_forward(q, k, v, _p(87), causal=True, lsh_num_projs=4,
+                                block_size=half if hyper else 128, sample_size=0,
+                                min_seq_len=half if hyper else half + 1)
+    ref, lref = O.exact_attention(q, k, v, None, True)
+    assert torch.allclose(attn, ref, atol=1e-10)
+    assert torch.allclose(lse.squeeze(-1), lref, atol=1e-6)  # "+eps" inside the merge's log
+
+
+def test_forward_non_causal_thresholds():
+    q, k, v = (_rand((1, 1, 256, 16), s, torch.float32).double() for s in (88, 89, 90))
+    # min_seq_len > n -> exact; min_seq_len == n -> hashed path (hyper_attention.py:109 is strict)
+    a, _ = O.hyper_forward(q, k, v, _p(91), causal=False, min_seq_len=257, block_size=128, sample_size=0, lsh_num_projs=4)
+    assert torch.allclose(a, torch.nn.functional.scaled_dot_product_attention(q, k, v), atol=1e-12)
+    b, _ = O.hyper_forward(q, k, v, _p(91), causal=False, min_seq_len=256, block_size=128, sample_size=0, lsh_num_projs=4)
+    assert not torch.allclose(b, a, atol=1e-3)
+
+
+def test_forward_causal_bruteforce_definition():
+    """Row i = exact causal inside its leaf, plus (block U sampled) of each level's first half."""
+    n, d, r, msl, blk, smp = 1024, 16, 4, 256, 128, 128
+    q, k, v = (_rand((1, 1, n, d), s, torch.float32).double() for s in (92, 93, 94))
+    proj = _p(95, d, r)
+    attn, lse = O.hyper_forward(q, k, v, proj, scale=0.25, causal=True, lsh_num_projs=r, block_size=blk,
+                                sample_size=smp, min_seq_len=msl)
+    hq = O.lsh_hash(q, proj)[0, 0]
+    hk = O.lsh_hash(k, proj)[0, 0]
+    Q, K, V = q[0, 0], k[0, 0], v[0, 0]
+    # levels: segments of length 1024 and 512 are split; leaves have length 256
+    for i in (0, 255, 256, 300, 511, 512, 700, 800, 1023):
+        cols = list(range((i // msl) * msl, i + 1))  # leaf: exact causal
+        seg = n
+        while seg > msl:
+            base = (i // seg) * seg
+            half = seg // 2
+            if i - base >= half:  # second half at this level
+                qrows = np.arange(base + half, base + seg)
+                krows = np.arange(base, base + half)
+                qperm = qrows[np.argsort(hq[qrows], kind="stable")]
+                kperm = krows[np.argsort(hk[krows], kind="stable")]
+                pos = int(np.nonzero(qperm == i)[0][0])
+                blkid = pos // blk
+                cols += kperm[blkid * blk:(blkid + 1) * blk].tolist()
+                cols += list(range(base, base + smp))
+            seg //= 2
+        s = (K[cols] @ Q[i]) * 0.25
+        want_lse = torch.logsumexp(s, 0)
+        want = (torch.softmax(s, 0)[:, None] * V[cols]).sum(0)
+        assert torch.allclose(attn[0, 0, i], want, atol=1e-9)
+        assert abs(lse[0, 0, i, 0] - want_lse) < 1e-5
