@@ -1,0 +1,7 @@
+"""MI355X-native HyperAttention forward path (HIP kernels behind the reference's module API)."""
+from .hyper_attention import HyperAttention
+from .angular_lsh import AngularLSH, AngularLSHTriton
+from .ops import (add_self_attentions, bucket_argsort, flash_attn_func, hyper_attn_func, indexing, lsh_hash)
+
+__all__ = ["HyperAttention", "AngularLSH", "AngularLSHTriton", "add_self_attentions", "bucket_argsort",
+           "flash_attn_func", "hyper_attn_func", "indexing", "lsh_hash"]

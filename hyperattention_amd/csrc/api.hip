@@ -1,0 +1,349 @@
+// C entry points for the attention operators and the whole-forward orchestration.
+// Argument checks mirror the reference's assertions (src/hyper_attn_triton.py:678-695, :911,
+// src/flash_attn_triton.py:797-804, hyper_attention.py:45); nothing is launched when a check fails.
+#include "ha_common.h"
+#include "attn_fwd.h"
+#include "bucket_sort.h"
+
+#include <math.h>
+
+char* ha_error_buffer() {
+  static thread_local char buf[512] = {0};
+  return buf;
+}
+
+extern "C" int ha_abi_version(void) { return HA_ABI_VERSION; }
+extern "C" const char* ha_last_error(void) { return ha_error_buffer(); }
+
+namespace {
+
+constexpr float LOG2E_F = 1.4426950408889634f;
+
+int check_operands(const ha_attn_operands& t, const char* who) {
+  HA_REQUIRE(t.q && t.k && t.v && t.out && t.lse, HA_ERR_NULL, "%s: null tensor pointer", who);
+  HA_REQUIRE(t.dtype == HA_F16 || t.dtype == HA_BF16, HA_ERR_DTYPE, "%s: Only support fp16 and bf16", who);
+  HA_REQUIRE(t.batch > 0 && t.heads > 0 && t.n_q > 0 && t.n_k > 0, HA_ERR_SHAPE, "%s: sizes must be positive", who);
+  HA_REQUIRE(t.n_q < (1ll << 30) && t.n_k < (1ll << 30), HA_ERR_SHAPE, "%s: sequence too long", who);
+  HA_REQUIRE(t.d <= 128, HA_ERR_HEADDIM, "%s: FlashAttention only support head dimensions up to 128", who);
+  HA_REQUIRE(t.d == 64 || t.d == 128, HA_ERR_UNSUPPORTED, "%s: head dim %lld not built (64 and 128 are)", who,
+             (long long)t.d);
+  HA_REQUIRE(t.dv == t.d, HA_ERR_UNSUPPORTED, "%s: value head dim must equal the key head dim in this build", who);
+  HA_REQUIRE(t.segs >= 1 && t.kv_group >= 1 && t.heads % t.kv_group == 0, HA_ERR_SHAPE,
+             "%s: segs >= 1 and kv_group dividing heads required", who);
+  HA_REQUIRE(t.scale > 0.f && isfinite(t.scale), HA_ERR_SHAPE, "%s: softmax scale must be positive and finite", who);
+  const int64_t strides[] = {t.q_stride_b, t.q_stride_h, t.q_stride_n, t.k_stride_b, t.k_stride_h, t.k_stride_n,
+                             t.v_stride_b, t.v_stride_h, t.v_stride_n, t.o_stride_b, t.o_stride_h, t.o_stride_n};
+  for (int64_t s : strides) HA_REQUIRE(s % 8 == 0, HA_ERR_SHAPE, "%s: rows must be 16-byte aligned", who);
+  HA_REQUIRE(((uintptr_t)t.q % 16) == 0 && ((uintptr_t)t.k % 16) == 0 && ((uintptr_t)t.v % 16) == 0 &&
+                 ((uintptr_t)t.out % 16) == 0,
+             HA_ERR_SHAPE, "%s: tensors must be 16-byte aligned", who);
+  return HA_OK;
+}
+
+void fill_params(const ha_attn_operands& t, ha_attn_kernel_params& p) {
+  p.q = t.q; p.k = t.k; p.v = t.v; p.out = t.out; p.lse = t.lse;
+  p.q_idx = nullptr; p.k_idx = nullptr; p.sampled_idx = nullptr;
+  p.q_sb = t.q_stride_b; p.q_sh = t.q_stride_h; p.q_sn = t.q_stride_n;
+  p.k_sb = t.k_stride_b; p.k_sh = t.k_stride_h; p.k_sn = t.k_stride_n;
+  p.v_sb = t.v_stride_b; p.v_sh = t.v_stride_h; p.v_sn = t.v_stride_n;
+  p.o_sb = t.o_stride_b; p.o_sh = t.o_stride_h; p.o_sn = t.o_stride_n;
+  p.lse_sb = t.lse_stride_b; p.lse_sh = t.lse_stride_h;
+  p.qi_sb = p.qi_sh = p.qi_sn = 0;
+  p.ki_sb = p.ki_sh = p.ki_sn = 0;
+  p.si_sb = p.si_sh = 0;
+  p.seg_stride = t.seg_stride_rows; p.q_seg_off = t.q_seg_offset; p.k_seg_off = t.k_seg_offset;
+  p.batch = (int)t.batch; p.heads = (int)t.heads; p.segs = (int)t.segs; p.kv_group = (int)t.kv_group;
+  p.n_q = (int)t.n_q; p.n_k = (int)t.n_k;
+  p.block_tiles = 1; p.sample_chunks = 0; p.smooth = 0; p.accumulate = 0; p.idx64 = 0;
+  p.scale_log2 = t.scale * LOG2E_F;
+}
+
+int block_attn(const ha_block_attn_args& a, hipStream_t stream) {
+  int st = check_operands(a.t, "ha_block_attn_fwd");
+  if (st != HA_OK) return st;
+  HA_REQUIRE(a.q_idx && a.k_idx, HA_ERR_NULL, "ha_block_attn_fwd: null index pointer");
+  HA_REQUIRE(a.idx_type == HA_IDX_I32 || a.idx_type == HA_IDX_I64, HA_ERR_DTYPE, "ha_block_attn_fwd: bad idx_type");
+  HA_REQUIRE(a.t.n_k % 128 == 0, HA_ERR_SHAPE, "ha_block_attn_fwd: keys sequence length must be divisible by 128");
+  HA_REQUIRE(a.t.n_q % 128 == 0, HA_ERR_SHAPE, "ha_block_attn_fwd: query sequence length must be divisible by 128");
+  HA_REQUIRE(a.sample_size >= 0 && a.sample_size % 128 == 0, HA_ERR_SHAPE,
+             "ha_block_attn_fwd: sample_size must be a non-negative multiple of 128");
+  HA_REQUIRE(a.block_size > 0, HA_ERR_SHAPE, "ha_block_attn_fwd: block_size must be positive");
+  HA_REQUIRE(a.sampled_idx || a.sample_size <= a.t.n_k, HA_ERR_SHAPE,
+             "ha_block_attn_fwd: default sampled rows 0..sample_size-1 exceed the key length");
+  ha_attn_kernel_params p;
+  fill_params(a.t, p);
+  p.q_idx = a.q_idx; p.k_idx = a.k_idx; p.sampled_idx = a.sampled_idx;
+  p.qi_sb = a.q_idx_stride_b; p.qi_sh = a.q_idx_stride_h; p.qi_sn = a.q_idx_stride_n;
+  p.ki_sb = a.k_idx_stride_b; p.ki_sh = a.k_idx_stride_h; p.ki_sn = a.k_idx_stride_n;
+  p.si_sb = a.sampled_stride_b; p.si_sh = a.sampled_stride_h;
+  p.block_tiles = (int)((a.block_size + 127) / 128);
+  p.sample_chunks = (int)(a.sample_size / 64);
+  p.smooth = a.smooth_block != 0;
+  p.accumulate = a.accumulate != 0;
+  p.idx64 = a.idx_type == HA_IDX_I64;
+  return ha_attn_launch(p, (int)a.t.d, a.t.dtype, true, false, stream);
+}
+
+int flash_attn(const ha_attn_operands& t, int causal, int accumulate, hipStream_t stream) {
+  int st = check_operands(t, "ha_flash_attn_fwd");
+  if (st != HA_OK) return st;
+  ha_attn_kernel_params p;
+  fill_params(t, p);
+  p.accumulate = accumulate != 0;
+  return ha_attn_launch(p, (int)t.d, t.dtype, false, causal != 0, stream);
+}
+
+inline int64_t align256(int64_t v) { return (v + 255) & ~(int64_t)255; }
+
+// Static shape of the causal divide-and-conquer (hyper_attention.py:51-96): lengths per level.
+struct Plan {
+  int levels;          // number of halvings
+  int64_t len[48];     // len[j] = sequence length of a virtual head at level j; len[levels] = leaf
+  bool level_hyper[48];  // off-diagonal of level j uses the hashed kernel (else exact, hyper_attention.py:109)
+  bool any_hyper;
+};
+
+int make_plan(const ha_forward_args& a, Plan& pl) {
+  pl.levels = 0;
+  pl.any_hyper = false;
+  pl.len[0] = a.n;
+  if (!a.causal) {
+    pl.level_hyper[0] = !(a.min_seq_len > a.n);  // hyper_attention.py:109
+    pl.any_hyper = pl.level_hyper[0];
+    if (pl.any_hyper)
+      HA_REQUIRE(a.n % 128 == 0, HA_ERR_SHAPE, "ha_forward: keys sequence length must be divisible by 128");
+    return HA_OK;
+  }
+  while (pl.len[pl.levels] > a.min_seq_len) {  // hyper_attention.py:52
+    const int64_t cur = pl.len[pl.levels];
+    HA_REQUIRE(cur % 2 == 0, HA_ERR_UNSUPPORTED,
+               "ha_forward: odd length %lld inside the causal recursion; compose this shape from the operators",
+               (long long)cur);
+    const int64_t half = cur / 2;
+    pl.level_hyper[pl.levels] = !(a.min_seq_len > half);
+    if (pl.level_hyper[pl.levels]) {
+      HA_REQUIRE(half % 128 == 0, HA_ERR_SHAPE, "ha_forward: keys sequence length must be divisible by 128");
+      pl.any_hyper = true;
+    }
+    pl.len[++pl.levels] = half;
+    HA_REQUIRE(pl.levels < 40, HA_ERR_SHAPE, "ha_forward: recursion too deep");
+  }
+  return HA_OK;
+}
+
+struct Workspace {
+  int64_t buckets_q, buckets_k;        // byte offsets
+  int64_t qidx[48], kidx[48];          // per hyper level (index 0 for the non-causal case)
+  int64_t hist_q[48], hist_k[48];
+  int64_t total;
+};
+
+void layout_workspace(const ha_forward_args& a, const Plan& pl, Workspace& w) {
+  int64_t off = 0;
+  w.buckets_q = w.buckets_k = 0;
+  if (pl.any_hyper) {
+    w.buckets_q = off; off += align256(a.batch * a.heads * a.n * 4);
+    w.buckets_k = off; off += align256(a.batch * a.kv_heads * a.n * 4);
+  }
+  const int nlev = a.causal ? pl.levels : 1;
+  for (int j = 0; j < nlev; ++j) {
+    w.qidx[j] = w.kidx[j] = w.hist_q[j] = w.hist_k[j] = 0;
+    if (!pl.level_hyper[j]) continue;
+    const int64_t seg_len = a.causal ? pl.len[j] / 2 : a.n;
+    const int64_t segs = a.causal ? (1ll << j) : 1;
+    const int64_t chunks = (seg_len + HA_SORT_CHUNK - 1) / HA_SORT_CHUNK;
+    w.qidx[j] = off; off += align256(a.batch * a.heads * segs * seg_len * 4);
+    w.kidx[j] = off; off += align256(a.batch * a.kv_heads * segs * seg_len * 4);
+    w.hist_q[j] = off; off += align256(a.batch * a.heads * segs * chunks * 256 * 4);
+    w.hist_k[j] = off; off += align256(a.batch * a.kv_heads * segs * chunks * 256 * 4);
+  }
+  w.total = off > 0 ? off : 256;
+}
+
+int check_forward(const ha_forward_args& a) {
+  HA_REQUIRE(a.q && a.k && a.v && a.out && a.lse, HA_ERR_NULL, "ha_forward: null tensor pointer");
+  HA_REQUIRE(a.dtype == HA_F16 || a.dtype == HA_BF16, HA_ERR_DTYPE, "ha_forward: Only support fp16 and bf16");
+  HA_REQUIRE(a.batch > 0 && a.heads > 0 && a.kv_heads > 0 && a.n > 0, HA_ERR_SHAPE, "ha_forward: sizes must be positive");
+  HA_REQUIRE(a.heads % a.kv_heads == 0, HA_ERR_SHAPE, "ha_forward: kv_heads must divide heads");
+  HA_REQUIRE(a.n < (1ll << 30), HA_ERR_SHAPE, "ha_forward: sequence too long");
+  HA_REQUIRE(a.d <= 128, HA_ERR_HEADDIM, "ha_forward: FlashAttention only support head dimensions up to 128");
+  HA_REQUIRE(a.d == 64 || a.d == 128, HA_ERR_UNSUPPORTED, "ha_forward: head dim %lld not built (64 and 128 are)",
+             (long long)a.d);
+  HA_REQUIRE(a.dv == a.d, HA_ERR_UNSUPPORTED, "ha_forward: value head dim must equal the key head dim in this build");
+  HA_REQUIRE(a.scale > 0.f && isfinite(a.scale), HA_ERR_SHAPE, "ha_forward: softmax scale must be positive and finite");
+  HA_REQUIRE(a.block_size > 0 && a.sample_size >= 0 && a.sample_size % 128 == 0 && a.min_seq_len >= 0, HA_ERR_SHAPE,
+             "ha_forward: block_size > 0 and sample_size a non-negative multiple of 128 required");
+  return HA_OK;
+}
+
+}  // namespace
+
+extern "C" int ha_block_attn_fwd(const ha_block_attn_args* args, void* stream) {
+  HA_REQUIRE(args, HA_ERR_NULL, "ha_block_attn_fwd: null argument block");
+  return block_attn(*args, (hipStream_t)stream);
+}
+
+extern "C" int ha_flash_attn_fwd(const ha_attn_operands* t, int causal, void* stream) {
+  HA_REQUIRE(t, HA_ERR_NULL, "ha_flash_attn_fwd: null argument block");
+  return flash_attn(*t, causal, 0, (hipStream_t)stream);
+}
+
+extern "C" int64_t ha_forward_workspace_bytes(const ha_forward_args* args) {
+  if (!args) return ha_fail(HA_ERR_NULL, "ha_forward_workspace_bytes: null argument block");
+  ha_forward_args a = *args;
+  // pointers are not needed to size the workspace
+  Plan pl;
+  if (a.batch <= 0 || a.heads <= 0 || a.kv_heads <= 0 || a.n <= 0 || a.min_seq_len < 0)
+    return ha_fail(HA_ERR_SHAPE, "ha_forward_workspace_bytes: sizes must be positive");
+  int st = make_plan(a, pl);
+  if (st != HA_OK) return st;
+  Workspace w;
+  layout_workspace(a, pl, w);
+  return w.total;
+}
+
+extern "C" int ha_forward(const ha_forward_args* args, void* stream_) {
+  HA_REQUIRE(args, HA_ERR_NULL, "ha_forward: null argument block");
+  const ha_forward_args& a = *args;
+  hipStream_t stream = (hipStream_t)stream_;
+  int st = check_forward(a);
+  if (st != HA_OK) return st;
+  Plan pl;
+  st = make_plan(a, pl);
+  if (st != HA_OK) return st;
+  Workspace w;
+  layout_workspace(a, pl, w);
+  if (pl.any_hyper) {
+    HA_REQUIRE(a.proj, HA_ERR_NULL, "ha_forward: null projection matrix");
+    HA_REQUIRE(a.lsh_num_projs >= 1, HA_ERR_SHAPE, "ha_forward: Invalid value for num_projs");
+    HA_REQUIRE(a.lsh_num_projs <= 8, HA_ERR_UNSUPPORTED, "ha_forward: lsh_num_projs > 8; compose from the operators");
+    HA_REQUIRE(a.workspace && a.workspace_bytes >= w.total, HA_ERR_WORKSPACE, "ha_forward: workspace of %lld bytes needed",
+               (long long)w.total);
+  }
+  unsigned char* ws = (unsigned char*)a.workspace;
+  const int64_t group = a.heads / a.kv_heads;
+
+  // operands shared by every launch: contiguous (batch, heads, n, d) tensors
+  ha_attn_operands t;
+  t.q = a.q; t.k = a.k; t.v = a.v; t.out = a.out; t.lse = a.lse;
+  t.batch = a.batch; t.heads = a.heads; t.d = a.d; t.dv = a.dv;
+  t.q_stride_b = a.heads * a.n * a.d; t.q_stride_h = a.n * a.d; t.q_stride_n = a.d;
+  t.k_stride_b = a.kv_heads * a.n * a.d; t.k_stride_h = a.n * a.d; t.k_stride_n = a.d;
+  t.v_stride_b = a.kv_heads * a.n * a.dv; t.v_stride_h = a.n * a.dv; t.v_stride_n = a.dv;
+  t.o_stride_b = a.heads * a.n * a.dv; t.o_stride_h = a.n * a.dv; t.o_stride_n = a.dv;
+  t.lse_stride_b = a.heads * a.n; t.lse_stride_h = a.n;
+  t.kv_group = group;
+  t.scale = a.scale;
+  t.dtype = a.dtype;
+
+  // 1. bucket ids, once for the whole tensors (the projection does not depend on the level)
+  int32_t* bq = nullptr;
+  int32_t* bk = nullptr;
+  if (pl.any_hyper) {
+    bq = (int32_t*)(ws + w.buckets_q);
+    bk = (int32_t*)(ws + w.buckets_k);
+    st = ha_lsh_hash(a.q, a.proj, bq, a.batch, a.heads, a.n, a.d, a.lsh_num_projs, t.q_stride_b, t.q_stride_h,
+                     t.q_stride_n, 0, 0, a.dtype, stream);
+    if (st != HA_OK) return st;
+    st = ha_lsh_hash(a.k, a.proj, bk, a.batch, a.kv_heads, a.n, a.d, a.lsh_num_projs, t.k_stride_b, t.k_stride_h,
+                     t.k_stride_n, 0, 0, a.dtype, stream);
+    if (st != HA_OK) return st;
+
+    // 2. all segmented sorts of all levels in one batch of launches
+    ha_sort_jobs jobs;
+    jobs.num_jobs = 0;
+    jobs.shift = 0;
+    jobs.idx64 = 0;
+    int blocks = 0, segments = 0;
+    bool multi = false;
+    const int nlev = a.causal ? pl.levels : 1;
+    for (int j = 0; j < nlev; ++j) {
+      if (!pl.level_hyper[j]) continue;
+      const int64_t seg_len = a.causal ? pl.len[j] / 2 : a.n;
+      const int64_t segs = a.causal ? (1ll << j) : 1;
+      const int64_t stride = a.causal ? pl.len[j] : a.n;
+      const int64_t chunks = (seg_len + HA_SORT_CHUNK - 1) / HA_SORT_CHUNK;
+      for (int side = 0; side < 2; ++side) {
+        HA_REQUIRE(jobs.num_jobs < HA_SORT_MAX_JOBS, HA_ERR_SHAPE, "ha_forward: too many sort jobs");
+        ha_sort_job& job = jobs.job[jobs.num_jobs++];
+        const int64_t nseg = a.batch * (side == 0 ? a.heads : a.kv_heads) * segs;
+        job.keys = side == 0 ? bq : bk;
+        job.prev = nullptr;
+        job.out = ws + (side == 0 ? w.qidx[j] : w.kidx[j]);
+        job.hist = (uint32_t*)(ws + (side == 0 ? w.hist_q[j] : w.hist_k[j]));
+        job.seg_stride = stride;
+        job.seg_offset = (a.causal && side == 0) ? seg_len : 0;  // queries: second halves, keys: first halves
+        job.seg_len = (int)seg_len;
+        job.num_segments = (int)nseg;
+        job.chunks_per_seg = (int)chunks;
+        job.first_block = blocks;
+        job.first_segment = segments;
+        HA_REQUIRE(nseg * chunks + blocks < (1ll << 30), HA_ERR_SHAPE, "ha_forward: too many sort chunks");
+        blocks += (int)(nseg * chunks);
+        segments += (int)nseg;
+        multi = multi || chunks > 1;
+      }
+    }
+    st = ha_sort_launch(jobs, blocks, segments, multi, stream);
+    if (st != HA_OK) return st;
+  }
+
+  auto hyper_level = [&](int j, bool accumulate) -> int {
+    const int64_t seg_len = a.causal ? pl.len[j] / 2 : a.n;
+    const int64_t segs = a.causal ? (1ll << j) : 1;
+    ha_block_attn_args b;
+    b.t = t;
+    b.t.n_q = b.t.n_k = seg_len;
+    b.t.segs = segs;
+    b.t.seg_stride_rows = a.causal ? pl.len[j] : a.n;
+    b.t.q_seg_offset = a.causal ? seg_len : 0;
+    b.t.k_seg_offset = 0;
+    b.q_idx = ws + w.qidx[j];
+    b.k_idx = ws + w.kidx[j];
+    b.sampled_idx = a.sampled_idx;
+    b.idx_type = HA_IDX_I32;
+    b.q_idx_stride_b = a.heads * segs * seg_len; b.q_idx_stride_h = segs * seg_len; b.q_idx_stride_n = 1;
+    b.k_idx_stride_b = a.kv_heads * segs * seg_len; b.k_idx_stride_h = segs * seg_len; b.k_idx_stride_n = 1;
+    b.sampled_stride_b = b.sampled_stride_h = 0;
+    b.block_size = a.block_size;
+    b.sample_size = a.sample_size;
+    b.smooth_block = a.smooth_block;
+    b.accumulate = accumulate;
+    return block_attn(b, stream);
+  };
+
+  if (!a.causal) {
+    if (pl.level_hyper[0]) return hyper_level(0, false);
+    ha_attn_operands f = t;
+    f.n_q = f.n_k = a.n;
+    f.segs = 1; f.seg_stride_rows = a.n; f.q_seg_offset = f.k_seg_offset = 0;
+    return flash_attn(f, 0, 0, stream);
+  }
+
+  // 3. leaves: exact causal attention on every segment of the deepest level
+  {
+    ha_attn_operands f = t;
+    f.n_q = f.n_k = pl.len[pl.levels];
+    f.segs = 1ll << pl.levels;
+    f.seg_stride_rows = pl.len[pl.levels];
+    f.q_seg_offset = f.k_seg_offset = 0;
+    st = flash_attn(f, 1, 0, stream);
+    if (st != HA_OK) return st;
+  }
+  // 4. off-diagonal parts, deepest level first, merged in place into the second halves
+  for (int j = pl.levels - 1; j >= 0; --j) {
+    if (pl.level_hyper[j]) {
+      st = hyper_level(j, true);
+    } else {
+      ha_attn_operands f = t;
+      f.n_q = f.n_k = pl.len[j] / 2;
+      f.segs = 1ll << j;
+      f.seg_stride_rows = pl.len[j];
+      f.q_seg_offset = pl.len[j] / 2;
+      f.k_seg_offset = 0;
+      st = flash_attn(f, 0, 1, stream);
+    }
+    if (st != HA_OK) return st;
+  }
+  return HA_OK;
+}

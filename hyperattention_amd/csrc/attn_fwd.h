@@ -1,0 +1,32 @@
+// Device-side parameter block of the attention kernels (validated and filled by the C entry points).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+struct ha_attn_kernel_params {
+  const void* q;
+  const void* k;
+  const void* v;
+  void* out;
+  float* lse;
+  const void* q_idx;        // gather mode only
+  const void* k_idx;
+  const void* sampled_idx;  // may be null: rows 0..sample-1
+  int64_t q_sb, q_sh, q_sn;
+  int64_t k_sb, k_sh, k_sn;
+  int64_t v_sb, v_sh, v_sn;
+  int64_t o_sb, o_sh, o_sn;
+  int64_t lse_sb, lse_sh;
+  int64_t qi_sb, qi_sh, qi_sn;
+  int64_t ki_sb, ki_sh, ki_sn;
+  int64_t si_sb, si_sh;
+  int64_t seg_stride, q_seg_off, k_seg_off;
+  int batch, heads, segs, kv_group;
+  int n_q, n_k;
+  int block_tiles;    // ceil(block_size / 128)
+  int sample_chunks;  // sample_size / 64
+  int smooth, accumulate, idx64;
+  float scale_log2;   // softmax scale * log2(e)
+};
+
+int ha_attn_launch(const ha_attn_kernel_params& p, int d, int dtype, bool gather, bool causal, hipStream_t stream);

@@ -1,0 +1,265 @@
+// Segmented stable counting sort (argsort) of small integer keys.
+// Stands in for torch.sort(buckets, dim=2, stable=True) at hyper_attention.py:116-117 of the
+// reference: within every segment the output lists row numbers by non-decreasing key, ties in
+// ascending row number.
+//
+// A segment is cut into chunks of SORT_CHUNK keys, one workgroup each.  Ranking inside a wave
+// uses ballot matching (8 ballots give every lane the set of lanes holding the same 8-bit digit),
+// so skewed key distributions cost the same as uniform ones and no LDS atomics are needed for the
+// order-sensitive part.  Segments longer than one chunk use three launches (per-chunk histograms,
+// per-segment scan, scatter); shorter ones a single launch.  Keys above 255 take one extra
+// least-significant-digit pass per byte.  Several jobs (for instance all recursion levels of a
+// causal forward) share one launch through a small by-value job table.
+#include "ha_common.h"
+#include "bucket_sort.h"
+
+namespace {
+
+constexpr int SORT_THREADS = 256;
+constexpr int SORT_WAVES = SORT_THREADS / HA_WAVE;
+constexpr int SORT_STEPS = HA_SORT_CHUNK / SORT_THREADS;  // 64-key steps per wave per chunk
+
+struct BlockRef {
+  int job, seg, chunk;
+};
+
+__device__ __forceinline__ BlockRef locate_block(const ha_sort_jobs& jobs, int block, bool per_segment) {
+  int j = 0;
+  while (j + 1 < jobs.num_jobs &&
+         block >= (per_segment ? jobs.job[j + 1].first_segment : jobs.job[j + 1].first_block))
+    ++j;
+  BlockRef r;
+  r.job = j;
+  if (per_segment) {
+    r.seg = block - jobs.job[j].first_segment;
+    r.chunk = 0;
+  } else {
+    const int local = block - jobs.job[j].first_block;
+    r.seg = local / jobs.job[j].chunks_per_seg;
+    r.chunk = local % jobs.job[j].chunks_per_seg;
+  }
+  return r;
+}
+
+// lanes of the wave holding the same digit as this lane, restricted to valid lanes
+__device__ __forceinline__ uint64_t match_digit(int digit, bool valid) {
+  uint64_t mask = __ballot(valid);
+#pragma unroll
+  for (int bit = 0; bit < 8; ++bit) {
+    const bool set = (digit >> bit) & 1;
+    const uint64_t b = __ballot(set);
+    mask &= set ? b : ~b;
+  }
+  return mask;
+}
+
+__device__ __forceinline__ uint64_t lanemask_lt() {
+  const int lane = threadIdx.x & (HA_WAVE - 1);
+  return lane == 0 ? 0ull : (~0ull >> (HA_WAVE - lane));
+}
+
+// ---- per-chunk histograms (only for segments longer than one chunk) -------------------------
+__global__ __launch_bounds__(SORT_THREADS) void sort_hist_kernel(ha_sort_jobs jobs) {
+  __shared__ uint32_t hist[256];
+  const BlockRef br = locate_block(jobs, blockIdx.x, false);
+  const ha_sort_job& job = jobs.job[br.job];
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  hist[tid] = 0;
+  __syncthreads();
+  const int64_t seg_base = job.seg_offset + (int64_t)br.seg * job.seg_stride;
+  const int32_t* prev = job.prev ? job.prev + (int64_t)br.seg * job.seg_len : nullptr;
+  const int chunk_start = br.chunk * HA_SORT_CHUNK;
+  for (int s = 0; s < SORT_STEPS; ++s) {
+    const int i = chunk_start + (wave * SORT_STEPS + s) * HA_WAVE + lane;
+    const bool valid = i < job.seg_len;
+    int digit = 0;
+    if (valid) {
+      const int src = prev ? prev[i] : i;
+      digit = (job.keys[seg_base + src] >> jobs.shift) & 255;
+    }
+    const uint64_t m = match_digit(digit, valid);
+    if (valid && (m & lanemask_lt()) == 0) atomicAdd(&hist[digit], (uint32_t)__popcll(m));
+  }
+  __syncthreads();
+  job.hist[((int64_t)br.seg * job.chunks_per_seg + br.chunk) * 256 + tid] = hist[tid];
+}
+
+// exclusive scan of one value per thread over a 256-thread block
+__device__ __forceinline__ uint32_t block_exclusive_scan(uint32_t v, uint32_t* wave_totals) {
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  uint32_t incl = v;
+#pragma unroll
+  for (int off = 1; off < HA_WAVE; off <<= 1) {
+    const uint32_t up = __shfl_up(incl, off);
+    if (lane >= off) incl += up;
+  }
+  if (lane == HA_WAVE - 1) wave_totals[wave] = incl;
+  __syncthreads();
+  uint32_t base = 0;
+  for (int w = 0; w < wave; ++w) base += wave_totals[w];
+  __syncthreads();
+  return base + incl - v;
+}
+
+// ---- per-segment scan: hist[c][k] -> first output slot of (chunk c, key k) -------------------
+__global__ __launch_bounds__(SORT_THREADS) void sort_scan_kernel(ha_sort_jobs jobs) {
+  __shared__ uint32_t wave_totals[SORT_WAVES];
+  const BlockRef br = locate_block(jobs, blockIdx.x, true);
+  const ha_sort_job& job = jobs.job[br.job];
+  const int k = threadIdx.x;
+  uint32_t* h = job.hist + (int64_t)br.seg * job.chunks_per_seg * 256;
+  uint32_t running = 0;
+  for (int c = 0; c < job.chunks_per_seg; ++c) {
+    const uint32_t t = h[c * 256 + k];
+    h[c * 256 + k] = running;
+    running += t;
+  }
+  const uint32_t base = block_exclusive_scan(running, wave_totals);
+  for (int c = 0; c < job.chunks_per_seg; ++c) h[c * 256 + k] += base;
+}
+
+// ---- stable scatter --------------------------------------------------------------------------
+__global__ __launch_bounds__(SORT_THREADS) void sort_scatter_kernel(ha_sort_jobs jobs) {
+  __shared__ uint32_t wave_hist[SORT_WAVES][256];
+  __shared__ uint32_t wave_totals[SORT_WAVES];
+  const BlockRef br = locate_block(jobs, blockIdx.x, false);
+  const ha_sort_job& job = jobs.job[br.job];
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+#pragma unroll
+  for (int w = 0; w < SORT_WAVES; ++w) wave_hist[w][tid] = 0;
+  __syncthreads();
+
+  const int64_t seg_base = job.seg_offset + (int64_t)br.seg * job.seg_stride;
+  const int32_t* prev = job.prev ? job.prev + (int64_t)br.seg * job.seg_len : nullptr;
+  const int chunk_start = br.chunk * HA_SORT_CHUNK;
+  const uint64_t lt = lanemask_lt();
+
+  int digit[SORT_STEPS];
+  int src[SORT_STEPS];
+  // pass 1: per-wave digit counts (a wave owns a contiguous run of the chunk, so wave order = key order)
+#pragma unroll
+  for (int s = 0; s < SORT_STEPS; ++s) {
+    const int i = chunk_start + (wave * SORT_STEPS + s) * HA_WAVE + lane;
+    const bool valid = i < job.seg_len;
+    digit[s] = 0;
+    src[s] = -1;
+    if (valid) {
+      src[s] = prev ? prev[i] : i;
+      digit[s] = (job.keys[seg_base + src[s]] >> jobs.shift) & 255;
+    }
+    const uint64_t m = match_digit(digit[s], valid);
+    if (valid && (m & lt) == 0) wave_hist[wave][digit[s]] += (uint32_t)__popcll(m);
+  }
+  __syncthreads();
+
+  // first output slot of (this chunk, key tid): from the scan kernel, or computed here when the
+  // segment is a single chunk
+  uint32_t total = 0;
+#pragma unroll
+  for (int w = 0; w < SORT_WAVES; ++w) total += wave_hist[w][tid];
+  uint32_t base;
+  if (job.chunks_per_seg > 1) {
+    base = job.hist[((int64_t)br.seg * job.chunks_per_seg + br.chunk) * 256 + tid];
+    __syncthreads();
+  } else {
+    base = block_exclusive_scan(total, wave_totals);
+  }
+  // turn the per-wave counts into per-wave first slots
+  uint32_t run = base;
+#pragma unroll
+  for (int w = 0; w < SORT_WAVES; ++w) {
+    const uint32_t c = wave_hist[w][tid];
+    wave_hist[w][tid] = run;
+    run += c;
+  }
+  __syncthreads();
+
+  // pass 2: rank inside the wave step and scatter
+  const int64_t out_base = (int64_t)br.seg * job.seg_len;
+#pragma unroll
+  for (int s = 0; s < SORT_STEPS; ++s) {
+    const bool valid = src[s] >= 0;
+    const uint64_t m = match_digit(digit[s], valid);
+    if (valid) {
+      const uint32_t slot = wave_hist[wave][digit[s]] + (uint32_t)__popcll(m & lt);
+      if (jobs.idx64)
+        ((int64_t*)job.out)[out_base + slot] = src[s];
+      else
+        ((int32_t*)job.out)[out_base + slot] = src[s];
+    }
+    // all lanes of the wave have read their slot before the leaders advance it (same wave,
+    // LDS operations complete in program order)
+    __builtin_amdgcn_wave_barrier();
+    if (valid && (m & lt) == 0) wave_hist[wave][digit[s]] += (uint32_t)__popcll(m);
+    __builtin_amdgcn_wave_barrier();
+  }
+}
+
+}  // namespace
+
+int ha_sort_launch(const ha_sort_jobs& jobs, int total_blocks, int total_segments, bool any_multi_chunk,
+                   hipStream_t stream) {
+  if (any_multi_chunk) {
+    hipLaunchKernelGGL(sort_hist_kernel, dim3(total_blocks), dim3(SORT_THREADS), 0, stream, jobs);
+    hipLaunchKernelGGL(sort_scan_kernel, dim3(total_segments), dim3(SORT_THREADS), 0, stream, jobs);
+  }
+  hipLaunchKernelGGL(sort_scatter_kernel, dim3(total_blocks), dim3(SORT_THREADS), 0, stream, jobs);
+  return ha_launch_status("ha_bucket_argsort");
+}
+
+static inline int64_t align256(int64_t v) { return (v + 255) & ~(int64_t)255; }
+
+extern "C" int64_t ha_bucket_argsort_workspace_bytes(int64_t num_segments, int64_t seg_len, int64_t num_keys) {
+  if (num_segments <= 0 || seg_len <= 0) return 0;
+  const int64_t chunks = (seg_len + HA_SORT_CHUNK - 1) / HA_SORT_CHUNK;
+  int64_t bytes = align256(num_segments * chunks * 256 * (int64_t)sizeof(uint32_t));
+  if (num_keys > 256) bytes += 2 * align256(num_segments * seg_len * (int64_t)sizeof(int32_t));
+  return bytes;
+}
+
+extern "C" int ha_bucket_argsort(const int32_t* keys, void* idx_out, int idx_type, int64_t num_segments,
+                                 int64_t seg_len, int64_t seg_stride, int64_t seg_offset, int64_t num_keys,
+                                 void* workspace, int64_t workspace_bytes, void* stream) {
+  HA_REQUIRE(keys && idx_out, HA_ERR_NULL, "ha_bucket_argsort: null pointer");
+  HA_REQUIRE(idx_type == HA_IDX_I32 || idx_type == HA_IDX_I64, HA_ERR_DTYPE, "ha_bucket_argsort: bad idx_type");
+  HA_REQUIRE(num_segments > 0 && seg_len > 0, HA_ERR_SHAPE, "ha_bucket_argsort: sizes must be positive");
+  HA_REQUIRE(seg_len < (1ll << 31) && num_segments < (1ll << 24), HA_ERR_SHAPE, "ha_bucket_argsort: too large");
+  HA_REQUIRE(num_keys >= 1 && num_keys <= 65536, HA_ERR_UNSUPPORTED, "ha_bucket_argsort: num_keys must be in [1, 65536]");
+  const int64_t need = ha_bucket_argsort_workspace_bytes(num_segments, seg_len, num_keys);
+  HA_REQUIRE(workspace && workspace_bytes >= need, HA_ERR_WORKSPACE,
+             "ha_bucket_argsort: workspace of %lld bytes needed", (long long)need);
+  const int64_t chunks = (seg_len + HA_SORT_CHUNK - 1) / HA_SORT_CHUNK;
+  HA_REQUIRE(num_segments * chunks < (1ll << 31), HA_ERR_SHAPE, "ha_bucket_argsort: too many chunks");
+
+  ha_sort_jobs jobs;
+  jobs.num_jobs = 1;
+  ha_sort_job& j = jobs.job[0];
+  j.keys = keys;
+  j.seg_stride = seg_stride;
+  j.seg_offset = seg_offset;
+  j.seg_len = (int)seg_len;
+  j.num_segments = (int)num_segments;
+  j.chunks_per_seg = (int)chunks;
+  j.first_block = 0;
+  j.first_segment = 0;
+  j.hist = (uint32_t*)workspace;
+  unsigned char* ws = (unsigned char*)workspace + align256(num_segments * chunks * 256 * (int64_t)sizeof(uint32_t));
+  const int passes = num_keys > 256 ? 2 : 1;
+  int32_t* tmp[2] = {nullptr, nullptr};
+  if (passes > 1) {
+    tmp[0] = (int32_t*)ws;
+    tmp[1] = (int32_t*)(ws + align256(num_segments * seg_len * (int64_t)sizeof(int32_t)));
+  }
+  const int32_t* prev = nullptr;
+  for (int p = 0; p < passes; ++p) {
+    const bool last = p == passes - 1;
+    j.prev = prev;
+    j.out = last ? idx_out : (void*)tmp[p & 1];
+    jobs.shift = 8 * p;
+    jobs.idx64 = last && idx_type == HA_IDX_I64;
+    int st = ha_sort_launch(jobs, (int)(num_segments * chunks), (int)num_segments, chunks > 1, (hipStream_t)stream);
+    if (st != HA_OK) return st;
+    prev = tmp[p & 1];
+  }
+  return HA_OK;
+}

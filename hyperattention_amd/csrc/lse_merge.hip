@@ -1,0 +1,57 @@
+// Merge of two partial attentions computed over disjoint key sets.
+// Stands in for add_self_attentions (src/attn_utils.py:6-24 of the reference):
+//   c = 1 / (1 + exp(lse2 - lse1)); attn = c*attn1 + (1-c)*attn2; lse = lse1 - log(c + eps).
+// The arithmetic here is fp32 throughout (the reference rounds c to fp16/bf16 first), with the
+// same eps = 2^-23 inside the log.  One 8-element piece (16 bytes) per lane.
+#include "ha_common.h"
+
+namespace {
+
+template <typename T>
+__global__ __launch_bounds__(256) void lse_merge_kernel(const T* __restrict__ a1, const float* __restrict__ l1,
+                                                        const T* __restrict__ a2, const float* __restrict__ l2,
+                                                        T* __restrict__ ao, float* __restrict__ lo, int64_t rows,
+                                                        int pieces, int64_t s1, int64_t s2, int64_t so,
+                                                        int64_t ls1, int64_t ls2, int64_t lso) {
+  typedef typename ElemTraits<T>::vec8 vec8;
+  const int64_t item = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t row = item / pieces;
+  const int piece = (int)(item % pieces);
+  if (row >= rows) return;
+  const float x1 = l1[row * ls1], x2 = l2[row * ls2];
+  const float c = 1.0f / (1.0f + __expf(x2 - x1));
+  const vec8 v1 = *reinterpret_cast<const vec8*>(a1 + row * s1 + piece * 8);
+  const vec8 v2 = *reinterpret_cast<const vec8*>(a2 + row * s2 + piece * 8);
+  vec8 r;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) r[e] = (T)(c * (float)v1[e] + (1.0f - c) * (float)v2[e]);
+  *reinterpret_cast<vec8*>(ao + row * so + piece * 8) = r;
+  if (piece == 0) lo[row * lso] = x1 - __logf(c + 1.1920929e-07f);
+}
+
+}  // namespace
+
+extern "C" int ha_lse_merge(const void* attn1, const float* lse1, const void* attn2, const float* lse2,
+                            void* attn_out, float* lse_out, int64_t rows, int64_t d, int64_t attn1_stride,
+                            int64_t attn2_stride, int64_t out_stride, int64_t lse1_stride, int64_t lse2_stride,
+                            int64_t lse_out_stride, int dtype, void* stream) {
+  HA_REQUIRE(attn1 && lse1 && attn2 && lse2 && attn_out && lse_out, HA_ERR_NULL, "ha_lse_merge: null pointer");
+  HA_REQUIRE(dtype == HA_F16 || dtype == HA_BF16, HA_ERR_DTYPE, "ha_lse_merge: Only support fp16 and bf16");
+  HA_REQUIRE(rows > 0 && d > 0 && d % 8 == 0, HA_ERR_SHAPE, "ha_lse_merge: rows > 0 and d % 8 == 0 required");
+  HA_REQUIRE(attn1_stride % 8 == 0 && attn2_stride % 8 == 0 && out_stride % 8 == 0 &&
+                 ((uintptr_t)attn1 % 16) == 0 && ((uintptr_t)attn2 % 16) == 0 && ((uintptr_t)attn_out % 16) == 0,
+             HA_ERR_SHAPE, "ha_lse_merge: rows must be 16-byte aligned");
+  const int pieces = (int)(d / 8);
+  const int64_t items = rows * pieces;
+  dim3 grid((unsigned)((items + 255) / 256));
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == HA_F16)
+    hipLaunchKernelGGL((lse_merge_kernel<f16_t>), grid, dim3(256), 0, s, (const f16_t*)attn1, lse1,
+                       (const f16_t*)attn2, lse2, (f16_t*)attn_out, lse_out, rows, pieces, attn1_stride,
+                       attn2_stride, out_stride, lse1_stride, lse2_stride, lse_out_stride);
+  else
+    hipLaunchKernelGGL((lse_merge_kernel<bf16_t>), grid, dim3(256), 0, s, (const bf16_t*)attn1, lse1,
+                       (const bf16_t*)attn2, lse2, (bf16_t*)attn_out, lse_out, rows, pieces, attn1_stride,
+                       attn2_stride, out_stride, lse1_stride, lse2_stride, lse_out_stride);
+  return ha_launch_status("ha_lse_merge");
+}

@@ -1,0 +1,265 @@
+"""Operator layer: the reference's L2 functions (same names, argument order and layouts), each a thin
+shim that checks its tensors and hands raw device pointers to one C symbol of libhyperattn.so.
+
+Reference interfaces mirrored here:
+  hash            <- AngularLSHTriton.hash_triton           src/angular_lsh_triton.py:99-145,181-182
+  bucket_argsort  <- torch.sort(..., dim=2, stable=True)[1] hyper_attention.py:116-117
+  indexing        <- indexing                               src/attn_utils.py:27-50
+  hyper_attn_func <- hyper_attn_func (forward)              src/hyper_attn_triton.py:668-742,895-920
+  flash_attn_func <- flash_attn_func (forward, no bias)     src/flash_attn_triton.py:795-872,995-1012
+  add_self_attentions <- add_self_attentions                src/attn_utils.py:6-24
+"""
+from __future__ import annotations
+
+import ctypes
+import math
+
+import torch
+
+from . import _lib
+from ._lib import HA_BF16, HA_F16, HA_IDX_I32, HA_IDX_I64, AttnOperands, BlockAttnArgs, ForwardArgs
+
+
+def _dtype_code(t: torch.Tensor) -> int:
+    assert t.dtype in (torch.float16, torch.bfloat16), "Only support fp16 and bf16"
+    return HA_F16 if t.dtype == torch.float16 else HA_BF16
+
+
+def _idx_code(t: torch.Tensor) -> int:
+    assert t.dtype in (torch.int32, torch.int64), "index tensors must be int32 or int64"
+    return HA_IDX_I32 if t.dtype == torch.int32 else HA_IDX_I64
+
+
+def _stream(t: torch.Tensor):
+    return ctypes.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+
+
+def _ptr(t):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None else None
+
+
+# ------------------------------------------------------------------------------------- hash
+def lsh_hash(mat: torch.Tensor, proj_dir: torch.Tensor) -> torch.Tensor:
+    """int32 bucket ids (b,h,n) of mat (b,h,n,d); proj_dir is (b,h,d,r) or (1,1,d,r)."""
+    batch, nheads, seqlen, d = mat.shape
+    num_projs = proj_dir.shape[-1]
+    assert proj_dir.shape == (batch, nheads, d, num_projs) or proj_dir.shape == (1, 1, d, num_projs)
+    assert mat.dtype == proj_dir.dtype, "All three tensors must have the same type"
+    assert mat.dtype in (torch.float16, torch.bfloat16), "Only support fp16 and bf16"
+    assert mat.is_cuda and proj_dir.is_cuda
+    if mat.stride(-1) != 1:
+        mat = mat.contiguous()
+    proj_dir = proj_dir.contiguous()
+    if proj_dir.shape[:2] == (1, 1):
+        psb, psh = 0, 0
+    else:
+        psb, psh = proj_dir.stride(0), proj_dir.stride(1)
+    buckets = torch.empty((batch, nheads, seqlen), device=mat.device, dtype=torch.int32)
+    with torch.cuda.device(mat.device):
+        _lib.check(_lib.lib().ha_lsh_hash(
+            _ptr(mat), _ptr(proj_dir), _ptr(buckets), batch, nheads, seqlen, d, num_projs,
+            mat.stride(0), mat.stride(1), mat.stride(2), psb, psh, _dtype_code(mat), _stream(mat)))
+    return buckets
+
+
+# ------------------------------------------------------------------------------------- sort
+def bucket_argsort(buckets: torch.Tensor, num_keys: int = 256, out_dtype=torch.int64) -> torch.Tensor:
+    """Stable argsort along the last dim of int32 keys in [0, num_keys); (b,h,n) -> (b,h,n)."""
+    assert buckets.is_cuda and buckets.dtype == torch.int32
+    buckets = buckets.contiguous()
+    n = buckets.shape[-1]
+    segs = buckets.numel() // n
+    out = torch.empty(buckets.shape, device=buckets.device, dtype=out_dtype)
+    L = _lib.lib()
+    ws_bytes = L.ha_bucket_argsort_workspace_bytes(segs, n, num_keys)
+    ws = torch.empty(max(int(ws_bytes), 256), device=buckets.device, dtype=torch.uint8)
+    with torch.cuda.device(buckets.device):
+        _lib.check(L.ha_bucket_argsort(_ptr(buckets), _ptr(out), _idx_code(out), segs, n, n, 0, num_keys,
+                                       _ptr(ws), ws.numel(), _stream(buckets)))
+    return out
+
+
+# ----------------------------------------------------------------------------------- gather
+def indexing(x: torch.Tensor, indices: torch.Tensor, chunk_size: int = -1) -> torch.Tensor:
+    """out[b,h,s] = x[b,h,indices[b,h,s]]; rows zero-padded up to a multiple of chunk_size when
+    x.shape[2] is not one (the reference's padding branch)."""
+    assert x.is_cuda and indices.is_cuda and x.dim() == 4 and indices.dim() == 3
+    b, h, n, d = x.shape
+    s = indices.shape[2]
+    if x.stride(-1) != 1:
+        x = x.contiguous()
+    indices = indices.contiguous()
+    n_out = s
+    if not (chunk_size < 0 or (chunk_size > 0 and n % chunk_size == 0)):
+        n_out = math.ceil(s / chunk_size) * chunk_size
+    out = torch.empty((b, h, n_out, d), device=x.device, dtype=x.dtype)
+    with torch.cuda.device(x.device):
+        _lib.check(_lib.lib().ha_gather_rows(
+            _ptr(x), _ptr(indices), _idx_code(indices), _ptr(out), b, h, n, s, n_out, d,
+            x.stride(0), x.stride(1), x.stride(2), x.element_size(), _stream(x)))
+    return out
+
+
+# -------------------------------------------------------------------------------- attention
+def _operands(q, k, v, out, lse, scale, *, layout_bnhd: bool, lse_row_stride: int):
+    """Fill AttnOperands from tensors laid out (b,n,h,d) [layout_bnhd] or (b,h,n,d)."""
+    t = AttnOperands()
+    t.q, t.k, t.v, t.out, t.lse = q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr()
+    if layout_bnhd:
+        b, nq, h, d = q.shape
+        nk = k.shape[1]
+        hk = k.shape[2]
+        sn, sh = 1, 2
+    else:
+        b, h, nq, d = q.shape
+        nk = k.shape[2]
+        hk = k.shape[1]
+        sn, sh = 2, 1
+    t.batch, t.heads, t.n_q, t.n_k, t.d, t.dv = b, h, nq, nk, d, v.shape[-1]
+    t.q_stride_b, t.q_stride_h, t.q_stride_n = q.stride(0), q.stride(sh), q.stride(sn)
+    t.k_stride_b, t.k_stride_h, t.k_stride_n = k.stride(0), k.stride(sh), k.stride(sn)
+    t.v_stride_b, t.v_stride_h, t.v_stride_n = v.stride(0), v.stride(sh), v.stride(sn)
+    t.o_stride_b, t.o_stride_h, t.o_stride_n = out.stride(0), out.stride(sh), out.stride(sn)
+    t.lse_stride_b, t.lse_stride_h = h * lse_row_stride, lse_row_stride
+    t.segs, t.seg_stride_rows, t.q_seg_offset, t.k_seg_offset = 1, 0, 0, 0
+    t.kv_group = h // hk
+    t.scale = scale
+    t.dtype = _dtype_code(q)
+    return t
+
+
+def hyper_attn_func(q, k, v, q_sort_idx, k_sort_idx, block_size, sample_size=0, softmax_scale=None,
+                    smooth_block=False, *, sampled_idx=None):
+    """q, k: (batch, seqlen, nheads, headdim); v: (batch, seqlen, nheads, v_headdim);
+    q_sort_idx, k_sort_idx: (batch, seqlen, nheads) permutations; returns o (batch, seqlen, nheads,
+    v_headdim) and lse (batch, nheads, seqlen) fp32.  `sampled_idx` (keyword only, not in the
+    reference) lists the sampled key rows, shape (sample_size,); default 0..sample_size-1."""
+    q, k, v = [x if x.stride(-1) == 1 else x.contiguous() for x in [q, k, v]]
+    assert sample_size % 128 == 0
+    batch, seqlen_q, nheads, d = q.shape
+    _, seqlen_k, _, _ = k.shape
+    assert k.shape == (batch, seqlen_k, nheads, d)
+    assert v.shape[:3] == (batch, seqlen_k, nheads)
+    assert q_sort_idx.shape == q.shape[:3]
+    assert k_sort_idx.shape == k.shape[:3]
+    assert d <= 128, "FlashAttention only support head dimensions up to 128"
+    assert q.dtype == k.dtype == v.dtype, "All tensors must have the same type"
+    assert q.dtype in [torch.float16, torch.bfloat16], "Only support fp16 and bf16"
+    assert q.is_cuda and k.is_cuda and v.is_cuda and q_sort_idx.is_cuda and k_sort_idx.is_cuda
+    assert q_sort_idx.dtype == k_sort_idx.dtype
+    softmax_scale = softmax_scale or 1.0 / math.sqrt(d)
+    lse = torch.empty((batch, nheads, seqlen_q), device=q.device, dtype=torch.float32)
+    o = torch.empty((batch, seqlen_q, nheads, v.shape[-1]), device=q.device, dtype=q.dtype)
+    assert seqlen_k % 128 == 0, "keys sequence length must be divisible by 128"
+
+    a = BlockAttnArgs()
+    a.t = _operands(q, k, v, o, lse, softmax_scale, layout_bnhd=True, lse_row_stride=seqlen_q)
+    a.q_idx, a.k_idx = q_sort_idx.data_ptr(), k_sort_idx.data_ptr()
+    a.idx_type = _idx_code(q_sort_idx)
+    a.q_idx_stride_b, a.q_idx_stride_h, a.q_idx_stride_n = q_sort_idx.stride(0), q_sort_idx.stride(2), q_sort_idx.stride(1)
+    a.k_idx_stride_b, a.k_idx_stride_h, a.k_idx_stride_n = k_sort_idx.stride(0), k_sort_idx.stride(2), k_sort_idx.stride(1)
+    keep = None
+    if sampled_idx is not None:
+        keep = sampled_idx.to(device=q.device, dtype=q_sort_idx.dtype).contiguous()
+        assert keep.shape == (sample_size,)
+        a.sampled_idx = keep.data_ptr()
+    a.sampled_stride_b = a.sampled_stride_h = 0
+    a.block_size, a.sample_size = block_size, sample_size
+    a.smooth_block, a.accumulate = int(bool(smooth_block)), 0
+    with torch.cuda.device(q.device):
+        _lib.check(_lib.lib().ha_block_attn_fwd(ctypes.byref(a), _stream(q)))
+    return o, lse
+
+
+def flash_attn_func(q, k, v, bias=None, causal=False, softmax_scale=None):
+    """q: (batch, seqlen_q, nheads, headdim); k, v: (batch, seqlen_k, nheads, headdim).
+    Returns o like q and lse (batch, nheads, ceil(seqlen_q/128)*128) fp32 (padding rows undefined)."""
+    if bias is not None:
+        raise NotImplementedError("attention bias is not part of the HyperAttention forward path")
+    q, k, v = [x if x.stride(-1) == 1 else x.contiguous() for x in [q, k, v]]
+    batch, seqlen_q, nheads, d = q.shape
+    _, seqlen_k, _, _ = k.shape
+    assert k.shape == (batch, seqlen_k, nheads, d)
+    assert v.shape == (batch, seqlen_k, nheads, d)
+    assert d <= 128, "FlashAttention only support head dimensions up to 128"
+    assert q.dtype == k.dtype == v.dtype, "All tensors must have the same type"
+    assert q.dtype in [torch.float16, torch.bfloat16], "Only support fp16 and bf16"
+    assert q.is_cuda and k.is_cuda and v.is_cuda
+    softmax_scale = softmax_scale or 1.0 / math.sqrt(d)
+    seqlen_q_rounded = math.ceil(seqlen_q / 128) * 128
+    lse = torch.empty((batch, nheads, seqlen_q_rounded), device=q.device, dtype=torch.float32)
+    o = torch.empty_like(q)
+    t = _operands(q, k, v, o, lse, softmax_scale, layout_bnhd=True, lse_row_stride=seqlen_q_rounded)
+    with torch.cuda.device(q.device):
+        _lib.check(_lib.lib().ha_flash_attn_fwd(ctypes.byref(t), int(bool(causal)), _stream(q)))
+    return o, lse
+
+
+def add_self_attentions(attn1, lse1, attn2, lse2):
+    """attn1, attn2: [b, h, n, d]; lse1, lse2: [b, h, n, 1] fp32.  Returns (attn, lse)."""
+    assert attn1.is_cuda and attn1.shape == attn2.shape and attn1.dtype == attn2.dtype
+    b, h, n, d = attn1.shape
+    a1 = attn1.contiguous()
+    a2 = attn2.contiguous()
+    l1 = lse1.to(torch.float32).contiguous().view(-1)
+    l2 = lse2.to(torch.float32).contiguous().view(-1)
+    assert l1.numel() == b * h * n and l2.numel() == b * h * n
+    out = torch.empty_like(a1)
+    lse = torch.empty((b, h, n, 1), device=attn1.device, dtype=torch.float32)
+    with torch.cuda.device(attn1.device):
+        _lib.check(_lib.lib().ha_lse_merge(_ptr(a1), _ptr(l1), _ptr(a2), _ptr(l2), _ptr(out), _ptr(lse),
+                                           b * h * n, d, d, d, d, 1, 1, 1, _dtype_code(a1), _stream(a1)))
+    return out, lse
+
+
+# ------------------------------------------------------------------------- whole forward pass
+def forward_plan_supported(n: int, min_seq_len: int, causal: bool, lsh_num_projs: int) -> bool:
+    """True when ha_forward covers this shape: every causal recursion level has an even length."""
+    if lsh_num_projs > 8:
+        return False
+    if not causal:
+        return True
+    while n > min_seq_len:
+        if n % 2:
+            return False
+        n //= 2
+    return True
+
+
+def hyper_forward(q, k, v, proj, *, scale, causal, lsh_num_projs, block_size, sample_size, min_seq_len,
+                  smooth_block, sampled_idx=None):
+    """One-call forward for contiguous (b,h,n,d) q and (b,h_kv,n,d) k, v.  Returns out (b,h,n,dv) and
+    lse (b,h,n) fp32."""
+    assert q.is_cuda and k.is_cuda and v.is_cuda and q.is_contiguous() and k.is_contiguous() and v.is_contiguous()
+    assert q.dtype == k.dtype == v.dtype, "All tensors must have the same type"
+    b, h, n, d = q.shape
+    hk = k.shape[1]
+    a = ForwardArgs()
+    out = torch.empty((b, h, n, v.shape[-1]), device=q.device, dtype=q.dtype)
+    lse = torch.empty((b, h, n), device=q.device, dtype=torch.float32)
+    a.q, a.k, a.v, a.out, a.lse = q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr()
+    keep = []
+    if proj is not None:
+        assert proj.dtype == q.dtype, "All three tensors must have the same type"
+        p = proj.reshape(d, lsh_num_projs).contiguous()
+        keep.append(p)
+        a.proj = p.data_ptr()
+    if sampled_idx is not None:
+        s = sampled_idx.to(device=q.device, dtype=torch.int32).contiguous()
+        assert s.shape == (sample_size,)
+        keep.append(s)
+        a.sampled_idx = s.data_ptr()
+    a.batch, a.heads, a.kv_heads, a.n, a.d, a.dv = b, h, hk, n, d, v.shape[-1]
+    a.lsh_num_projs, a.block_size, a.sample_size, a.min_seq_len = lsh_num_projs, block_size, sample_size, min_seq_len
+    a.smooth_block, a.causal = int(bool(smooth_block)), int(bool(causal))
+    a.scale = scale
+    a.dtype = _dtype_code(q)
+    L = _lib.lib()
+    ws_bytes = L.ha_forward_workspace_bytes(ctypes.byref(a))
+    if ws_bytes < 0:
+        _lib.check(int(ws_bytes))
+    ws = torch.empty(int(ws_bytes), device=q.device, dtype=torch.uint8)
+    a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
+    with torch.cuda.device(q.device):
+        _lib.check(L.ha_forward(ctypes.byref(a), _stream(q)))
+    return out, lse

@@ -1,0 +1,193 @@
+/*
+ * hyperattn.h — C ABI of libhyperattn.so, the MI355X (gfx950) HyperAttention forward path.
+ *
+ * Every entry point takes raw DEVICE pointers, sizes and strides (in ELEMENTS of the tensor's
+ * type unless stated otherwise) and a HIP stream passed as void* (hipStream_t; NULL = the
+ * default stream).  The library launches asynchronously on that stream, never synchronises,
+ * never allocates or frees device memory and keeps no state between calls: the caller owns
+ * every buffer including workspaces.  Return value: 0 on success, a negative ha_status for an
+ * argument error detected before any launch, or a positive hipError_t from the launch.
+ * ha_last_error() returns a thread-local human readable message for the last non-zero status.
+ *
+ * The reference being replaced is pure Python + Triton; "replaces" below names the reference
+ * interface (path relative to the reference checkout : line) each symbol stands in for.
+ */
+#ifndef HYPERATTN_H
+#define HYPERATTN_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define HA_ABI_VERSION 1
+
+typedef enum {
+  HA_OK = 0,
+  HA_ERR_NULL = -1,        /* a required pointer is NULL                                   */
+  HA_ERR_DTYPE = -2,       /* dtype is not HA_F16 / HA_BF16 ("Only support fp16 and bf16") */
+  HA_ERR_SHAPE = -3,       /* a size is non-positive / not a supported multiple            */
+  HA_ERR_HEADDIM = -4,     /* head dim > 128 or not a multiple of 16                        */
+  HA_ERR_UNSUPPORTED = -5, /* valid in the reference, not built here (message says what)   */
+  HA_ERR_WORKSPACE = -6    /* workspace pointer NULL or too small                           */
+} ha_status;
+
+typedef enum { HA_F16 = 0, HA_BF16 = 1 } ha_dtype;
+typedef enum { HA_IDX_I32 = 0, HA_IDX_I64 = 1 } ha_idx_type;
+
+int ha_abi_version(void);
+const char* ha_last_error(void);
+
+/* ---------------------------------------------------------------------------------------------
+ * Angular LSH bucket ids.
+ * replaces: AngularLSHTriton.hash_triton -> _angular_lsh -> _angular_lsh_kernel
+ *           (src/angular_lsh_triton.py:181-182, :99-145, :14-96)
+ * bucket[b,h,i] = gray(sum_j [x[b,h,i,:] . proj[:,j] > 0] << j), gray(v) = v ^ (v >> 1), the closed
+ * form of the `perm` table (src/angular_lsh_triton.py:168-173).  The sign is that of the exact dot
+ * product (products of fp16/bf16 values are exact; accumulation is in fp64).
+ * x: (batch, heads, n, d), last dim contiguous.  proj: (d, r) row-major, shared when
+ * proj_stride_b == proj_stride_h == 0, else one matrix per (b,h).  buckets: int32 (batch, heads, n)
+ * contiguous.  1 <= r <= 16, d <= 256.
+ */
+int ha_lsh_hash(const void* x, const void* proj, int32_t* buckets,
+                int64_t batch, int64_t heads, int64_t n, int64_t d, int64_t r,
+                int64_t x_stride_b, int64_t x_stride_h, int64_t x_stride_n,
+                int64_t proj_stride_b, int64_t proj_stride_h,
+                int dtype, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Segmented stable argsort of small non-negative integer keys (counting sort).
+ * replaces: torch.sort(buckets, dim=2, stable=True)[1] at hyper_attention.py:116-117
+ * Segment s (0 <= s < num_segments) is keys[seg_offset + s*seg_stride + (0..seg_len)).
+ * idx_out[s*seg_len + p] = i such that keys are non-decreasing in p, ties in ascending i;
+ * i is LOCAL to the segment (0 <= i < seg_len).  Keys must lie in [0, num_keys); num_keys <= 65536
+ * (one 8-bit pass per key byte).  idx_type selects int32 or int64 output.
+ * Workspace: ha_bucket_argsort_workspace_bytes(num_segments, seg_len, num_keys) bytes.
+ */
+int64_t ha_bucket_argsort_workspace_bytes(int64_t num_segments, int64_t seg_len, int64_t num_keys);
+int ha_bucket_argsort(const int32_t* keys, void* idx_out, int idx_type,
+                      int64_t num_segments, int64_t seg_len, int64_t seg_stride, int64_t seg_offset,
+                      int64_t num_keys, void* workspace, int64_t workspace_bytes, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Permuting row gather.
+ * replaces: indexing(x, indices) (src/attn_utils.py:27-50), the chunk_size < 0 branch; rows
+ * [n_idx, n_out) of the output are zero-filled, which is the padding branch (:45-50).
+ * out[b,h,s,:] = x[b,h,idx[b,h,s],:].  x (batch,heads,n_src,d) strided, out (batch,heads,n_out,d)
+ * contiguous, idx (batch,heads,n_idx) contiguous; elem_bytes is 2 or 4; d*elem_bytes % 16 == 0.
+ */
+int ha_gather_rows(const void* x, const void* idx, int idx_type, void* out,
+                   int64_t batch, int64_t heads, int64_t n_src, int64_t n_idx, int64_t n_out, int64_t d,
+                   int64_t x_stride_b, int64_t x_stride_h, int64_t x_stride_n,
+                   int elem_bytes, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Attention operands.  All tensors are addressed as ptr + b*stride_b + h*stride_h + row*stride_n
+ * (+ col); the last dim is contiguous.  lse is fp32, addressed lse + b*lse_stride_b + h*lse_stride_h
+ * + row.  "Virtual heads": when segs > 1 every (b,h) sequence is cut into `segs` consecutive
+ * segments of n_q (resp. n_k) rows that are treated as independent heads; segment g of a q/out/lse
+ * sequence starts at row q_seg_offset + g*seg_stride_rows, of a k/v sequence at row
+ * k_seg_offset + g*seg_stride_rows.  This is the halves-as-heads view of hyper_attention.py:67-69
+ * and the half slicing of :82-84 expressed as index arithmetic.  segs == 1 with zero offsets is the
+ * plain case.
+ */
+typedef struct {
+  const void* q;
+  const void* k;
+  const void* v;
+  void* out;      /* (.., n_q, dv) in dtype                                   */
+  float* lse;     /* (.., n_q) fp32                                           */
+  int64_t batch, heads, n_q, n_k, d, dv;
+  int64_t q_stride_b, q_stride_h, q_stride_n;
+  int64_t k_stride_b, k_stride_h, k_stride_n;
+  int64_t v_stride_b, v_stride_h, v_stride_n;
+  int64_t o_stride_b, o_stride_h, o_stride_n;
+  int64_t lse_stride_b, lse_stride_h;
+  int64_t segs, seg_stride_rows, q_seg_offset, k_seg_offset;
+  int64_t kv_group; /* grouped-query: q head h reads k/v (and k_idx) head h / kv_group; 1 = plain */
+  float scale;    /* softmax scale; <= 0 or NaN is an error (callers resolve the default)  */
+  int dtype;      /* ha_dtype                                                               */
+} ha_attn_operands;
+
+/* Sorted block-diagonal + sampled-column attention, forward.
+ * replaces: hyper_attn_func -> HyperAttnFunc.forward -> _hyper_attn_forward -> _fwd_hyper_kernel
+ *           (src/hyper_attn_triton.py:895-920, :668-742, :26-192)
+ * q_idx / k_idx: permutations of the rows of each (virtual) head, LOCAL row numbers, addressed
+ * idx + b*idx_stride_b + h*idx_stride_h + g*n + p*idx_stride_n (g = segment); sampled_idx: sample_size
+ * key rows (local), shared by all heads when sampled_stride_h == 0 (sampled_idx == NULL means
+ * 0,1,..,sample_size-1, the reference's intended set, src/hyper_attn_triton.py:576-581).
+ * n_q % 128 == 0, n_k % 128 == 0 (:695), sample_size % 128 == 0 (:911), d and dv in {64, 128}.
+ * accumulate != 0: out/lse already hold a partial attention over a disjoint key set for every row;
+ * the result is merged into them in place (add_self_attentions, src/attn_utils.py:6-24, fused).
+ */
+typedef struct {
+  ha_attn_operands t;
+  const void* q_idx;
+  const void* k_idx;
+  const void* sampled_idx;
+  int idx_type;
+  int64_t q_idx_stride_b, q_idx_stride_h, q_idx_stride_n;
+  int64_t k_idx_stride_b, k_idx_stride_h, k_idx_stride_n;
+  int64_t sampled_stride_b, sampled_stride_h;
+  int64_t block_size, sample_size;
+  int smooth_block;
+  int accumulate;
+} ha_block_attn_args;
+
+int ha_block_attn_fwd(const ha_block_attn_args* args, void* stream);
+
+/* Exact (flash) attention, forward.
+ * replaces: flash_attn_func -> FlashAttnFunc.forward -> _flash_attn_forward -> _fwd_kernel with
+ *           bias=None (src/flash_attn_triton.py:995-1012, :795-872, :57-267)
+ * Any n_q, n_k >= 1; causal mask row >= col (:177); d == dv in {64, 128}.
+ */
+int ha_flash_attn_fwd(const ha_attn_operands* t, int causal, void* stream);
+
+/* Merge of two partial attentions.
+ * replaces: add_self_attentions (src/attn_utils.py:6-24)
+ * rows = batch*heads*n flattened; attn*: (rows, d) with row strides; lse*: fp32 with element
+ * strides.  Outputs may alias the first inputs.
+ */
+int ha_lse_merge(const void* attn1, const float* lse1, const void* attn2, const float* lse2,
+                 void* attn_out, float* lse_out, int64_t rows, int64_t d,
+                 int64_t attn1_stride, int64_t attn2_stride, int64_t out_stride,
+                 int64_t lse1_stride, int64_t lse2_stride, int64_t lse_out_stride,
+                 int dtype, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Whole forward pass of the module for contiguous (batch, heads, n, d) tensors, one call, no host
+ * synchronisation and no tensor copies.
+ * replaces: HyperAttention.forward / forward_no_causal_mask (hyper_attention.py:25-132) for the
+ * shapes where every recursion level has an even length (n = leaf_len * 2^levels); other shapes
+ * are composed by the caller from the operators above.
+ * proj: (d, r) in dtype.  sampled_idx: int32 key rows local to each un-masked call (NULL = first
+ * sample_size rows), shared by all heads and levels.  out (batch,heads,n,dv) dtype, lse
+ * (batch,heads,n) fp32.  kv_heads divides heads (grouped-query: q head h reads kv head
+ * h / (heads/kv_heads)); k and v are (batch, kv_heads, n, d).
+ */
+typedef struct {
+  const void* q;
+  const void* k;
+  const void* v;
+  const void* proj;
+  const int32_t* sampled_idx;
+  void* out;
+  float* lse;
+  int64_t batch, heads, kv_heads, n, d, dv;
+  int64_t lsh_num_projs, block_size, sample_size, min_seq_len;
+  int smooth_block;
+  int causal;
+  float scale;
+  int dtype;
+  void* workspace;
+  int64_t workspace_bytes;
+} ha_forward_args;
+
+int64_t ha_forward_workspace_bytes(const ha_forward_args* args);
+int ha_forward(const ha_forward_args* args, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HYPERATTN_H */

@@ -1,0 +1,207 @@
+"""GPU parity tests of the HyperAttention module (whole forward pass) against the CPU oracle, plus
+size-independent properties at the full benchmark shapes.  Tolerances as in test_gpu_ops.py."""
+import numpy as np
+import pytest
+import torch
+
+from _util import _gen, _randn, assert_close
+from oracle import hyper_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ha():
+    import hyperattention_amd
+    from hyperattention_amd import _lib
+    _lib.lib()
+    return hyperattention_amd
+
+
+def _module(ha, d, dtype, seed, **kw):
+    m = ha.HyperAttention(input_dim=d, rng=_gen(seed), **kw).to(device="cuda", dtype=dtype)
+    return m, m.lsh.proj_dir[0, 0].cpu()
+
+
+def _oracle(q, k, v, proj, m, causal, scale=None, sampled_idx=None):
+    return O.hyper_forward(q, k, v, proj, scale=scale, causal=causal, lsh_num_projs=m.lsh_num_projs,
+                           block_size=m.block_size, sample_size=m.sample_size, min_seq_len=m.min_seq_len,
+                           smooth_block=m.smooth_block, sampled_idx=sampled_idx)
+
+
+# --------------------------------------------------------------------------- non-causal
+def test_non_causal_config1(ha):
+    """BASELINE config 1: batch 1, 4 heads, seq 4096, d 64, r 8, block 256, sample 256, min_seq_len 2048
+    (inputs cast to fp16 for the GPU; both the default and an explicit seeded sample set)."""
+    g = _gen(100)
+    q, k, v = (torch.randn((1, 4, 4096, 64), generator=g).half() for _ in range(3))
+    proj = torch.randn((64, 8), generator=g).half()
+    sampled = torch.randint(0, 4096, (256,), generator=g)
+    for s_idx in (None, sampled):
+        m = ha.HyperAttention(input_dim=64, proj_dir=proj, sampled_idx=s_idx).to(device="cuda", dtype=torch.float16)
+        attn, lse = m(q.cuda(), k.cuda(), v.cuda(), causal=False, return_lse=True)
+        assert attn.shape == (1, 4, 4096, 64) and lse.shape == (1, 4, 4096, 1) and lse.dtype == torch.float32
+        ro, rl = _oracle(q, k, v, proj, m, False, sampled_idx=s_idx)
+        assert_close(attn, ro, "attn", torch.float16)
+        assert_close(lse, rl, "lse")
+    only = m(q.cuda(), k.cuda(), v.cuda())
+    assert torch.equal(only, attn)
+
+
+@pytest.mark.parametrize("dtype,d,block,sample,smooth", [
+    (torch.bfloat16, 128, 512, 512, True),    # BASELINE config 4 at reduced batch/heads/length
+    (torch.float16, 64, 256, 256, True),
+    (torch.bfloat16, 64, 128, 128, False),
+])
+def test_non_causal_variants(ha, dtype, d, block, sample, smooth):
+    q, k, v = (_randn((2, 2, 2048, d), s, dtype) for s in (110, 111, 112))
+    m, proj = _module(ha, d, dtype, 113, block_size=block, sample_size=sample, smooth_block=smooth)
+    attn, lse = m(q.cuda(), k.cuda(), v.cuda(), scale=0.1, return_lse=True)
+    ro, rl = _oracle(q, k, v, proj, m, False, scale=0.1)
+    assert_close(attn, ro, "attn", dtype)
+    assert_close(lse, rl, "lse")
+
+
+def test_non_causal_short_sequence_is_exact(ha):
+    q, k, v = (_randn((1, 2, 1000, 64), s, torch.float16) for s in (120, 121, 122))
+    m, proj = _module(ha, 64, torch.float16, 123)  # min_seq_len 2048 > 1000
+    attn, lse = m(q.cuda(), k.cuda(), v.cuda(), return_lse=True)
+    ro, rl = O.exact_attention(q, k, v)
+    assert_close(attn, ro, "attn", torch.float16)
+    assert_close(lse.squeeze(-1), rl, "lse")
+
+
+# ------------------------------------------------------------------------------- causal
+@pytest.mark.parametrize("dtype,d,n,msl,block,sample", [
+    (torch.float16, 64, 4096, 512, 256, 256),    # three levels (2048, 1024, 512 halves) + leaves of 512
+    (torch.bfloat16, 128, 2048, 256, 256, 128),
+    (torch.float16, 64, 2048, 2048, 256, 256),   # top-level leaf: exact causal
+    (torch.float16, 64, 3000, 2048, 256, 256),   # one level whose off-diagonal is the exact kernel
+])
+def test_causal_forward(ha, dtype, d, n, msl, block, sample):
+    q, k, v = (_randn((1, 2, n, d), s, dtype) for s in (130, 131, 132))
+    m, proj = _module(ha, d, dtype, 133, block_size=block, sample_size=sample, min_seq_len=msl)
+    attn, lse = m(q.cuda(), k.cuda(), v.cuda(), causal=True, return_lse=True)
+    ro, rl = _oracle(q, k, v, proj, m, True)
+    assert attn.shape == (1, 2, n, d)
+    assert_close(attn, ro, "attn", dtype)
+    if n <= msl:  # the reference returns the exact kernel's padded (b, h, n_rounded) lse here
+        assert lse.shape == (1, 2, -(-n // 128) * 128)
+        assert_close(lse[:, :, :n], rl.squeeze(-1), "lse")
+    else:
+        assert lse.shape == (1, 2, n, 1)
+        assert_close(lse, rl, "lse")
+
+
+def test_causal_odd_lengths_composed_path(ha):
+    # 2047 -> padded to 2048 -> halves of 1024: hashed off-diagonal, exact leaves.
+    # 1001 -> padded to 1002 -> halves of 501 < 600: exact off-diagonal (arbitrary length), exact leaves.
+    for n, msl in ((2047, 1024), (1001, 600)):
+        q, k, v = (_randn((1, 2, n, 64), s, torch.float16) for s in (140, 141, 142))
+        m, proj = _module(ha, 64, torch.float16, 143, block_size=256, sample_size=128, min_seq_len=msl)
+        attn, lse = m(q.cuda(), k.cuda(), v.cuda(), causal=True, return_lse=True)
+        ro, rl = _oracle(q, k, v, proj, m, True)
+        assert attn.shape == (1, 2, n, 64) and lse.shape == (1, 2, n, 1)
+        assert_close(attn, ro, "attn", torch.float16)
+        assert_close(lse, rl, "lse")
+
+
+def test_causal_composed_path_equals_fused_path(ha):
+    q, k, v = (_randn((1, 2, 2048, 64), s, torch.float16).cuda() for s in (150, 151, 152))
+    m, _ = _module(ha, 64, torch.float16, 153, min_seq_len=512)
+    fused, lse_f = m(q, k, v, causal=True, return_lse=True)
+    comp, lse_c = m._forward_composed(q, k, v, 64 ** -0.5, True)
+    assert_close(comp, fused, "composed vs fused", torch.float16)
+    assert_close(lse_c, lse_f, "composed vs fused lse")
+
+
+def test_module_argument_errors(ha):
+    m, _ = _module(ha, 64, torch.float16, 160)
+    q = torch.zeros((1, 1, 256, 64), dtype=torch.float16, device="cuda")
+    with pytest.raises(AssertionError):
+        m(q, q[:, :, :128], q[:, :, :128])            # n_query != n_key
+    with pytest.raises(AssertionError):
+        m(q.float(), q.float(), q.float())            # fp32 on the GPU path
+    with pytest.raises(ValueError):
+        ha.HyperAttention(lsh_num_projs=0)
+    m2 = ha.HyperAttention(input_dim=64, min_seq_len=128, bogus_keyword=1).to("cuda", torch.float16)
+    bad = torch.zeros((1, 1, 192, 64), dtype=torch.float16, device="cuda")
+    with pytest.raises(AssertionError):
+        m2(bad, bad, bad)                             # hashed path needs n % 128 == 0
+
+
+# ----------------------------------------------- full-size shapes: size-independent properties
+def test_full_size_non_causal_properties(ha):
+    """BASELINE config 2 (batch 1, 32 heads, seq 32768, d 64, fp16): permutations are valid and stable,
+    the fused forward equals the operator-by-operator composition, and a sampled head slice matches
+    the oracle."""
+    b, h, n, d = 1, 32, 32768, 64
+    g = torch.Generator(device="cuda").manual_seed(170)
+    q, k, v = (torch.randn((b, h, n, d), generator=g, device="cuda", dtype=torch.float16) for _ in range(3))
+    m, proj = _module(ha, d, torch.float16, 171)
+    attn, lse = m(q, k, v, return_lse=True)
+    buckets = m.lsh.hash(q)
+    perm = ha.bucket_argsort(buckets)
+    sorted_b = torch.gather(buckets.long(), 2, perm)
+    assert (sorted_b[:, :, 1:] >= sorted_b[:, :, :-1]).all()
+    ties = sorted_b[:, :, 1:] == sorted_b[:, :, :-1]
+    assert (perm[:, :, 1:][ties] > perm[:, :, :-1][ties]).all()
+    assert torch.equal(torch.sort(perm, dim=2)[0], torch.arange(n, device="cuda").expand(b, h, n))
+    comp, lse_c = m.forward_no_causal_mask(q, k, v, d ** -0.5)
+    assert torch.equal(comp, attn) and torch.equal(lse_c, lse)
+    for head in (0, 17, 31):
+        sl = slice(head, head + 1)
+        ro, rl = _oracle(q[:, sl].cpu(), k[:, sl].cpu(), v[:, sl].cpu(), proj, m, False)
+        assert_close(attn[:, sl], ro, f"attn head {head}", torch.float16)
+        assert_close(lse[:, sl], rl, f"lse head {head}")
+
+
+def test_full_size_causal_properties(ha):
+    """BASELINE config 3 (batch 1, 32 heads, seq 131072, d 64, fp16, causal): the first leaf is exact
+    causal attention, lse is finite, heads are independent, and one head matches the oracle."""
+    b, h, n, d = 1, 32, 131072, 64
+    g = torch.Generator(device="cuda").manual_seed(180)
+    q, k, v = (torch.randn((b, h, n, d), generator=g, device="cuda", dtype=torch.float16) for _ in range(3))
+    m, proj = _module(ha, d, torch.float16, 181)
+    attn, lse = m(q, k, v, causal=True, return_lse=True)
+    assert attn.shape == (b, h, n, d) and lse.shape == (b, h, n, 1)
+    assert torch.isfinite(attn).all() and torch.isfinite(lse).all()
+    # rows of the first leaf (2048) only ever see exact causal attention
+    leaf = slice(0, 2048)
+    ro, rl = O.exact_attention(q[:, :4, leaf].cpu(), k[:, :4, leaf].cpu(), v[:, :4, leaf].cpu(), None, True)
+    assert_close(attn[:, :4, leaf], ro, "first leaf", torch.float16)
+    assert_close(lse[:, :4, leaf, 0], rl, "first leaf lse")
+    # the result for one head does not depend on the other heads being there
+    one, lse_one = m(q[:, 5:6].contiguous(), k[:, 5:6].contiguous(), v[:, 5:6].contiguous(), causal=True,
+                     return_lse=True)
+    assert torch.equal(one, attn[:, 5:6]) and torch.equal(lse_one, lse[:, 5:6])
+    # whole-head parity on a slice of the sequence (the oracle recursion at full length, one head)
+    ro, rl = _oracle(q[:, 5:6].cpu(), k[:, 5:6].cpu(), v[:, 5:6].cpu(), proj, m, True)
+    assert_close(one, ro, "attn head 5", torch.float16)
+    assert_close(lse_one, rl, "lse head 5")
+
+
+def test_grouped_query_heads(ha):
+    """BASELINE config 5 shape family (32 query heads on 2 KV heads, d 128, bf16, causal, clustered
+    keys) at reduced length: the expanded-KV module call matches the oracle, and the native grouped
+    call (K/V not expanded) gives bit-identical results."""
+    from hyperattention_amd import ops
+    b, hq, hkv, n, d = 1, 8, 2, 4096, 128
+    g = _gen(190)
+    cent = torch.nn.functional.normalize(torch.randn((64, d), generator=g), dim=-1)
+    kc = torch.randint(0, 64, (b, hkv, n), generator=g)
+    qc = torch.randint(0, 64, (b, hq, n), generator=g)
+    k = (4 * cent[kc] + 0.5 * torch.randn((b, hkv, n, d), generator=g)).bfloat16()
+    q = (4 * cent[qc] + 0.5 * torch.randn((b, hq, n, d), generator=g)).bfloat16()
+    v = torch.randn((b, hkv, n, d), generator=g).bfloat16()
+    k_exp = k.repeat_interleave(hq // hkv, dim=1)
+    v_exp = v.repeat_interleave(hq // hkv, dim=1)
+    m, proj = _module(ha, d, torch.bfloat16, 191, min_seq_len=1024)
+    attn, lse = m(q.cuda(), k_exp.cuda(), v_exp.cuda(), causal=True, return_lse=True)
+    ro, rl = _oracle(q, k_exp, v_exp, proj, m, True)
+    assert_close(attn, ro, "attn", torch.bfloat16)
+    assert_close(lse, rl, "lse")
+    native, lse_n = ops.hyper_forward(q.cuda(), k.cuda(), v.cuda(), m.lsh.proj_dir, scale=d ** -0.5, causal=True,
+                                      lsh_num_projs=8, block_size=256, sample_size=256, min_seq_len=1024,
+                                      smooth_block=False)
+    assert torch.equal(native, attn) and torch.equal(lse_n.unsqueeze(-1), lse)
