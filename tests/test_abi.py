@@ -1,0 +1,139 @@
+"""CPU-only checks of the C ABI: the library loads, exports every symbol include/hyperattn.h declares,
+the ctypes mirrors of its structs have the C layout, and argument errors are reported with a negative
+status before anything is launched (so these calls are safe without a GPU)."""
+import ctypes
+import os
+import re
+import subprocess
+
+import pytest
+
+from hyperattention_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "hyperattn.h")
+
+
+@pytest.fixture(scope="module")
+def lib():
+    if not os.path.exists(_lib.LIB_PATH):
+        _lib.build()
+    return _lib.lib()
+
+
+def _declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(ha_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_every_declared_symbol_is_exported(lib):
+    declared = _declared_symbols()
+    assert declared == sorted(_lib.SYMBOLS)
+    for name in declared:
+        assert hasattr(lib, name), f"{name} declared in hyperattn.h but not exported"
+    assert lib.ha_abi_version() == 1
+
+
+def test_struct_layouts_match_the_header(tmp_path):
+    """Compile a tiny C program against the header and compare sizeof/offsetof with ctypes."""
+    src = tmp_path / "layout.c"
+    src.write_text(r'''
+#include <stdio.h>
+#include <stddef.h>
+#include "hyperattn.h"
+int main(void) {
+  printf("%zu %zu %zu\n", sizeof(ha_attn_operands), sizeof(ha_block_attn_args), sizeof(ha_forward_args));
+  printf("%zu %zu %zu\n", offsetof(ha_attn_operands, scale), offsetof(ha_block_attn_args, accumulate),
+         offsetof(ha_forward_args, workspace_bytes));
+  printf("%zu %zu\n", offsetof(ha_block_attn_args, q_idx), offsetof(ha_forward_args, scale));
+  return 0;
+}''')
+    exe = tmp_path / "layout"
+    subprocess.run(["gcc", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe)], check=True)
+    out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split()
+    got = [int(x) for x in out]
+    want = [ctypes.sizeof(_lib.AttnOperands), ctypes.sizeof(_lib.BlockAttnArgs), ctypes.sizeof(_lib.ForwardArgs),
+            _lib.AttnOperands.scale.offset, _lib.BlockAttnArgs.accumulate.offset,
+            _lib.ForwardArgs.workspace_bytes.offset, _lib.BlockAttnArgs.q_idx.offset, _lib.ForwardArgs.scale.offset]
+    assert got == want
+
+
+def test_argument_errors_before_any_launch(lib):
+    one = ctypes.c_void_p(16)
+    # null pointers
+    assert lib.ha_lsh_hash(None, None, None, 1, 1, 128, 64, 8, 0, 0, 64, 0, 0, 0, None) == -1
+    assert b"null" in lib.ha_last_error()
+    # bad dtype, bad r, bad d
+    assert lib.ha_lsh_hash(one, one, one, 1, 1, 128, 64, 8, 0, 0, 64, 0, 0, 7, None) == -2
+    assert lib.ha_lsh_hash(one, one, one, 1, 1, 128, 64, 0, 0, 0, 64, 0, 0, 0, None) == -3
+    assert b"Invalid value for num_projs" in lib.ha_last_error()
+    assert lib.ha_lsh_hash(one, one, one, 1, 1, 128, 60, 8, 0, 0, 64, 0, 0, 0, None) == -4
+    # sort: workspace too small, too many keys
+    assert lib.ha_bucket_argsort_workspace_bytes(4, 8192, 256) == 4 * 2 * 256 * 4
+    assert lib.ha_bucket_argsort(one, one, 0, 4, 8192, 8192, 0, 256, one, 16, None) == -6
+    assert lib.ha_bucket_argsort(one, one, 0, 4, 8192, 8192, 0, 1 << 20, one, 1 << 30, None) == -5
+    # gather: row bytes not a multiple of 16
+    assert lib.ha_gather_rows(one, one, 0, one, 1, 1, 8, 8, 8, 3, 0, 0, 3, 2, None) == -4
+    # merge
+    assert lib.ha_lse_merge(one, one, one, one, one, one, 8, 12, 12, 12, 12, 1, 1, 1, 0, None) == -3
+
+
+def _operands(**kw):
+    t = _lib.AttnOperands()
+    t.q = t.k = t.v = t.out = t.lse = 16
+    t.batch, t.heads, t.n_q, t.n_k, t.d, t.dv = 1, 1, 256, 256, 64, 64
+    t.q_stride_n = t.k_stride_n = t.v_stride_n = t.o_stride_n = 64
+    t.segs, t.kv_group, t.scale, t.dtype = 1, 1, 0.125, 0
+    for k, v in kw.items():
+        setattr(t, k, v)
+    return t
+
+
+def test_attention_argument_errors(lib):
+    assert lib.ha_flash_attn_fwd(None, 0, None) == -1
+    assert lib.ha_flash_attn_fwd(ctypes.byref(_operands(dtype=3)), 0, None) == -2
+    assert lib.ha_flash_attn_fwd(ctypes.byref(_operands(d=256, dv=256)), 0, None) == -4
+    assert b"head dimensions up to 128" in lib.ha_last_error()
+    assert lib.ha_flash_attn_fwd(ctypes.byref(_operands(d=32, dv=32)), 0, None) == -5
+    assert lib.ha_flash_attn_fwd(ctypes.byref(_operands(scale=0.0)), 0, None) == -3
+    assert lib.ha_flash_attn_fwd(ctypes.byref(_operands(q_stride_n=60)), 0, None) == -3
+    a = _lib.BlockAttnArgs()
+    a.t = _operands()
+    a.q_idx = a.k_idx = 16
+    a.block_size, a.sample_size = 256, 100
+    assert lib.ha_block_attn_fwd(ctypes.byref(a), None) == -3  # sample_size % 128
+    a.sample_size = 0
+    a.t = _operands(n_k=192)
+    assert lib.ha_block_attn_fwd(ctypes.byref(a), None) == -3
+    assert b"divisible by 128" in lib.ha_last_error()
+    a.t = _operands()
+    a.q_idx = None
+    assert lib.ha_block_attn_fwd(ctypes.byref(a), None) == -1
+
+
+def test_forward_plan_and_workspace(lib):
+    f = _lib.ForwardArgs()
+    f.batch, f.heads, f.kv_heads, f.n, f.d, f.dv = 1, 32, 32, 131072, 64, 64
+    f.lsh_num_projs, f.block_size, f.sample_size, f.min_seq_len = 8, 256, 256, 2048
+    f.causal, f.scale, f.dtype = 1, 0.125, 0
+    ws = lib.ha_forward_workspace_bytes(ctypes.byref(f))
+    # buckets (2 x 4 Mi x 4 B) + six levels of (q_idx + k_idx) (2 x 2 Mi x 4 B each) + histograms
+    assert ws >= 2 * 4194304 * 4 + 6 * 2 * 2097152 * 4
+    assert ws < 200 << 20
+    f.n = 4095  # an odd length above min_seq_len needs the padded copy: not a shape of the one-call entry point
+    assert lib.ha_forward_workspace_bytes(ctypes.byref(f)) == -5
+    f.n = 131072 + 2  # the first halves (65537) are hashed and must be a multiple of 128
+    assert lib.ha_forward_workspace_bytes(ctypes.byref(f)) == -3
+    f.n, f.causal = 4000, 0  # hashed path needs n % 128 == 0
+    assert lib.ha_forward_workspace_bytes(ctypes.byref(f)) == -3
+    f.n, f.min_seq_len = 1000, 2048  # exact path: no workspace needed beyond the minimum
+    assert lib.ha_forward_workspace_bytes(ctypes.byref(f)) == 256
+    assert lib.ha_forward(ctypes.byref(f), None) == -1  # null tensors
+
+
+def test_python_layer_fails_loudly_without_library(monkeypatch, tmp_path):
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "missing.so"))
+    monkeypatch.setattr(_lib, "_lib", None)
+    with pytest.raises(RuntimeError, match="no fallback"):
+        _lib.lib()
