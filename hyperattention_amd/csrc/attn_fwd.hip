@@ -29,6 +29,7 @@ constexpr int WG_QUERIES = 256;  // sorted query positions per workgroup
 constexpr int KC = 64;           // keys per LDS chunk
 constexpr float LOG2E = 1.4426950408889634f;
 constexpr float LN2 = 0.6931471805599453f;
+constexpr float RESCALE_SLACK = 8.0f;  // log2 units
 
 template <typename T>
 struct Mfma;
@@ -37,11 +38,20 @@ struct Mfma<f16_t> {
   static __device__ __forceinline__ f32x16 run(f16x8 a, f16x8 b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
   }
+  // c + a[0] + a[1]
+  static __device__ __forceinline__ float pair_sum(f16x2 a, float c) {
+    const f16x2 ones = {(f16_t)1.0f, (f16_t)1.0f};
+    return __builtin_amdgcn_fdot2(a, ones, c, false);
+  }
 };
 template <>
 struct Mfma<bf16_t> {
   static __device__ __forceinline__ f32x16 run(bf16x8 a, bf16x8 b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ float pair_sum(bf16x2 a, float c) {
+    const bf16x2 ones = {(bf16_t)1.0f, (bf16_t)1.0f};
+    return __builtin_amdgcn_fdot2_f32_bf16(a, ones, c, false);
   }
 };
 
@@ -53,6 +63,13 @@ __device__ __forceinline__ int vt_key_pos(int k) {
 }
 __device__ __forceinline__ int vt_swizzle(int dvrow) { return (dvrow & 7) ^ ((dvrow >> 3) & 7); }
 
+constexpr int NUM_XCD = 8;
+__device__ __forceinline__ int xcd_contiguous_id(int linear, int total) {
+  const int xcd = linear % NUM_XCD, k = linear / NUM_XCD;
+  const int q = total / NUM_XCD, r = total % NUM_XCD;
+  return xcd * q + (xcd < r ? xcd : r) + k;
+}
+
 template <typename T, int D, bool GATHER, bool CAUSAL>
 __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void attn_fwd_kernel(const ha_attn_kernel_params p) {
   typedef typename ElemTraits<T>::vec8 vec8;
@@ -63,8 +80,6 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void attn_fwd_kernel
   constexpr int DB = DV / 32;         // 32-row blocks of O^T
   constexpr int PR = D / 8;           // 16-byte pieces per K row
   constexpr int PV = DV / 8;          // 16-byte pieces per V row
-  constexpr int NPK = KC * PR / WG_THREADS;      // K pieces staged per thread per chunk
-  constexpr int NPV = (KC / 2) * PV / WG_THREADS;  // V key-pairs staged per thread per chunk
 
   __shared__ __attribute__((aligned(16))) T lds_k[2][KC * D];
   __shared__ __attribute__((aligned(16))) T lds_vt[2][DV * KC];
@@ -74,9 +89,13 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void attn_fwd_kernel
   const int hi = lane >> 5, col = lane & 31;
 
   // ---- which (virtual) head and query tile -----------------------------------------------------
+  // Workgroups are handed to the 8 XCDs round-robin by their linear id, and each XCD has its own
+  // L2.  Re-number them so that every XCD works through one contiguous range of (head, query tile):
+  // the query tiles that share a head's K/V then meet in the same L2.
+  const int wg = xcd_contiguous_id(blockIdx.x, gridDim.x);
   const int qtiles = (p.n_q + WG_QUERIES - 1) / WG_QUERIES;
-  const int vhead = blockIdx.x / qtiles;
-  const int qt = blockIdx.x % qtiles;
+  const int vhead = wg / qtiles;
+  const int qt = wg % qtiles;
   const int seg = vhead % p.segs;
   const int bh = vhead / p.segs;
   const int b = bh / p.heads, h = bh % p.heads;
@@ -170,8 +189,17 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void attn_fwd_kernel
   const int wave_q_first = qt * WG_QUERIES + wave * 64;
 
   // ---- staging: global -> registers -> LDS ------------------------------------------------------
-  vec8 stage_k[NPK];
-  vec8 stage_v[NPV][2];
+  // Every thread owns the same 16-byte piece `pc` of two adjacent key rows (pair `pr`) of the chunk,
+  // for K and for V (NP passes when a row has more than 8 pieces).  The original row numbers of the
+  // chunk after next are fetched while the current one is computed, so the row loads never wait for
+  // an index load.
+  constexpr int NP = (KC / 2) * PR / WG_THREADS;  // 1 for d = 64, 2 for d = 128
+  constexpr int PAIRS_PER_PASS = WG_THREADS / PR;
+  vec8 stage_k[NP][2];
+  vec8 stage_v[NP][2];
+  int rows[NP][2];
+  const int my_pc = tid % PR;
+  const int my_pr = tid / PR;
 
   auto key_row = [&](int ci, int r) -> int {  // original row of key r of chunk ci, or -1
     if (GATHER) {
@@ -186,45 +214,41 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void attn_fwd_kernel
     return row < p.n_k ? row : -1;
   };
 
-  auto load_chunk = [&](int ci) {
+  auto fetch_rows = [&](int ci) {
 #pragma unroll
-    for (int j = 0; j < NPK; ++j) {
-      const int i = tid + j * WG_THREADS;
-      const int r = i / PR, pc = i % PR;
-      const int row = key_row(ci, r);
-      vec8 z = {};
-      if (row >= 0) z = *reinterpret_cast<const vec8*>(kb + (int64_t)row * p.k_sn + pc * 8);
-      stage_k[j] = z;
-    }
+    for (int j = 0; j < NP; ++j)
 #pragma unroll
-    for (int j = 0; j < NPV; ++j) {
-      const int i = tid + j * WG_THREADS;
-      const int pr = i / PV, pc = i % PV;
+      for (int u = 0; u < 2; ++u) rows[j][u] = key_row(ci, (my_pr + j * PAIRS_PER_PASS) * 2 + u);
+  };
+
+  auto load_chunk = [&]() {
+#pragma unroll
+    for (int j = 0; j < NP; ++j)
 #pragma unroll
       for (int u = 0; u < 2; ++u) {
-        const int row = key_row(ci, pr * 2 + u);
-        vec8 z = {};
-        if (row >= 0) z = *reinterpret_cast<const vec8*>(vb + (int64_t)row * p.v_sn + pc * 8);
-        stage_v[j][u] = z;
+        vec8 zk = {}, zv = {};
+        if (rows[j][u] >= 0) {
+          zk = *reinterpret_cast<const vec8*>(kb + (int64_t)rows[j][u] * p.k_sn + my_pc * 8);
+          zv = *reinterpret_cast<const vec8*>(vb + (int64_t)rows[j][u] * p.v_sn + my_pc * 8);
+        }
+        stage_k[j][u] = zk;
+        stage_v[j][u] = zv;
       }
-    }
   };
 
   auto store_chunk = [&](int buf) {
 #pragma unroll
-    for (int j = 0; j < NPK; ++j) {
-      const int i = tid + j * WG_THREADS;
-      const int r = i / PR, pc = i % PR;
-      *reinterpret_cast<vec8*>(&lds_k[buf][r * D + ((pc ^ (r & 7)) * 8)]) = stage_k[j];
-    }
+    for (int j = 0; j < NP; ++j) {
+      const int r0 = (my_pr + j * PAIRS_PER_PASS) * 2;
 #pragma unroll
-    for (int j = 0; j < NPV; ++j) {
-      const int i = tid + j * WG_THREADS;
-      const int pr = i / PV, pc = i % PV;
-      const int pos = vt_key_pos(pr * 2);
+      for (int u = 0; u < 2; ++u) {
+        const int r = r0 + u;
+        *reinterpret_cast<vec8*>(&lds_k[buf][r * D + ((my_pc ^ (r & 7)) * 8)]) = stage_k[j][u];
+      }
+      const int pos = vt_key_pos(r0);
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        const int dvrow = pc * 8 + e;
+        const int dvrow = my_pc * 8 + e;
         vec2 pair;
         pair[0] = stage_v[j][0][e];
         pair[1] = stage_v[j][1][e];
@@ -234,7 +258,9 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void attn_fwd_kernel
   };
 
   if (n_chunks > 0) {
-    load_chunk(0);
+    fetch_rows(0);
+    load_chunk();
+    if (n_chunks > 1) fetch_rows(1);
     store_chunk(0);
   }
   __syncthreads();
@@ -242,7 +268,10 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void attn_fwd_kernel
   for (int ci = 0; ci < n_chunks; ++ci) {
     const int buf = ci & 1;
     const bool more = ci + 1 < n_chunks;
-    if (more) load_chunk(ci + 1);
+    if (more) {
+      load_chunk();                            // rows of chunk ci+1 (fetched one iteration ago)
+      if (ci + 2 < n_chunks) fetch_rows(ci + 2);  // in flight during this chunk's compute
+    }
 
     bool active = true;
     bool need_mask = false;
@@ -295,48 +324,68 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void attn_fwd_kernel
           }
       }
 
-      // ---- online soft-max (base 2) ----------------------------------------------------------
+      // ---- online soft-max (base 2) with a lazily updated reference maximum ---------------------
+      // m_run is only raised when some row's maximum exceeds it by more than RESCALE_SLACK (in log2
+      // units), so the accumulator rescale is skipped in most chunks; until then p may grow up to
+      // 2^RESCALE_SLACK, which fp16/bf16 and the fp32 sums hold comfortably.
+      float mx[2];
+      bool grow = false;
 #pragma unroll
       for (int nb = 0; nb < 2; ++nb) {
-        float mx = s[0][nb][0];
+        float v = s[0][nb][0];
 #pragma unroll
         for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
-          for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[mb][nb][i]);
-        mx = fmaxf(mx, __shfl_xor(mx, 32));
-        const float m_new = fmaxf(m_run[nb], mx * p.scale_log2);
-        const float alpha = __builtin_amdgcn_exp2f(m_run[nb] - m_new);
-        m_run[nb] = m_new;
-        float sum = 0.f;
+          for (int i = 0; i < 16; ++i) v = fmaxf(v, s[mb][nb][i]);
+        v = fmaxf(v, __shfl_xor(v, 32)) * p.scale_log2;
+        mx[nb] = v;
+        grow = grow || (v > m_run[nb] + RESCALE_SLACK);
+      }
+      if (__any(grow)) {
 #pragma unroll
-        for (int mb = 0; mb < 2; ++mb)
+        for (int nb = 0; nb < 2; ++nb) {
+          const float m_new = fmaxf(m_run[nb], mx[nb]);
+          const float alpha = __builtin_amdgcn_exp2f(m_run[nb] - m_new);
+          m_run[nb] = m_new;
+          l_run[nb] *= alpha;
 #pragma unroll
-          for (int i = 0; i < 16; ++i) {
-            const float pe = __builtin_amdgcn_exp2f(__builtin_fmaf(s[mb][nb][i], p.scale_log2, -m_new));
-            s[mb][nb][i] = pe;
-            sum += pe;
+          for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) acc[db][nb][i] *= alpha;
+        }
+      }
+
+      // p = 2^(s*scale - m), rounded to the input type; row sums are taken over the rounded values
+      vec8 pb[KC / 16][2];
+#pragma unroll
+      for (int nb = 0; nb < 2; ++nb) {
+        const float m_use = m_run[nb];
+        float sum = l_run[nb];
+#pragma unroll
+        for (int ks = 0; ks < KC / 16; ++ks) {
+#pragma unroll
+          for (int e = 0; e < 8; e += 2) {
+            const int i = (ks & 1) * 8 + e;
+            vec2 pp;
+            pp[0] = (T)__builtin_amdgcn_exp2f(__builtin_fmaf(s[ks >> 1][nb][i], p.scale_log2, -m_use));
+            pp[1] = (T)__builtin_amdgcn_exp2f(__builtin_fmaf(s[ks >> 1][nb][i + 1], p.scale_log2, -m_use));
+            sum = Mfma<T>::pair_sum(pp, sum);
+            pb[ks][nb][e] = pp[0];
+            pb[ks][nb][e + 1] = pp[1];
           }
-        l_run[nb] = l_run[nb] * alpha + sum;
-#pragma unroll
-        for (int db = 0; db < DB; ++db)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) acc[db][nb][i] *= alpha;
+        }
+        l_run[nb] = sum;
       }
 
       // ---- O^T += V^T P^T ---------------------------------------------------------------------
 #pragma unroll
       for (int ks = 0; ks < KC / 16; ++ks) {
-        vec8 pb[2];
-#pragma unroll
-        for (int nb = 0; nb < 2; ++nb)
-#pragma unroll
-          for (int e = 0; e < 8; ++e) pb[nb][e] = (T)s[ks >> 1][nb][(ks & 1) * 8 + e];
 #pragma unroll
         for (int db = 0; db < DB; ++db) {
           const int dvrow = db * 32 + col;
           const vec8 a = *reinterpret_cast<const vec8*>(&lds_vt[buf][dvrow * KC + (((ks * 2 + hi) ^ vt_swizzle(dvrow)) * 8)]);
 #pragma unroll
-          for (int nb = 0; nb < 2; ++nb) acc[db][nb] = Mfma<T>::run(a, pb[nb], acc[db][nb]);
+          for (int nb = 0; nb < 2; ++nb) acc[db][nb] = Mfma<T>::run(a, pb[ks][nb], acc[db][nb]);
         }
       }
     }
