@@ -6,19 +6,32 @@
 //
 // Work decomposition.  A workgroup of 4 waves owns 256 consecutive (sorted) query positions of one
 // (virtual) head; wave w owns 64 of them as two 32-wide MFMA column blocks.  Keys are streamed in
-// chunks of 64 rows through double-buffered LDS: K row-major, V transposed so that both MFMA
-// operands are read as 16-byte ds_reads.  16-byte pieces are XOR-swizzled instead of padded.
+// chunks of 64 rows straight from HBM into LDS (global_load_lds, 16 bytes per lane, no staging
+// registers), K and V both row-major with their 16-byte pieces XOR-swizzled by the row number (the
+// swizzle is applied on the source side: a lane fetches the piece that belongs in its LDS slot).
+// The K operand is read with ds_read_b128, the V^T operand with the transposing ds_read_b64_tr_b16.
 //
 // MFMA formulation (v_mfma_f32_32x32x16_{f16,bf16}; A: lane -> row lane%32, k = 8*(lane/32)..+7;
 // B: lane -> column lane%32, same k; C: lane -> column lane%32, rows 8*(i/4) + 4*(lane/32) + i%4):
 //   S^T = K  Q^T   (M = keys,  N = queries, K = head dim)   -> a lane holds 16 keys of ONE query
 //   O^T = V^T P^T  (M = dv,    N = queries, K = keys)       -> P^T comes straight from the S^T registers
 // so the soft-max statistics (running max, running sum) are per-lane scalars; only one exchange
-// with lane^32 per chunk is needed for the row maximum.  The key order inside every group of 16 is
-// permuted in the transposed V tile to match the C-register -> B-operand reuse.
+// with lane^32 per 32 keys is needed for the row maximum.  ds_read_b64_tr_b16 gives lane i of a
+// 16-lane group element i%4 of the 8-byte words addressed by lanes 4j + i/4 (j = 0..3), so a group
+// that points its lanes at (key j, dv word w) receives V[key 0..3][dv base + i]: the V^T operand in
+// exactly the key order of the C registers.
+//
+// Software pipeline.  On this hardware a wave's MFMAs overlap only with vector instructions of the
+// SAME wave, so the loop is pipelined in steps of 32 keys: the straight-line block that soft-maxes
+// the S^T block of 32 keys (exp, rounding, row sums) and multiplies it into O also issues the MFMAs
+// of the NEXT 32-key S^T block, and the LDS operands of a step are fetched into registers one step
+// (K) or half a step (V) before the MFMAs that use them.  K therefore runs one chunk ahead of V in
+// LDS.  Two waves per SIMD keep the vector pipe fed (256 registers each at d = 64).
 //
 // The soft-max runs in base 2 (scale*log2(e) folded into one FMA, v_exp_f32 is 2^x); P is rounded
-// to the input type before P.V as the reference does (src/hyper_attn_triton.py:135).
+// to the input type before P.V as the reference does (src/hyper_attn_triton.py:135) and the row sums
+// are taken over the rounded values.  The running maximum is only raised when a row exceeds it by
+// more than 2^RESCALE_SLACK, which removes the accumulator rescale from almost every step.
 #include "ha_common.h"
 #include "attn_fwd.h"
 
@@ -30,6 +43,7 @@ constexpr int KC = 64;           // keys per LDS chunk
 constexpr float LOG2E = 1.4426950408889634f;
 constexpr float LN2 = 0.6931471805599453f;
 constexpr float RESCALE_SLACK = 8.0f;  // log2 units
+constexpr int NUM_XCD = 8;
 
 template <typename T>
 struct Mfma;
@@ -55,43 +69,183 @@ struct Mfma<bf16_t> {
   }
 };
 
-// position of key k (0..63) inside the transposed V tile: within each group of 16 keys the order is
-// 0-3, 8-11, 4-7, 12-15, so that lane half `hi` of the MFMA reads its 8 keys contiguously
-__device__ __forceinline__ int vt_key_pos(int k) {
-  const int k16 = k & 15;
-  return (k & ~15) + ((k16 >> 2) & 1) * 8 + (k16 >> 3) * 4 + (k16 & 3);
-}
-__device__ __forceinline__ int vt_swizzle(int dvrow) { return (dvrow & 7) ^ ((dvrow >> 3) & 7); }
-
-constexpr int NUM_XCD = 8;
+// Workgroups are handed to the 8 XCDs round-robin by their linear id, and each XCD has its own L2.
+// Re-number them so that every XCD works through one contiguous range of (head, query tile): the
+// query tiles that share a head's K/V then meet in the same L2.
 __device__ __forceinline__ int xcd_contiguous_id(int linear, int total) {
   const int xcd = linear % NUM_XCD, k = linear / NUM_XCD;
   const int q = total / NUM_XCD, r = total % NUM_XCD;
   return xcd * q + (xcd < r ? xcd : r) + k;
 }
 
+// LDS byte offsets of one lane's operand reads, relative to a tile base (fixed for the whole kernel).
+template <int D>
+struct LaneOffsets {
+  int k[D / 16];  // K operand piece of k-step ks for key row `col` (add mb*32 rows)
+  int v[D / 32];  // V^T operand word for dv block db, keys 0..3 (+4 for the upper lane half) of a 16-key step
+};
+
+// 16-byte piece `piece` of row `row` of a row-major [rows][D] 2-byte tile, XOR-swizzled; byte offset
+template <int D>
+__device__ __forceinline__ int tile_offset(int row, int piece) {
+  return row * D * 2 + ((piece ^ (row & 7)) << 4);
+}
+
+template <typename T>
+__device__ __forceinline__ typename ElemTraits<T>::vec8 lds_read_k(const unsigned char* tile, int off) {
+  return *reinterpret_cast<const typename ElemTraits<T>::vec8*>(tile + off);
+}
+
+// 8 keys x 1 dv column of V, transposed by the LDS unit: two 4-key reads
+template <typename T>
+__device__ __forceinline__ typename ElemTraits<T>::vec8 lds_read_vt(const unsigned char* tile, int off, int row_bytes) {
+#if defined(__HIP_DEVICE_COMPILE__)  // the builtin only exists in the device pass
+  typedef short s16x4 __attribute__((ext_vector_type(4)));
+  typedef short s16x8 __attribute__((ext_vector_type(8)));
+  typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+  const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(tile + off));
+  const s16x4 hi8 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(tile + off + 8 * row_bytes));
+  const s16x8 both = __builtin_shufflevector(lo, hi8, 0, 1, 2, 3, 4, 5, 6, 7);
+  return __builtin_bit_cast(typename ElemTraits<T>::vec8, both);
+#else
+  return typename ElemTraits<T>::vec8{};
+#endif
+}
+
+// 16 bytes per lane from global memory straight into LDS at lds_dst + lane*16 (lds_dst wave-uniform)
+__device__ __forceinline__ void global_to_lds_16(const void* src, unsigned char* lds_dst) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  typedef __attribute__((address_space(3))) unsigned char lds_byte;
+  __builtin_amdgcn_global_load_lds(src, (lds_byte*)lds_dst, 16, 0, 0);
+#endif
+}
+
+// One pipeline step over 32 keys.
+//   s_use  : S^T of the 32 keys being consumed (per query block nb), complete on entry
+//   s_fill : receives S^T of the next 32 keys, from the K operands kf (already in registers)
+//   kf     : on entry the K operands of this step's MFMAs; on exit those of the next step, read from
+//            rows mb_pref*32.. of the K tile k_pref
+//   v_tile : V tile of the chunk being consumed; khalf selects its keys 32*khalf..+31
+template <typename T, int D>
+__device__ __forceinline__ void pipeline_step(f32x16 (&s_use)[2], f32x16 (&s_fill)[2],
+                                              typename ElemTraits<T>::vec8 (&kf)[D / 16],
+                                              const unsigned char* k_pref, int mb_pref,
+                                              const unsigned char* v_tile, int khalf, const LaneOffsets<D>& lo,
+                                              const typename ElemTraits<T>::vec8 (&qf)[2][D / 16],
+                                              f32x16 (&acc)[D / 32][2], float (&m_run)[2], float (&l_run)[2],
+                                              float scale_log2) {
+  typedef typename ElemTraits<T>::vec8 vec8;
+  typedef typename ElemTraits<T>::vec2 vec2;
+  constexpr int KSTEPS = D / 16;
+  constexpr int DB = D / 32;
+
+  // operands for later: V^T of this step's first 16 keys, K of the next step
+  vec8 vf[DB];
+#pragma unroll
+  for (int db = 0; db < DB; ++db) vf[db] = lds_read_vt<T>(v_tile, lo.v[db] + khalf * 32 * D * 2, D * 2);
+  vec8 kf_next[KSTEPS];
+#pragma unroll
+  for (int ks = 0; ks < KSTEPS; ++ks) kf_next[ks] = lds_read_k<T>(k_pref, lo.k[ks] + mb_pref * 32 * D * 2);
+
+  // row maxima of the 32 keys; raise the reference maximum only when needed (wave-uniform branch)
+  float mx[2];
+  bool grow = false;
+#pragma unroll
+  for (int nb = 0; nb < 2; ++nb) {
+    float v = s_use[nb][0];
+#pragma unroll
+    for (int i = 1; i < 16; ++i) v = fmaxf(v, s_use[nb][i]);
+    v = fmaxf(v, __shfl_xor(v, 32)) * scale_log2;
+    mx[nb] = v;
+    grow = grow || (v > m_run[nb] + RESCALE_SLACK);
+  }
+  if (__any(grow)) {
+#pragma unroll
+    for (int nb = 0; nb < 2; ++nb) {
+      const float m_new = fmaxf(m_run[nb], mx[nb]);
+      const float alpha = __builtin_amdgcn_exp2f(m_run[nb] - m_new);
+      m_run[nb] = m_new;
+      l_run[nb] *= alpha;
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[db][nb][i] *= alpha;
+    }
+  }
+
+  // ---- straight-line block: next S^T MFMAs | exp, round, row sums | P V MFMAs ---------------------
+#pragma unroll
+  for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) s_fill[nb][i] = 0.f;
+#pragma unroll
+  for (int ks = 0; ks < KSTEPS; ++ks)
+#pragma unroll
+    for (int nb = 0; nb < 2; ++nb) s_fill[nb] = Mfma<T>::run(kf[ks], qf[nb][ks], s_fill[nb]);
+
+#pragma unroll
+  for (int ks2 = 0; ks2 < 2; ++ks2) {
+    vec8 pb[2];
+#pragma unroll
+    for (int nb = 0; nb < 2; ++nb) {
+      // rows that have seen no key yet (every key so far masked) keep m_run = -inf: use 0 there
+      const float m_use = m_run[nb] == -INFINITY ? 0.f : m_run[nb];
+      float sum = l_run[nb];
+#pragma unroll
+      for (int e = 0; e < 8; e += 2) {
+        const int i = ks2 * 8 + e;
+        vec2 pp;
+        pp[0] = (T)__builtin_amdgcn_exp2f(__builtin_fmaf(s_use[nb][i], scale_log2, -m_use));
+        pp[1] = (T)__builtin_amdgcn_exp2f(__builtin_fmaf(s_use[nb][i + 1], scale_log2, -m_use));
+        sum = Mfma<T>::pair_sum(pp, sum);
+        pb[nb][e] = pp[0];
+        pb[nb][e + 1] = pp[1];
+      }
+      l_run[nb] = sum;
+    }
+    vec8 vf2[DB];
+    if (ks2 == 0) {
+#pragma unroll
+      for (int db = 0; db < DB; ++db) vf2[db] = lds_read_vt<T>(v_tile, lo.v[db] + (khalf * 32 + 16) * D * 2, D * 2);
+    }
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int nb = 0; nb < 2; ++nb) acc[db][nb] = Mfma<T>::run(vf[db], pb[nb], acc[db][nb]);
+    if (ks2 == 0) {
+#pragma unroll
+      for (int db = 0; db < DB; ++db) vf[db] = vf2[db];
+    }
+  }
+#pragma unroll
+  for (int ks = 0; ks < KSTEPS; ++ks) kf[ks] = kf_next[ks];
+}
+
+}  // namespace
+
 template <typename T, int D, bool GATHER, bool CAUSAL>
-__global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void attn_fwd_kernel(const ha_attn_kernel_params p) {
+__global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_kernel(const ha_attn_kernel_params p) {
   typedef typename ElemTraits<T>::vec8 vec8;
   typedef typename ElemTraits<T>::vec4 vec4;
   typedef typename ElemTraits<T>::vec2 vec2;
   constexpr int DV = D;
-  constexpr int KSTEPS = D / 16;      // MFMA k-steps of Q.K^T
-  constexpr int DB = DV / 32;         // 32-row blocks of O^T
-  constexpr int PR = D / 8;           // 16-byte pieces per K row
-  constexpr int PV = DV / 8;          // 16-byte pieces per V row
+  constexpr int KSTEPS = D / 16;  // MFMA k-steps of Q.K^T
+  constexpr int DB = DV / 32;     // 32-row blocks of O^T
+  constexpr int PR = D / 8;       // 16-byte pieces per K (and V) row
 
-  __shared__ __attribute__((aligned(16))) T lds_k[2][KC * D];
-  __shared__ __attribute__((aligned(16))) T lds_vt[2][DV * KC];
+  // Four separate LDS objects (two K tiles, two V tiles of KC rows): the compiler then knows that a
+  // tile being filled from HBM and a tile being read do not alias, and does not serialise them.
+  constexpr int TILE_BYTES = KC * D * 2;
+  __shared__ __attribute__((aligned(16))) unsigned char lds_k0[TILE_BYTES];
+  __shared__ __attribute__((aligned(16))) unsigned char lds_k1[TILE_BYTES];
+  __shared__ __attribute__((aligned(16))) unsigned char lds_v0[TILE_BYTES];
+  __shared__ __attribute__((aligned(16))) unsigned char lds_v1[TILE_BYTES];
 
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63;
   const int hi = lane >> 5, col = lane & 31;
 
   // ---- which (virtual) head and query tile -----------------------------------------------------
-  // Workgroups are handed to the 8 XCDs round-robin by their linear id, and each XCD has its own
-  // L2.  Re-number them so that every XCD works through one contiguous range of (head, query tile):
-  // the query tiles that share a head's K/V then meet in the same L2.
   const int wg = xcd_contiguous_id(blockIdx.x, gridDim.x);
   const int qtiles = (p.n_q + WG_QUERIES - 1) / WG_QUERIES;
   const int vhead = wg / qtiles;
@@ -109,47 +263,6 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void attn_fwd_kernel
   const int64_t qidx_off = b * p.qi_sb + h * p.qi_sh + (int64_t)seg * p.n_q * p.qi_sn;
   const int64_t kidx_off = b * p.ki_sb + hk * p.ki_sh + (int64_t)seg * p.n_k * p.ki_sn;
   const int64_t sidx_off = b * p.si_sb + hk * p.si_sh;
-
-  // original row of sorted query position pq of this head, or -1 past the end
-  auto query_row = [&](int pq) -> int {
-    if (pq >= p.n_q) return -1;
-    return GATHER ? ha_load_idx(p.q_idx, qidx_off + (int64_t)pq * p.qi_sn, p.idx64) : pq;
-  };
-
-  // ---- Q fragments (B operand), soft-max state, accumulators ------------------------------------
-  vec8 qf[2][KSTEPS];
-  float m_run[2], l_run[2];
-  f32x16 acc[DB][2];
-  int qrow[2];
-#pragma unroll
-  for (int nb = 0; nb < 2; ++nb) {
-    qrow[nb] = query_row(qt * WG_QUERIES + wave * 64 + nb * 32 + col);
-#pragma unroll
-    for (int ks = 0; ks < KSTEPS; ++ks) {
-      vec8 z = {};
-      if (qrow[nb] >= 0) z = *reinterpret_cast<const vec8*>(qb + (int64_t)qrow[nb] * p.q_sn + ks * 16 + hi * 8);
-      qf[nb][ks] = z;
-    }
-    m_run[nb] = -INFINITY;
-    l_run[nb] = 0.f;
-#pragma unroll
-    for (int db = 0; db < DB; ++db)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) acc[db][nb][i] = 0.f;
-    if (p.accumulate && qrow[nb] >= 0) {
-      // resume from a previous partial attention: weight exp(lse_prev) with normalised output
-      m_run[nb] = lb[qrow[nb]] * LOG2E;
-      l_run[nb] = hi == 0 ? 1.f : 0.f;
-#pragma unroll
-      for (int db = 0; db < DB; ++db)
-#pragma unroll
-        for (int q4 = 0; q4 < 4; ++q4) {
-          const vec4 o = *reinterpret_cast<const vec4*>(ob + (int64_t)qrow[nb] * p.o_sn + db * 32 + q4 * 8 + hi * 4);
-#pragma unroll
-          for (int e = 0; e < 4; ++e) acc[db][nb][q4 * 4 + e] = (float)o[e];
-        }
-    }
-  }
 
   // ---- key-chunk schedule -------------------------------------------------------------------
   // chunk positions are in units of KC sorted keys, "unwrapped" (taken modulo n_k/KC when used)
@@ -188,20 +301,21 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void attn_fwd_kernel
   }
   const int wave_q_first = qt * WG_QUERIES + wave * 64;
 
-  // ---- staging: global -> registers -> LDS ------------------------------------------------------
-  // Every thread owns the same 16-byte piece `pc` of two adjacent key rows (pair `pr`) of the chunk,
-  // for K and for V (NP passes when a row has more than 8 pieces).  The original row numbers of the
-  // chunk after next are fetched while the current one is computed, so the row loads never wait for
-  // an index load.
-  constexpr int NP = (KC / 2) * PR / WG_THREADS;  // 1 for d = 64, 2 for d = 128
-  constexpr int PAIRS_PER_PASS = WG_THREADS / PR;
-  vec8 stage_k[NP][2];
-  vec8 stage_v[NP][2];
-  int rows[NP][2];
-  const int my_pc = tid % PR;
-  const int my_pr = tid / PR;
+  // ---- tiles: HBM -> LDS without passing through registers ----------------------------------------
+  // One global_load_lds moves 16 bytes per lane to 1 KB of consecutive LDS: 64/PR rows of a tile.
+  // Wave w issues loads LPW*w .. LPW*w + LPW-1 of a tile.  A lane's LDS slot is (row, physical piece
+  // lane % PR); it fetches the logical piece that the swizzle puts there.  Original row numbers are
+  // fetched one chunk ahead of the rows, so a row load never waits for an index load.
+  constexpr int ROWS_PER_LOAD = 64 / PR;
+  constexpr int LPW = PR / 4;  // loads per wave per tile
+  int rows_k[LPW], rows_v[LPW];
+  const int my_pp = lane % PR;           // physical piece of this lane's LDS slot
+  const int my_lr = lane / PR;           // row inside one load
 
-  auto key_row = [&](int ci, int r) -> int {  // original row of key r of chunk ci, or -1
+  // original row of key r of chunk ci; chunks past the end and rows past n_k alias row 0 (their
+  // scores are masked or never used, and row 0 holds finite data)
+  auto key_row = [&](int ci, int r) -> int {
+    if (ci >= n_chunks) return 0;
     if (GATHER) {
       if (ci < n_blk_chunks) {
         const int pos = ((uni_start + ci) % nk_chunks) * KC + r;
@@ -211,240 +325,201 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void attn_fwd_kernel
       return p.sampled_idx ? ha_load_idx(p.sampled_idx, sidx_off + s, p.idx64) : s;
     }
     const int row = ci * KC + r;
-    return row < p.n_k ? row : -1;
+    return row < p.n_k ? row : 0;
   };
-
-  auto fetch_rows = [&](int ci) {
-#pragma unroll
-    for (int j = 0; j < NP; ++j)
-#pragma unroll
-      for (int u = 0; u < 2; ++u) rows[j][u] = key_row(ci, (my_pr + j * PAIRS_PER_PASS) * 2 + u);
-  };
-
-  auto load_chunk = [&]() {
-#pragma unroll
-    for (int j = 0; j < NP; ++j)
-#pragma unroll
-      for (int u = 0; u < 2; ++u) {
-        vec8 zk = {}, zv = {};
-        if (rows[j][u] >= 0) {
-          zk = *reinterpret_cast<const vec8*>(kb + (int64_t)rows[j][u] * p.k_sn + my_pc * 8);
-          zv = *reinterpret_cast<const vec8*>(vb + (int64_t)rows[j][u] * p.v_sn + my_pc * 8);
-        }
-        stage_k[j][u] = zk;
-        stage_v[j][u] = zv;
-      }
-  };
-
-  auto store_chunk = [&](int buf) {
-#pragma unroll
-    for (int j = 0; j < NP; ++j) {
-      const int r0 = (my_pr + j * PAIRS_PER_PASS) * 2;
-#pragma unroll
-      for (int u = 0; u < 2; ++u) {
-        const int r = r0 + u;
-        *reinterpret_cast<vec8*>(&lds_k[buf][r * D + ((my_pc ^ (r & 7)) * 8)]) = stage_k[j][u];
-      }
-      const int pos = vt_key_pos(r0);
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const int dvrow = my_pc * 8 + e;
-        vec2 pair;
-        pair[0] = stage_v[j][0][e];
-        pair[1] = stage_v[j][1][e];
-        *reinterpret_cast<vec2*>(&lds_vt[buf][dvrow * KC + (((pos >> 3) ^ vt_swizzle(dvrow)) * 8) + (pos & 7)]) = pair;
-      }
-    }
-  };
-
-  if (n_chunks > 0) {
-    fetch_rows(0);
-    load_chunk();
-    if (n_chunks > 1) fetch_rows(1);
-    store_chunk(0);
+#define HA_FETCH_ROWS(ci, rows) \
+  _Pragma("unroll") for (int j = 0; j < LPW; ++j) rows[j] = key_row((ci), (wave * LPW + j) * ROWS_PER_LOAD + my_lr);
+#define HA_LOAD_TILE(base, stride, rows, tile)                                                           \
+  _Pragma("unroll") for (int j = 0; j < LPW; ++j) {                                                      \
+    const int r = (wave * LPW + j) * ROWS_PER_LOAD + my_lr;                                              \
+    const T* src = (base) + (int64_t)rows[j] * (stride) + ((my_pp ^ (r & 7)) << 3);                      \
+    global_to_lds_16(src, (tile) + (wave * LPW + j) * 1024);                                             \
   }
+
+  // first loads: indices of the queries and of the first key chunks, then the rows themselves
+  int qrow[2];
+#pragma unroll
+  for (int nb = 0; nb < 2; ++nb) {
+    const int pq = qt * WG_QUERIES + wave * 64 + nb * 32 + col;
+    qrow[nb] = pq >= p.n_q ? -1 : (GATHER ? ha_load_idx(p.q_idx, qidx_off + (int64_t)pq * p.qi_sn, p.idx64) : pq);
+  }
+  HA_FETCH_ROWS(0, rows_k)
+  HA_FETCH_ROWS(0, rows_v)
+  HA_LOAD_TILE(kb, p.k_sn, rows_k, lds_k0)
+  HA_LOAD_TILE(vb, p.v_sn, rows_v, lds_v0)
+  HA_FETCH_ROWS(1, rows_k)
+  HA_LOAD_TILE(kb, p.k_sn, rows_k, lds_k1)
+  HA_FETCH_ROWS(2, rows_k)
+  HA_FETCH_ROWS(1, rows_v)
+
+  // ---- Q fragments (B operand), soft-max state, accumulators ------------------------------------
+  vec8 qf[2][KSTEPS];
+  float m_run[2], l_run[2];
+  f32x16 acc[DB][2];
+#pragma unroll
+  for (int nb = 0; nb < 2; ++nb) {
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) {
+      vec8 z = {};
+      if (qrow[nb] >= 0) z = *reinterpret_cast<const vec8*>(qb + (int64_t)qrow[nb] * p.q_sn + ks * 16 + hi * 8);
+      qf[nb][ks] = z;
+    }
+    m_run[nb] = -INFINITY;
+    l_run[nb] = 0.f;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[db][nb][i] = 0.f;
+    if (p.accumulate && qrow[nb] >= 0) {
+      // resume from a previous partial attention: weight exp(lse_prev) with normalised output
+      m_run[nb] = lb[qrow[nb]] * LOG2E;
+      l_run[nb] = hi == 0 ? 1.f : 0.f;
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4) {
+          const vec4 o = *reinterpret_cast<const vec4*>(ob + (int64_t)qrow[nb] * p.o_sn + db * 32 + q4 * 8 + hi * 4);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) acc[db][nb][q4 * 4 + e] = (float)o[e];
+        }
+    }
+  }
+
+  // per-lane LDS offsets of the MFMA operand reads
+  LaneOffsets<D> lo;
+#pragma unroll
+  for (int ks = 0; ks < KSTEPS; ++ks) lo.k[ks] = tile_offset<D>(col, ks * 2 + hi);
+  {
+    // transposing read: lane s = 4j + w of a 16-lane group addresses key j (+4 for the upper lane
+    // half), dv word w of the 16 dv columns of its group
+    const int g = lane >> 4, sl = lane & 15;
+    const int key = (g >> 1) * 4 + (sl >> 2);
+    const int w = sl & 3;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+      lo.v[db] = tile_offset<D>(key, db * 4 + (g & 1) * 2 + (w >> 1)) + (w & 1) * 8;
+  }
+
+  // every wave's part of K(0), V(0), K(1) has landed before anyone reads the tiles
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
   __syncthreads();
 
-  for (int ci = 0; ci < n_chunks; ++ci) {
-    const int buf = ci & 1;
-    const bool more = ci + 1 < n_chunks;
-    if (more) {
-      load_chunk();                            // rows of chunk ci+1 (fetched one iteration ago)
-      if (ci + 2 < n_chunks) fetch_rows(ci + 2);  // in flight during this chunk's compute
-    }
-
-    bool active = true;
-    bool need_mask = false;
-    if (GATHER) {
-      if (ci < n_blk_chunks) {
-        const int u = uni_start + ci;
-        active = u >= my_lo && u < my_hi;
-      }
-    } else {
-      const int k_first = ci * KC;
-      if (CAUSAL) {
-        active = k_first <= wave_q_first + 63;
-        need_mask = k_first + KC - 1 > wave_q_first;
-      }
-      need_mask = need_mask || (k_first + KC > p.n_k);
-    }
-
-    if (active) {
-      // ---- S^T = K Q^T ---------------------------------------------------------------------
-      f32x16 s[2][2];
-#pragma unroll
-      for (int mb = 0; mb < 2; ++mb)
-#pragma unroll
-        for (int nb = 0; nb < 2; ++nb)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) s[mb][nb][i] = 0.f;
-#pragma unroll
-      for (int ks = 0; ks < KSTEPS; ++ks) {
-#pragma unroll
-        for (int mb = 0; mb < 2; ++mb) {
-          const int key = mb * 32 + col;
-          const vec8 a = *reinterpret_cast<const vec8*>(&lds_k[buf][key * D + (((ks * 2 + hi) ^ (key & 7)) * 8)]);
-#pragma unroll
-          for (int nb = 0; nb < 2; ++nb) s[mb][nb] = Mfma<T>::run(a, qf[nb][ks], s[mb][nb]);
-        }
-      }
-
-      if (need_mask) {
-#pragma unroll
-        for (int mb = 0; mb < 2; ++mb)
-#pragma unroll
-          for (int nb = 0; nb < 2; ++nb) {
-            const int qpos = wave_q_first + nb * 32 + col;
-#pragma unroll
-            for (int i = 0; i < 16; ++i) {
-              const int key = ci * KC + mb * 32 + 8 * (i >> 2) + 4 * hi + (i & 3);
-              const bool dead = key >= p.n_k || (CAUSAL && key > qpos);
-              if (dead) s[mb][nb][i] = -INFINITY;
-            }
-          }
-      }
-
-      // ---- online soft-max (base 2) with a lazily updated reference maximum ---------------------
-      // m_run is only raised when some row's maximum exceeds it by more than RESCALE_SLACK (in log2
-      // units), so the accumulator rescale is skipped in most chunks; until then p may grow up to
-      // 2^RESCALE_SLACK, which fp16/bf16 and the fp32 sums hold comfortably.
-      float mx[2];
-      bool grow = false;
-#pragma unroll
-      for (int nb = 0; nb < 2; ++nb) {
-        float v = s[0][nb][0];
-#pragma unroll
-        for (int mb = 0; mb < 2; ++mb)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) v = fmaxf(v, s[mb][nb][i]);
-        v = fmaxf(v, __shfl_xor(v, 32)) * p.scale_log2;
-        mx[nb] = v;
-        grow = grow || (v > m_run[nb] + RESCALE_SLACK);
-      }
-      if (__any(grow)) {
-#pragma unroll
-        for (int nb = 0; nb < 2; ++nb) {
-          const float m_new = fmaxf(m_run[nb], mx[nb]);
-          const float alpha = __builtin_amdgcn_exp2f(m_run[nb] - m_new);
-          m_run[nb] = m_new;
-          l_run[nb] *= alpha;
-#pragma unroll
-          for (int db = 0; db < DB; ++db)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) acc[db][nb][i] *= alpha;
-        }
-      }
-
-      // p = 2^(s*scale - m), rounded to the input type; row sums are taken over the rounded values
-      vec8 pb[KC / 16][2];
-#pragma unroll
-      for (int nb = 0; nb < 2; ++nb) {
-        const float m_use = m_run[nb];
-        float sum = l_run[nb];
-#pragma unroll
-        for (int ks = 0; ks < KC / 16; ++ks) {
-#pragma unroll
-          for (int e = 0; e < 8; e += 2) {
-            const int i = (ks & 1) * 8 + e;
-            vec2 pp;
-            pp[0] = (T)__builtin_amdgcn_exp2f(__builtin_fmaf(s[ks >> 1][nb][i], p.scale_log2, -m_use));
-            pp[1] = (T)__builtin_amdgcn_exp2f(__builtin_fmaf(s[ks >> 1][nb][i + 1], p.scale_log2, -m_use));
-            sum = Mfma<T>::pair_sum(pp, sum);
-            pb[ks][nb][e] = pp[0];
-            pb[ks][nb][e + 1] = pp[1];
-          }
-        }
-        l_run[nb] = sum;
-      }
-
-      // ---- O^T += V^T P^T ---------------------------------------------------------------------
-#pragma unroll
-      for (int ks = 0; ks < KC / 16; ++ks) {
-#pragma unroll
-        for (int db = 0; db < DB; ++db) {
-          const int dvrow = db * 32 + col;
-          const vec8 a = *reinterpret_cast<const vec8*>(&lds_vt[buf][dvrow * KC + (((ks * 2 + hi) ^ vt_swizzle(dvrow)) * 8)]);
-#pragma unroll
-          for (int nb = 0; nb < 2; ++nb) acc[db][nb] = Mfma<T>::run(a, pb[ks][nb], acc[db][nb]);
-        }
-      }
-    }
-
-    if (more) store_chunk(buf ^ 1);
-    __syncthreads();
+  // ---- masks (wave-uniform decision per chunk) -------------------------------------------------
+  auto chunk_masked = [&](int ci) -> bool {
+    if (GATHER) return ci < n_blk_chunks && !(uni_start + ci >= my_lo && uni_start + ci < my_hi);
+    const int k_first = ci * KC;
+    return (CAUSAL && k_first + KC - 1 > wave_q_first) || (k_first + KC > p.n_k);
+  };
+#define HA_APPLY_MASK(ci, mb, s)                                               \
+  _Pragma("unroll") for (int nb = 0; nb < 2; ++nb) {                           \
+    const int qpos = wave_q_first + nb * 32 + col;                             \
+    _Pragma("unroll") for (int i = 0; i < 16; ++i) {                           \
+      const int key = (ci) * KC + (mb) * 32 + 8 * (i >> 2) + 4 * hi + (i & 3); \
+      const bool dead = GATHER || key >= p.n_k || (CAUSAL && key > qpos);      \
+      if (dead) s[nb][i] = -INFINITY;                                          \
+    }                                                                          \
   }
+
+  // ---- main loop -----------------------------------------------------------------------------------
+  // s_a / s_b hold S^T of keys 0..31 / 32..63 of the chunk being consumed.  On entry of iteration ci
+  // s_a is complete and kf holds the K operands of keys 32..63 of K(ci); step 0 consumes s_a, fills
+  // s_b and fetches the operands of keys 0..31 of K(ci+1); step 1 consumes s_b, fills s_a and fetches
+  // those of keys 32..63 of K(ci+1).  K(ci) itself is no longer read from LDS in iteration ci, so
+  // K(ci+2) streams into its buffer meanwhile, and V(ci+1) into the buffer V(ci-1) left.
+  f32x16 s_a[2], s_b[2];
+  vec8 kf[KSTEPS];
+  {
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) kf[ks] = lds_read_k<T>(lds_k0, lo.k[ks]);
+#pragma unroll
+    for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) s_a[nb][i] = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks)
+#pragma unroll
+      for (int nb = 0; nb < 2; ++nb) s_a[nb] = Mfma<T>::run(kf[ks], qf[nb][ks], s_a[nb]);
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) kf[ks] = lds_read_k<T>(lds_k0, lo.k[ks] + 32 * D * 2);
+  }
+  // all waves hold their operands of K(0): its buffer may be overwritten from iteration 0 on
+  __syncthreads();
+
+  // the loop is unrolled by two so that every tile access names its LDS object statically
+#define HA_ITERATION(ci, K_CUR, K_NXT, V_CUR, V_NXT)                                                        \
+  {                                                                                                         \
+    if ((ci) + 2 < n_chunks) { HA_LOAD_TILE(kb, p.k_sn, rows_k, K_CUR) } /* K(ci+2) */                      \
+    if ((ci) + 1 < n_chunks) { HA_LOAD_TILE(vb, p.v_sn, rows_v, V_NXT) } /* V(ci+1) */                      \
+    HA_FETCH_ROWS((ci) + 3, rows_k)                                                                         \
+    HA_FETCH_ROWS((ci) + 2, rows_v)                                                                         \
+    const bool masked = chunk_masked(ci);                                                                   \
+    if (masked) { HA_APPLY_MASK(ci, 0, s_a) }                                                               \
+    pipeline_step<T, D>(s_a, s_b, kf, K_NXT, 0, V_CUR, 0, lo, qf, acc, m_run, l_run, p.scale_log2);         \
+    if (masked) { HA_APPLY_MASK(ci, 1, s_b) }                                                               \
+    pipeline_step<T, D>(s_b, s_a, kf, K_NXT, 1, V_CUR, 1, lo, qf, acc, m_run, l_run, p.scale_log2);         \
+    __builtin_amdgcn_s_waitcnt(0x0F70); /* this wave's parts of K(ci+2), V(ci+1) have landed */             \
+    __syncthreads();                                                                                        \
+  }
+  for (int ci = 0; ci < n_chunks; ci += 2) {
+    HA_ITERATION(ci, lds_k0, lds_k1, lds_v0, lds_v1)
+    if (ci + 1 < n_chunks) HA_ITERATION(ci + 1, lds_k1, lds_k0, lds_v1, lds_v0)
+  }
+#undef HA_ITERATION
 
   // ---- epilogue: normalise, stage O through LDS, write whole rows ---------------------------------
-  // two halves of 128 queries each: the K buffers hold exactly 2*KC*D = 128*DV elements
-  T* lds_o = &lds_k[0][0];
-  static_assert(sizeof(lds_k) == (size_t)128 * DV * sizeof(T), "O staging tile");
-#pragma unroll 1
-  for (int half = 0; half < 2; ++half) {
-    if ((wave >> 1) == half) {
+  // A wave's 64 output rows are exactly one tile (64 rows of DV elements): wave w stages them in tile
+  // object w and writes them out itself, so no further workgroup barrier is needed.
+  unsigned char* const lds_o_raw = wave == 0 ? lds_k0 : (wave == 1 ? lds_k1 : (wave == 2 ? lds_v0 : lds_v1));
+  T* const lds_o = reinterpret_cast<T*>(lds_o_raw);
 #pragma unroll
-      for (int nb = 0; nb < 2; ++nb) {
-        const float l_tot = l_run[nb] + __shfl_xor(l_run[nb], 32);
-        const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
-        const int lrow = (wave & 1) * 64 + nb * 32 + col;  // row inside this half
-        if (hi == 0 && qrow[nb] >= 0)
-          lb[qrow[nb]] = l_tot > 0.f ? (m_run[nb] + __builtin_amdgcn_logf(l_tot)) * LN2 : -INFINITY;
+  for (int nb = 0; nb < 2; ++nb) {
+    const float l_tot = l_run[nb] + __shfl_xor(l_run[nb], 32);
+    const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+    const int lrow = nb * 32 + col;
+    if (hi == 0 && qrow[nb] >= 0)
+      lb[qrow[nb]] = l_tot > 0.f ? (m_run[nb] + __builtin_amdgcn_logf(l_tot)) * LN2 : -INFINITY;
 #pragma unroll
-        for (int db = 0; db < DB; ++db)
+    for (int db = 0; db < DB; ++db)
 #pragma unroll
-          for (int q4 = 0; q4 < 4; ++q4) {
-            vec4 o;
+      for (int q4 = 0; q4 < 4; ++q4) {
+        vec4 o;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) o[e] = (T)(acc[db][nb][q4 * 4 + e] * inv);
-            const int piece = db * 4 + q4;
-            *reinterpret_cast<vec4*>(&lds_o[lrow * DV + ((piece ^ (lrow & 7)) * 8) + hi * 4]) = o;
-          }
+        for (int e = 0; e < 4; ++e) o[e] = (T)(acc[db][nb][q4 * 4 + e] * inv);
+        const int piece = db * 4 + q4;
+        *reinterpret_cast<vec4*>(&lds_o[lrow * DV + ((piece ^ (lrow & 7)) * 8) + hi * 4]) = o;
       }
-    }
-    __syncthreads();
-    // 128 rows x PV pieces, all 256 threads
-#pragma unroll
-    for (int j = 0; j < 128 * PV / WG_THREADS; ++j) {
-      const int i = tid + j * WG_THREADS;
-      const int lrow = i / PV, pc = i % PV;
-      const int row = query_row(qt * WG_QUERIES + half * 128 + lrow);
-      if (row >= 0) {
-        const vec8 o = *reinterpret_cast<const vec8*>(&lds_o[lrow * DV + ((pc ^ (lrow & 7)) * 8)]);
-        *reinterpret_cast<vec8*>(ob + (int64_t)row * p.o_sn + pc * 8) = o;
-      }
-    }
-    __syncthreads();
   }
+  __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): this wave's LDS writes are done
+  __builtin_amdgcn_wave_barrier();
+#pragma unroll
+  for (int j = 0; j < 64 * PR / HA_WAVE; ++j) {
+    const int i = lane + j * HA_WAVE;
+    const int lrow = i / PR, pc = i % PR;
+    const int pq = qt * WG_QUERIES + wave * 64 + lrow;
+    if (pq < p.n_q) {
+      const int row = GATHER ? ha_load_idx(p.q_idx, qidx_off + (int64_t)pq * p.qi_sn, p.idx64) : pq;
+      const vec8 o = *reinterpret_cast<const vec8*>(&lds_o[lrow * DV + ((pc ^ (lrow & 7)) * 8)]);
+      *reinterpret_cast<vec8*>(ob + (int64_t)row * p.o_sn + pc * 8) = o;
+    }
+  }
+#undef HA_FETCH_ROWS
+#undef HA_LOAD_TILE
+#undef HA_APPLY_MASK
+}
+
+namespace {
+
+template <typename T, int D, bool GATHER, bool CAUSAL>
+int launch_one(const ha_attn_kernel_params& p, int grid, hipStream_t stream, const char* what) {
+  hipLaunchKernelGGL((ha_attn_fwd_kernel<T, D, GATHER, CAUSAL>), dim3(grid), dim3(WG_THREADS), 0, stream, p);
+  return ha_launch_status(what);
 }
 
 template <typename T, int D>
 int launch_variant(const ha_attn_kernel_params& p, int grid, bool gather, bool causal, hipStream_t stream) {
-  if (gather)
-    hipLaunchKernelGGL((attn_fwd_kernel<T, D, true, false>), dim3(grid), dim3(WG_THREADS), 0, stream, p);
-  else if (causal)
-    hipLaunchKernelGGL((attn_fwd_kernel<T, D, false, true>), dim3(grid), dim3(WG_THREADS), 0, stream, p);
-  else
-    hipLaunchKernelGGL((attn_fwd_kernel<T, D, false, false>), dim3(grid), dim3(WG_THREADS), 0, stream, p);
-  return ha_launch_status(gather ? "ha_block_attn_fwd" : "ha_flash_attn_fwd");
+  if (gather) return launch_one<T, D, true, false>(p, grid, stream, "ha_block_attn_fwd");
+  if (causal) return launch_one<T, D, false, true>(p, grid, stream, "ha_flash_attn_fwd");
+  return launch_one<T, D, false, false>(p, grid, stream, "ha_flash_attn_fwd");
 }
 
 }  // namespace
