@@ -343,12 +343,15 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
     const int pq = qt * WG_QUERIES + wave * 64 + nb * 32 + col;
     qrow[nb] = pq >= p.n_q ? -1 : (GATHER ? ha_load_idx(p.q_idx, qidx_off + (int64_t)pq * p.qi_sn, p.idx64) : pq);
   }
-  HA_FETCH_ROWS(0, rows_k)
-  HA_FETCH_ROWS(0, rows_v)
-  HA_LOAD_TILE(kb, p.k_sn, rows_k, lds_k0)
-  HA_LOAD_TILE(vb, p.v_sn, rows_v, lds_v0)
-  HA_FETCH_ROWS(1, rows_k)
-  HA_LOAD_TILE(kb, p.k_sn, rows_k, lds_k1)
+  {
+    int rows_k1[LPW];
+    HA_FETCH_ROWS(0, rows_k)
+    HA_FETCH_ROWS(0, rows_v)
+    HA_FETCH_ROWS(1, rows_k1)
+    HA_LOAD_TILE(kb, p.k_sn, rows_k, lds_k0)
+    HA_LOAD_TILE(vb, p.v_sn, rows_v, lds_v0)
+    HA_LOAD_TILE(kb, p.k_sn, rows_k1, lds_k1)
+  }
   HA_FETCH_ROWS(2, rows_k)
   HA_FETCH_ROWS(1, rows_v)
 
@@ -410,14 +413,16 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
     const int k_first = ci * KC;
     return (CAUSAL && k_first + KC - 1 > wave_q_first) || (k_first + KC > p.n_k);
   };
-#define HA_APPLY_MASK(ci, mb, s)                                               \
-  _Pragma("unroll") for (int nb = 0; nb < 2; ++nb) {                           \
-    const int qpos = wave_q_first + nb * 32 + col;                             \
-    _Pragma("unroll") for (int i = 0; i < 16; ++i) {                           \
-      const int key = (ci) * KC + (mb) * 32 + 8 * (i >> 2) + 4 * hi + (i & 3); \
-      const bool dead = GATHER || key >= p.n_k || (CAUSAL && key > qpos);      \
-      if (dead) s[nb][i] = -INFINITY;                                          \
-    }                                                                          \
+  // element i of a lane is key  first + 8*(i/4) + i%4  with first = chunk*64 + mb*32 + 4*hi; it is
+  // dead when that exceeds `limit` = min(n_k - 1, query position) (everything is dead in gather mode)
+#define HA_APPLY_MASK(ci, mb, s)                                                        \
+  _Pragma("unroll") for (int nb = 0; nb < 2; ++nb) {                                    \
+    const int first = (ci) * KC + (mb) * 32 + 4 * hi;                                   \
+    int limit = p.n_k - 1;                                                              \
+    if (CAUSAL) limit = min(limit, wave_q_first + nb * 32 + col);                       \
+    const int slack = GATHER ? -1 : limit - first;                                      \
+    _Pragma("unroll") for (int i = 0; i < 16; ++i)                                      \
+      if (8 * (i >> 2) + (i & 3) > slack) s[nb][i] = -INFINITY;                         \
   }
 
   // ---- main loop -----------------------------------------------------------------------------------
@@ -452,11 +457,14 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
     if ((ci) + 1 < n_chunks) { HA_LOAD_TILE(vb, p.v_sn, rows_v, V_NXT) } /* V(ci+1) */                      \
     HA_FETCH_ROWS((ci) + 3, rows_k)                                                                         \
     HA_FETCH_ROWS((ci) + 2, rows_v)                                                                         \
-    const bool masked = chunk_masked(ci);                                                                   \
-    if (masked) { HA_APPLY_MASK(ci, 0, s_a) }                                                               \
-    pipeline_step<T, D>(s_a, s_b, kf, K_NXT, 0, V_CUR, 0, lo, qf, acc, m_run, l_run, p.scale_log2);         \
-    if (masked) { HA_APPLY_MASK(ci, 1, s_b) }                                                               \
-    pipeline_step<T, D>(s_b, s_a, kf, K_NXT, 1, V_CUR, 1, lo, qf, acc, m_run, l_run, p.scale_log2);         \
+    /* causal: once a chunk lies wholly above this wave's queries, so do all later ones */                  \
+    if (!(CAUSAL && (ci) * KC > wave_q_first + 63)) {                                                       \
+      const bool masked = chunk_masked(ci);                                                                 \
+      if (masked) { HA_APPLY_MASK(ci, 0, s_a) }                                                             \
+      pipeline_step<T, D>(s_a, s_b, kf, K_NXT, 0, V_CUR, 0, lo, qf, acc, m_run, l_run, p.scale_log2);       \
+      if (masked) { HA_APPLY_MASK(ci, 1, s_b) }                                                             \
+      pipeline_step<T, D>(s_b, s_a, kf, K_NXT, 1, V_CUR, 1, lo, qf, acc, m_run, l_run, p.scale_log2);       \
+    }                                                                                                       \
     __builtin_amdgcn_s_waitcnt(0x0F70); /* this wave's parts of K(ci+2), V(ci+1) have landed */             \
     __syncthreads();                                                                                        \
   }
