@@ -53,32 +53,37 @@ __device__ __forceinline__ uint64_t match_digit(int digit, bool valid) {
   return mask;
 }
 
-__device__ __forceinline__ uint64_t lanemask_lt() {
-  const int lane = threadIdx.x & (HA_WAVE - 1);
-  return lane == 0 ? 0ull : (~0ull >> (HA_WAVE - lane));
+// number of set bits of `mask` below this lane
+__device__ __forceinline__ uint32_t rank_below(uint64_t mask) {
+  return __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0u));
+}
+
+__device__ __forceinline__ int load_digit(const ha_sort_job& job, const int32_t* prev, int64_t seg_base, int i,
+                                          int shift, int* src) {
+  const int s = prev ? prev[i] : i;
+  *src = s;
+  return (job.keys[seg_base + s] >> shift) & 255;
 }
 
 // ---- per-chunk histograms (only for segments longer than one chunk) -------------------------
+// Counting needs no order, so it uses LDS atomics.
 __global__ __launch_bounds__(SORT_THREADS) void sort_hist_kernel(ha_sort_jobs jobs) {
   __shared__ uint32_t hist[256];
   const BlockRef br = locate_block(jobs, blockIdx.x, false);
   const ha_sort_job& job = jobs.job[br.job];
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int tid = threadIdx.x;
   hist[tid] = 0;
   __syncthreads();
   const int64_t seg_base = job.seg_offset + (int64_t)br.seg * job.seg_stride;
   const int32_t* prev = job.prev ? job.prev + (int64_t)br.seg * job.seg_len : nullptr;
   const int chunk_start = br.chunk * HA_SORT_CHUNK;
+#pragma unroll 4
   for (int s = 0; s < SORT_STEPS; ++s) {
-    const int i = chunk_start + (wave * SORT_STEPS + s) * HA_WAVE + lane;
-    const bool valid = i < job.seg_len;
-    int digit = 0;
-    if (valid) {
-      const int src = prev ? prev[i] : i;
-      digit = (job.keys[seg_base + src] >> jobs.shift) & 255;
+    const int i = chunk_start + s * SORT_THREADS + tid;
+    if (i < job.seg_len) {
+      int src;
+      atomicAdd(&hist[load_digit(job, prev, seg_base, i, jobs.shift, &src)], 1u);
     }
-    const uint64_t m = match_digit(digit, valid);
-    if (valid && (m & lanemask_lt()) == 0) atomicAdd(&hist[digit], (uint32_t)__popcll(m));
   }
   __syncthreads();
   job.hist[((int64_t)br.seg * job.chunks_per_seg + br.chunk) * 256 + tid] = hist[tid];
@@ -119,6 +124,9 @@ __global__ __launch_bounds__(SORT_THREADS) void sort_scan_kernel(ha_sort_jobs jo
 }
 
 // ---- stable scatter --------------------------------------------------------------------------
+// A wave owns a contiguous run of the chunk (wave order = key order).  Pass 1 counts digits per wave
+// with LDS atomics; pass 2 re-reads the keys (they are cache resident) and ranks them inside each
+// 64-key step by ballot matching, which is what keeps equal keys in ascending row order.
 __global__ __launch_bounds__(SORT_THREADS) void sort_scatter_kernel(ha_sort_jobs jobs) {
   __shared__ uint32_t wave_hist[SORT_WAVES][256];
   __shared__ uint32_t wave_totals[SORT_WAVES];
@@ -131,24 +139,15 @@ __global__ __launch_bounds__(SORT_THREADS) void sort_scatter_kernel(ha_sort_jobs
 
   const int64_t seg_base = job.seg_offset + (int64_t)br.seg * job.seg_stride;
   const int32_t* prev = job.prev ? job.prev + (int64_t)br.seg * job.seg_len : nullptr;
-  const int chunk_start = br.chunk * HA_SORT_CHUNK;
-  const uint64_t lt = lanemask_lt();
+  const int wave_start = br.chunk * HA_SORT_CHUNK + wave * (SORT_STEPS * HA_WAVE);
 
-  int digit[SORT_STEPS];
-  int src[SORT_STEPS];
-  // pass 1: per-wave digit counts (a wave owns a contiguous run of the chunk, so wave order = key order)
-#pragma unroll
+#pragma unroll 4
   for (int s = 0; s < SORT_STEPS; ++s) {
-    const int i = chunk_start + (wave * SORT_STEPS + s) * HA_WAVE + lane;
-    const bool valid = i < job.seg_len;
-    digit[s] = 0;
-    src[s] = -1;
-    if (valid) {
-      src[s] = prev ? prev[i] : i;
-      digit[s] = (job.keys[seg_base + src[s]] >> jobs.shift) & 255;
+    const int i = wave_start + s * HA_WAVE + lane;
+    if (i < job.seg_len) {
+      int src;
+      atomicAdd(&wave_hist[wave][load_digit(job, prev, seg_base, i, jobs.shift, &src)], 1u);
     }
-    const uint64_t m = match_digit(digit[s], valid);
-    if (valid && (m & lt) == 0) wave_hist[wave][digit[s]] += (uint32_t)__popcll(m);
   }
   __syncthreads();
 
@@ -160,7 +159,6 @@ __global__ __launch_bounds__(SORT_THREADS) void sort_scatter_kernel(ha_sort_jobs
   uint32_t base;
   if (job.chunks_per_seg > 1) {
     base = job.hist[((int64_t)br.seg * job.chunks_per_seg + br.chunk) * 256 + tid];
-    __syncthreads();
   } else {
     base = block_exclusive_scan(total, wave_totals);
   }
@@ -174,23 +172,26 @@ __global__ __launch_bounds__(SORT_THREADS) void sort_scatter_kernel(ha_sort_jobs
   }
   __syncthreads();
 
-  // pass 2: rank inside the wave step and scatter
   const int64_t out_base = (int64_t)br.seg * job.seg_len;
-#pragma unroll
+#pragma unroll 2
   for (int s = 0; s < SORT_STEPS; ++s) {
-    const bool valid = src[s] >= 0;
-    const uint64_t m = match_digit(digit[s], valid);
+    const int i = wave_start + s * HA_WAVE + lane;
+    const bool valid = i < job.seg_len;
+    int src = 0, digit = 0;
+    if (valid) digit = load_digit(job, prev, seg_base, i, jobs.shift, &src);
+    const uint64_t m = match_digit(digit, valid);
+    const uint32_t below = rank_below(m);
     if (valid) {
-      const uint32_t slot = wave_hist[wave][digit[s]] + (uint32_t)__popcll(m & lt);
+      const uint32_t slot = wave_hist[wave][digit] + below;
       if (jobs.idx64)
-        ((int64_t*)job.out)[out_base + slot] = src[s];
+        ((int64_t*)job.out)[out_base + slot] = src;
       else
-        ((int32_t*)job.out)[out_base + slot] = src[s];
+        ((int32_t*)job.out)[out_base + slot] = src;
     }
-    // all lanes of the wave have read their slot before the leaders advance it (same wave,
-    // LDS operations complete in program order)
+    // every lane of the wave has read its slot before the first lane of each digit advances it
+    // (same wave: LDS operations complete in program order)
     __builtin_amdgcn_wave_barrier();
-    if (valid && (m & lt) == 0) wave_hist[wave][digit[s]] += (uint32_t)__popcll(m);
+    if (valid && below == 0) wave_hist[wave][digit] += (uint32_t)__popcll(m);
     __builtin_amdgcn_wave_barrier();
   }
 }

@@ -2,13 +2,19 @@
 // Follows the definition in src/angular_lsh_triton.py:76-88 and :175-179 of the reference
 // (bit_j = [x . P[:, j] > 0], bin = sum_j bit_j << j, bucket = perm[bin], perm[i] = i ^ (i >> 1)).
 //
-// One thread owns one row.  A block first copies its rows from HBM into LDS with fully
-// coalesced 16-byte loads (XOR-swizzled so the per-row reads that follow are bank-conflict
-// free), then every thread walks its row and accumulates the r dot products in fp64:
-// products of fp16/bf16 values are exact in fp64, so the sign equals that of the exact dot
-// product, independent of accumulation order.  fp64 FMA runs at the same rate as unpacked fp32
-// FMA on CDNA4, so exactness costs nothing extra.  The projection matrix is converted to fp64
-// once per block and read from LDS as wave-wide broadcasts.
+// Two kernels.
+//
+// lsh_hash_mfma_kernel (head dims that are multiples of 32): a wave projects 16 rows at a time with
+// v_mfma_f32_16x16x32 (rows x 16 projection slots, fp32 accumulation), reading the rows straight from
+// HBM as MFMA operands, so the kernel is purely bandwidth bound.  fp32 accumulation cannot decide the
+// sign of a projection that nearly cancels, so a second MFMA on |x| and |P| gives sum |x_k P_kj|, which
+// bounds the accumulation error of any summation order (d * 2^-23 * sum, used with a factor 2 margin;
+// fp16/bf16 products are exact in fp32 and subnormal inputs are not flushed).  Whenever some
+// |projection| is inside that bound, the 16-row tile is recomputed in fp64 (products exact, sum exact
+// to 2^-53), which happens for well under 1 % of the tiles on random data.
+//
+// lsh_hash_kernel (any head dim that is a multiple of 8): one thread per row, rows staged through
+// LDS with coalesced 16-byte loads, all projections accumulated in fp64.
 #include "ha_common.h"
 
 namespace {
@@ -72,6 +78,164 @@ __global__ void lsh_hash_kernel(const T* __restrict__ x, const T* __restrict__ p
 }
 
 template <typename T>
+struct HashMfma;
+template <>
+struct HashMfma<f16_t> {
+  static __device__ __forceinline__ f32x4 run(f16x8 a, f16x8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+  }
+};
+template <>
+struct HashMfma<bf16_t> {
+  static __device__ __forceinline__ f32x4 run(bf16x8 a, bf16x8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+  }
+};
+
+constexpr int HASH_TILES_PER_WAVE = 32;  // tiles of 512 elements (16 MFMA rows of 32 elements)
+constexpr int HASH_UNROLL = 8;           // tiles in flight per wave
+
+// A data row of D elements is cut into PARTS = D/32 MFMA rows of 32 elements, so that one load
+// instruction of the wave (16 bytes per lane) covers whole rows: 16/PARTS data rows of D*2 bytes.
+// MFMA row m = (data row)*PARTS + part; lane (m = lane%16, kg = lane/16) holds elements
+// part*32 + 8*kg .. +7 of its data row.  The C registers i = 0..3 of a lane are MFMA rows 4*kg + i
+// of projection slot lane%16; the partial projections of one data row are summed afterwards.
+template <typename T, int D>
+__global__ __launch_bounds__(256) void lsh_hash_mfma_kernel(const T* __restrict__ x, const T* __restrict__ proj,
+                                                            int32_t* __restrict__ buckets, int heads, int64_t n, int r,
+                                                            int64_t sb, int64_t sh, int64_t sn, int64_t psb,
+                                                            int64_t psh) {
+  typedef typename ElemTraits<T>::vec8 vec8;
+  constexpr int PARTS = D / 32;
+  constexpr int ROWS = 16 / PARTS;            // data rows per tile
+  constexpr int NS = PARTS >= 4 ? 1 : 4 / PARTS;  // data rows per lane (sums of C registers)
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int bh = blockIdx.y;
+  const int b = bh / heads, h = bh % heads;
+  const T* xbase = x + b * sb + h * sh;
+  const T* pbase = proj + b * psb + h * psh;
+  int32_t* obase = buckets + (int64_t)bh * n;
+  const int m = lane & 15, kg = lane >> 4;
+  const int my_row = m / PARTS, my_part = m % PARTS;  // data row inside a tile, 32-element part of it
+  const int j = m;                                    // projection slot of this lane's C registers
+
+  // the projection matrix goes through LDS once per block (one coalesced pass instead of a chain of
+  // dependent 2-byte loads per lane)
+  __shared__ T lds_p[D * 16];
+  for (int i = threadIdx.x; i < D * r; i += blockDim.x) lds_p[i] = pbase[i];
+  __syncthreads();
+  // B operands: P and |P| for every part: slot j, group kg holds P[part*32 + 8*kg + e][j]; slots >= r are zero
+  vec8 pf[PARTS], pa[PARTS];
+  const int jc = j < r ? j : 0;
+#pragma unroll
+  for (int pt = 0; pt < PARTS; ++pt)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float v = j < r ? ha_to_float(lds_p[(pt * 32 + 8 * kg + e) * r + jc]) : 0.f;
+      pf[pt][e] = (T)v;
+      pa[pt][e] = (T)__builtin_fabsf(v);
+    }
+  const float tol = (float)(D + 8) * 4.76837158203125e-07f;  // 2 * (d + 8) * 2^-23
+
+  // A row's parts meet different B operands, but an MFMA has one B operand per lane column, not per
+  // row: so the tile is multiplied once per part with the rows of the other parts zeroed.  (For
+  // PARTS == 1 this is a single MFMA.)
+  const int64_t wave_row0 = ((int64_t)blockIdx.x * 4 + wave) * HASH_TILES_PER_WAVE * ROWS;
+  for (int t0 = 0; t0 < HASH_TILES_PER_WAVE; t0 += HASH_UNROLL) {
+    if (wave_row0 + (int64_t)t0 * ROWS >= n) break;
+    vec8 xf[HASH_UNROLL];
+#pragma unroll
+    for (int u = 0; u < HASH_UNROLL; ++u) {
+      const int64_t row = wave_row0 + (int64_t)(t0 + u) * ROWS + my_row;
+      vec8 z = {};
+      if (row < n) z = *reinterpret_cast<const vec8*>(xbase + row * sn + my_part * 32 + 8 * kg);
+      xf[u] = z;
+    }
+#pragma unroll
+    for (int u = 0; u < HASH_UNROLL; ++u) {
+      const int64_t tile_row0 = wave_row0 + (int64_t)(t0 + u) * ROWS;
+      if (tile_row0 >= n) break;
+      f32x4 c = {0.f, 0.f, 0.f, 0.f}, ca = {0.f, 0.f, 0.f, 0.f};
+      const u32x4 raw = __builtin_bit_cast(u32x4, xf[u]);
+#pragma unroll
+      for (int pt = 0; pt < PARTS; ++pt) {
+        const u32x4 sel = (PARTS == 1 || my_part == pt) ? raw : u32x4{0u, 0u, 0u, 0u};
+        c = HashMfma<T>::run(__builtin_bit_cast(vec8, sel), pf[pt], c);
+        ca = HashMfma<T>::run(__builtin_bit_cast(vec8, sel & 0x7fff7fffu), pa[pt], ca);
+      }
+      // sum the parts of each data row: C register i of this lane is MFMA row 4*kg + i
+      float s[NS], sa[NS];
+      if (PARTS <= 4) {
+#pragma unroll
+        for (int q = 0; q < NS; ++q) {
+          s[q] = 0.f;
+          sa[q] = 0.f;
+#pragma unroll
+          for (int i = 0; i < 4 / NS; ++i) {
+            s[q] += c[q * (4 / NS) + i];
+            sa[q] += ca[q * (4 / NS) + i];
+          }
+        }
+      } else {  // PARTS == 8: a data row spans the C registers of lanes kg and kg^1
+        s[0] = c[0] + c[1] + c[2] + c[3];
+        sa[0] = ca[0] + ca[1] + ca[2] + ca[3];
+        s[0] += __shfl_xor(s[0], 16);
+        sa[0] += __shfl_xor(sa[0], 16);
+      }
+      uint64_t pos[NS];
+      bool unsure = false;
+#pragma unroll
+      for (int q = 0; q < NS; ++q) {
+        pos[q] = __ballot(s[q] > 0.f);
+        unsure = unsure || (j < r && __builtin_fabsf(s[q]) <= tol * sa[q]);
+      }
+      int bin;
+      if (__any(unsure)) {
+        // exact recomputation of the tile in fp64: this lane's 8 elements, then a sum over the lanes
+        // that share the data row (parts: lane bits 0..log2(PARTS)-1, groups kg: lane bits 4, 5)
+        const int64_t row = tile_row0 + my_row;
+        bin = 0;
+        for (int jj = 0; jj < r; ++jj) {
+          double part = 0.0;
+          if (row < n)
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+              part = __builtin_fma((double)ha_to_float(xf[u][e]),
+                                   (double)ha_to_float(lds_p[(my_part * 32 + 8 * kg + e) * r + jj]), part);
+          for (int off = 1; off < PARTS; off <<= 1) part += __shfl_xor(part, off);
+          part += __shfl_xor(part, 16);
+          part += __shfl_xor(part, 32);
+          bin |= (part > 0.0 ? 1 : 0) << jj;
+        }
+        // every lane of a data row now holds its bin; lane L < ROWS must hold the bin of row L
+        bin = __shfl(bin, (lane % ROWS) * PARTS);
+      } else {
+        // data row L of the tile sits in sum q = L % NS of the lanes with kg = L / NS (PARTS <= 4),
+        // or in the lanes with kg = 2*L (PARTS == 8); its bits are 16 consecutive ballot bits
+        const int L = lane % ROWS;
+        const int q = PARTS <= 4 ? L % NS : 0;
+        const int g = PARTS <= 4 ? L / NS : 2 * L;
+        uint64_t sel = pos[0];
+#pragma unroll
+        for (int qq = 1; qq < NS; ++qq) sel = q == qq ? pos[qq] : sel;
+        bin = (int)((sel >> (16 * g)) & ((1u << r) - 1u));
+      }
+      if (lane < ROWS && tile_row0 + lane < n) obase[tile_row0 + lane] = bin ^ (bin >> 1);
+    }
+  }
+}
+
+template <typename T, int D>
+int launch_hash_mfma(const void* x, const void* proj, int32_t* buckets, int64_t batch, int64_t heads, int64_t n,
+                     int64_t r, int64_t sb, int64_t sh, int64_t sn, int64_t psb, int64_t psh, hipStream_t stream) {
+  const int64_t rows_per_block = 4 * HASH_TILES_PER_WAVE * (16 / (D / 32));
+  dim3 grid((unsigned)((n + rows_per_block - 1) / rows_per_block), (unsigned)(batch * heads));
+  hipLaunchKernelGGL((lsh_hash_mfma_kernel<T, D>), grid, dim3(256), 0, stream, (const T*)x, (const T*)proj, buckets,
+                     (int)heads, n, (int)r, sb, sh, sn, psb, psh);
+  return ha_launch_status("ha_lsh_hash");
+}
+
+template <typename T>
 int launch_hash(const void* x, const void* proj, int32_t* buckets, int64_t batch, int64_t heads,
                 int64_t n, int64_t d, int64_t r, int64_t sb, int64_t sh, int64_t sn, int64_t psb,
                 int64_t psh, hipStream_t stream) {
@@ -104,6 +268,16 @@ extern "C" int ha_lsh_hash(const void* x, const void* proj, int32_t* buckets, in
   HA_REQUIRE(x_stride_n % 8 == 0 && x_stride_h % 8 == 0 && x_stride_b % 8 == 0 && ((uintptr_t)x % 16) == 0,
              HA_ERR_SHAPE, "ha_lsh_hash: rows must be 16-byte aligned");
   hipStream_t s = (hipStream_t)stream;
+#define HA_HASH_MFMA(DD)                                                                                             \
+  if (d == DD) {                                                                                                     \
+    if (dtype == HA_F16)                                                                                             \
+      return launch_hash_mfma<f16_t, DD>(x, proj, buckets, batch, heads, n, r, x_stride_b, x_stride_h, x_stride_n,   \
+                                         proj_stride_b, proj_stride_h, s);                                           \
+    return launch_hash_mfma<bf16_t, DD>(x, proj, buckets, batch, heads, n, r, x_stride_b, x_stride_h, x_stride_n,    \
+                                        proj_stride_b, proj_stride_h, s);                                            \
+  }
+  HA_HASH_MFMA(32) HA_HASH_MFMA(64) HA_HASH_MFMA(128) HA_HASH_MFMA(256)
+#undef HA_HASH_MFMA
   if (dtype == HA_F16)
     return launch_hash<f16_t>(x, proj, buckets, batch, heads, n, d, r, x_stride_b, x_stride_h, x_stride_n,
                               proj_stride_b, proj_stride_h, s);
