@@ -120,6 +120,9 @@ def main():
     ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-exact", action="store_true", help="skip timing the exact flash kernel at the same shape")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run three plain device copies of Q (a kernel of known traffic, to scale HBM byte "
+                         "counters collected with rocprofv3 --pmc)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; the path shards by (batch, head) with no communication, "
@@ -156,6 +159,13 @@ def main():
         return ops.hyper_forward(q, k, v, m.lsh.proj_dir, scale=scale, causal=w["causal"], lsh_num_projs=8,
                                  block_size=w["block"], sample_size=w["sample"], min_seq_len=w["min_seq_len"],
                                  smooth_block=w["smooth"])
+
+    if args.calibrate_copy:
+        dst = torch.empty_like(q)
+        for _ in range(3):
+            dst.copy_(q)
+        torch.cuda.synchronize()
+        del dst
 
     for _ in range(args.warmup):
         step()

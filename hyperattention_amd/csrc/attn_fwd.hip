@@ -312,23 +312,45 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
   const int my_pp = lane % PR;           // physical piece of this lane's LDS slot
   const int my_lr = lane / PR;           // row inside one load
 
-  // original row of key r of chunk ci; chunks past the end and rows past n_k alias row 0 (their
-  // scores are masked or never used, and row 0 holds finite data)
-  auto key_row = [&](int ci, int r) -> int {
-    if (ci >= n_chunks) return 0;
+  // Original rows of the keys of chunk ci.  The source of a chunk is wave-uniform: either a run of an
+  // index array (sorted keys of the block part, or an explicit sample list) or 64 consecutive rows
+  // (default samples, exact attention).  Index arrays are read as 4-byte words at a stride of 4 or 8
+  // bytes (row numbers fit the low word of an int64).  Rows past n_k alias row 0: their scores are
+  // masked and row 0 holds finite data; chunks past the end are never loaded.
+  const int idx_shift = p.idx64 ? 3 : 2;
+  auto fetch_rows = [&](int ci, int (&rows)[LPW]) {
+    const unsigned char* src = nullptr;  // index array run, or null for consecutive rows
+    int64_t stride = 0;
+    int first = 0;
     if (GATHER) {
       if (ci < n_blk_chunks) {
-        const int pos = ((uni_start + ci) % nk_chunks) * KC + r;
-        return ha_load_idx(p.k_idx, kidx_off + (int64_t)pos * p.ki_sn, p.idx64);
+        int u = uni_start + ci;  // smooth windows wrap around the key sequence
+        u -= u >= nk_chunks ? nk_chunks : 0;
+        u -= u >= nk_chunks ? nk_chunks : 0;
+        src = (const unsigned char*)p.k_idx + ((kidx_off + (int64_t)u * KC * p.ki_sn) << idx_shift);
+        stride = p.ki_sn << idx_shift;
+      } else {
+        first = (ci - n_blk_chunks) * KC;
+        if (p.sampled_idx) {
+          src = (const unsigned char*)p.sampled_idx + ((sidx_off + first) << idx_shift);
+          stride = (int64_t)1 << idx_shift;
+        }
       }
-      const int s = (ci - n_blk_chunks) * KC + r;
-      return p.sampled_idx ? ha_load_idx(p.sampled_idx, sidx_off + s, p.idx64) : s;
+    } else {
+      first = ci * KC;
     }
-    const int row = ci * KC + r;
-    return row < p.n_k ? row : 0;
+#pragma unroll
+    for (int j = 0; j < LPW; ++j) {
+      const int r = (wave * LPW + j) * ROWS_PER_LOAD + my_lr;
+      if (src) {
+        rows[j] = ci < n_chunks ? *reinterpret_cast<const int*>(src + r * stride) : 0;
+      } else {
+        const int row = first + r;
+        rows[j] = (GATHER || row < p.n_k) ? row : 0;
+      }
+    }
   };
-#define HA_FETCH_ROWS(ci, rows) \
-  _Pragma("unroll") for (int j = 0; j < LPW; ++j) rows[j] = key_row((ci), (wave * LPW + j) * ROWS_PER_LOAD + my_lr);
+#define HA_FETCH_ROWS(ci, rows) fetch_rows((ci), rows);
 #define HA_LOAD_TILE(base, stride, rows, tile)                                                           \
   _Pragma("unroll") for (int j = 0; j < LPW; ++j) {                                                      \
     const int r = (wave * LPW + j) * ROWS_PER_LOAD + my_lr;                                              \

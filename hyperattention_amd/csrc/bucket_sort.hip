@@ -126,10 +126,14 @@ __global__ __launch_bounds__(SORT_THREADS) void sort_scan_kernel(ha_sort_jobs jo
 // ---- stable scatter --------------------------------------------------------------------------
 // A wave owns a contiguous run of the chunk (wave order = key order).  Pass 1 counts digits per wave
 // with LDS atomics; pass 2 re-reads the keys (they are cache resident) and ranks them inside each
-// 64-key step by ballot matching, which is what keeps equal keys in ascending row order.
+// 64-key step by ballot matching, which is what keeps equal keys in ascending row order.  The chunk is
+// put in order in LDS first and then written out by consecutive threads, so that the runs of equal
+// keys leave as whole cache lines instead of scattered 4-byte writes.
 __global__ __launch_bounds__(SORT_THREADS) void sort_scatter_kernel(ha_sort_jobs jobs) {
   __shared__ uint32_t wave_hist[SORT_WAVES][256];
   __shared__ uint32_t wave_totals[SORT_WAVES];
+  __shared__ int32_t to_global[256];            // global slot minus chunk-local slot, per digit
+  __shared__ uint32_t staged[HA_SORT_CHUNK];    // (digit << 24) | row, in chunk-local sorted order
   const BlockRef br = locate_block(jobs, blockIdx.x, false);
   const ha_sort_job& job = jobs.job[br.job];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
@@ -139,7 +143,9 @@ __global__ __launch_bounds__(SORT_THREADS) void sort_scatter_kernel(ha_sort_jobs
 
   const int64_t seg_base = job.seg_offset + (int64_t)br.seg * job.seg_stride;
   const int32_t* prev = job.prev ? job.prev + (int64_t)br.seg * job.seg_len : nullptr;
-  const int wave_start = br.chunk * HA_SORT_CHUNK + wave * (SORT_STEPS * HA_WAVE);
+  const int chunk_start = br.chunk * HA_SORT_CHUNK;
+  const int wave_start = chunk_start + wave * (SORT_STEPS * HA_WAVE);
+  const bool stage = job.seg_len <= (1 << 24);  // rows fit 24 bits next to the digit
 
 #pragma unroll 4
   for (int s = 0; s < SORT_STEPS; ++s) {
@@ -151,19 +157,17 @@ __global__ __launch_bounds__(SORT_THREADS) void sort_scatter_kernel(ha_sort_jobs
   }
   __syncthreads();
 
-  // first output slot of (this chunk, key tid): from the scan kernel, or computed here when the
-  // segment is a single chunk
+  // chunk-local first slot of key tid, and the global first slot of (this chunk, key tid): from the
+  // scan kernel, or equal to the local one when the segment is a single chunk
   uint32_t total = 0;
 #pragma unroll
   for (int w = 0; w < SORT_WAVES; ++w) total += wave_hist[w][tid];
-  uint32_t base;
-  if (job.chunks_per_seg > 1) {
-    base = job.hist[((int64_t)br.seg * job.chunks_per_seg + br.chunk) * 256 + tid];
-  } else {
-    base = block_exclusive_scan(total, wave_totals);
-  }
-  // turn the per-wave counts into per-wave first slots
-  uint32_t run = base;
+  const uint32_t local_base = block_exclusive_scan(total, wave_totals);
+  uint32_t global_base = local_base;
+  if (job.chunks_per_seg > 1) global_base = job.hist[((int64_t)br.seg * job.chunks_per_seg + br.chunk) * 256 + tid];
+  to_global[tid] = (int32_t)(global_base - local_base);
+  // turn the per-wave counts into per-wave chunk-local first slots
+  uint32_t run = local_base;
 #pragma unroll
   for (int w = 0; w < SORT_WAVES; ++w) {
     const uint32_t c = wave_hist[w][tid];
@@ -183,16 +187,32 @@ __global__ __launch_bounds__(SORT_THREADS) void sort_scatter_kernel(ha_sort_jobs
     const uint32_t below = rank_below(m);
     if (valid) {
       const uint32_t slot = wave_hist[wave][digit] + below;
-      if (jobs.idx64)
-        ((int64_t*)job.out)[out_base + slot] = src;
-      else
-        ((int32_t*)job.out)[out_base + slot] = src;
+      if (stage) {
+        staged[slot] = ((uint32_t)digit << 24) | (uint32_t)src;
+      } else {
+        const int64_t g = out_base + (int64_t)slot + to_global[digit];
+        if (jobs.idx64)
+          ((int64_t*)job.out)[g] = src;
+        else
+          ((int32_t*)job.out)[g] = src;
+      }
     }
     // every lane of the wave has read its slot before the first lane of each digit advances it
     // (same wave: LDS operations complete in program order)
     __builtin_amdgcn_wave_barrier();
     if (valid && below == 0) wave_hist[wave][digit] += (uint32_t)__popcll(m);
     __builtin_amdgcn_wave_barrier();
+  }
+  if (!stage) return;
+  __syncthreads();
+  const int count = min(HA_SORT_CHUNK, job.seg_len - chunk_start);
+  for (int pos = tid; pos < count; pos += SORT_THREADS) {
+    const uint32_t v = staged[pos];
+    const int64_t g = out_base + pos + to_global[v >> 24];
+    if (jobs.idx64)
+      ((int64_t*)job.out)[g] = (int64_t)(v & 0xFFFFFFu);
+    else
+      ((int32_t*)job.out)[g] = (int32_t)(v & 0xFFFFFFu);
   }
 }
 
