@@ -2,36 +2,42 @@
 // the exact (flash) kernel share one body.
 //
 // Reference semantics: _fwd_hyper_kernel (src/hyper_attn_triton.py:26-192) and _fwd_kernel with
-// bias "none" (src/flash_attn_triton.py:57-267).
+// bias "none" (src/flash_attn_triton.py:57-267); the resume-from-a-previous-partial-result mode
+// folds add_self_attentions (src/attn_utils.py:6-50) into the kernel.
 //
 // Work decomposition.  A workgroup of 4 waves owns 256 consecutive (sorted) query positions of one
-// (virtual) head; wave w owns 64 of them as two 32-wide MFMA column blocks.  Keys are streamed in
-// chunks of 64 rows straight from HBM into LDS (global_load_lds, 16 bytes per lane, no staging
-// registers), K and V both row-major with their 16-byte pieces XOR-swizzled by the row number (the
-// swizzle is applied on the source side: a lane fetches the piece that belongs in its LDS slot).
-// The K operand is read with ds_read_b128, the V^T operand with the transposing ds_read_b64_tr_b16.
+// (virtual) head; wave w owns 64 of them as two 32-wide MFMA column blocks.  Query rows and key
+// rows go from HBM straight into LDS (global_load_lds, 16 bytes per lane, whole rows per
+// instruction, no staging registers), row-major with their 16-byte pieces XOR-swizzled by the row
+// number (the swizzle is applied on the source side: a lane fetches the piece that belongs in its
+// LDS slot).  Q and K operands are read with ds_read_b128, the V^T operand with the transposing
+// ds_read_b64_tr_b16.
 //
 // MFMA formulation (v_mfma_f32_32x32x16_{f16,bf16}; A: lane -> row lane%32, k = 8*(lane/32)..+7;
 // B: lane -> column lane%32, same k; C: lane -> column lane%32, rows 8*(i/4) + 4*(lane/32) + i%4):
 //   S^T = K  Q^T   (M = keys,  N = queries, K = head dim)   -> a lane holds 16 keys of ONE query
 //   O^T = V^T P^T  (M = dv,    N = queries, K = keys)       -> P^T comes straight from the S^T registers
-// so the soft-max statistics (running max, running sum) are per-lane scalars; only one exchange
-// with lane^32 per 32 keys is needed for the row maximum.  ds_read_b64_tr_b16 gives lane i of a
-// 16-lane group element i%4 of the 8-byte words addressed by lanes 4j + i/4 (j = 0..3), so a group
-// that points its lanes at (key j, dv word w) receives V[key 0..3][dv base + i]: the V^T operand in
+// so the soft-max statistics are per-lane scalars.  ds_read_b64_tr_b16 gives lane i of a 16-lane
+// group element i%4 of the 8-byte words addressed by lanes 4j + i/4 (j = 0..3), so a group that
+// points its lanes at (key j, dv word w) receives V[key 0..3][dv base + i]: the V^T operand in
 // exactly the key order of the C registers.
 //
 // Software pipeline.  On this hardware a wave's MFMAs overlap only with vector instructions of the
-// SAME wave, so the loop is pipelined in steps of 32 keys: the straight-line block that soft-maxes
-// the S^T block of 32 keys (exp, rounding, row sums) and multiplies it into O also issues the MFMAs
-// of the NEXT 32-key S^T block, and the LDS operands of a step are fetched into registers one step
-// (K) or half a step (V) before the MFMAs that use them.  K therefore runs one chunk ahead of V in
-// LDS.  Two waves per SIMD keep the vector pipe fed (256 registers each at d = 64).
+// SAME wave, so the loop body is a chain of straight-line blocks, one per half-step of 16 keys, and
+// each block mixes three independent things: the exponentials of half-step u, the P.V MFMAs of
+// half-step u-1 and half of the S^T MFMAs of the next 32-key step.  Keys are streamed in tiles of 64
+// rows; the K tiles are shifted by 32 keys against the V tiles (K tile c holds keys 64c-32..64c+31),
+// so the K rows read during an iteration all sit in one tile, which is read in that iteration only
+// and can be refilled in the next, and the V^T operands of a half-step are fetched one block ahead.
 //
-// The soft-max runs in base 2 (scale*log2(e) folded into one FMA, v_exp_f32 is 2^x); P is rounded
-// to the input type before P.V as the reference does (src/hyper_attn_triton.py:135) and the row sums
-// are taken over the rounded values.  The running maximum is only raised when a row exceeds it by
-// more than 2^RESCALE_SLACK, which removes the accumulator rescale from almost every step.
+// Soft-max without a running maximum.  The exponentials use the current reference exponent m of
+// the row as is (base 2, scale*log2(e) folded into one FMA; v_exp_f32 is 2^x); P is rounded to the
+// input type before P.V as the reference does (src/hyper_attn_triton.py:135) and the row sums are
+// taken over the rounded values.  Only when the sum of a lane's 8 values of a half-step reaches 2^14
+// (or is not a number: nothing seen yet) is the row maximum computed, m raised, the accumulators
+// rescaled and the half-step redone; below that bound every value is finite in fp16 and the result
+// does not depend on m beyond rounding.  m only ever grows, and starts from the true maximum of the
+// first keys or from the log-sum-exp of the partial result that is being resumed.
 #include "ha_common.h"
 #include "attn_fwd.h"
 
@@ -39,10 +45,10 @@ namespace {
 
 constexpr int WG_THREADS = 256;
 constexpr int WG_QUERIES = 256;  // sorted query positions per workgroup
-constexpr int KC = 64;           // keys per LDS chunk
+constexpr int KC = 64;           // keys per LDS tile
 constexpr float LOG2E = 1.4426950408889634f;
 constexpr float LN2 = 0.6931471805599453f;
-constexpr float RESCALE_SLACK = 8.0f;  // log2 units
+constexpr float HALF_SUM_LIMIT = 16384.f;  // 2^14: a lane's half-step sum below this has no fp16 overflow
 constexpr int NUM_XCD = 8;
 
 template <typename T>
@@ -81,8 +87,8 @@ __device__ __forceinline__ int xcd_contiguous_id(int linear, int total) {
 // LDS byte offsets of one lane's operand reads, relative to a tile base (fixed for the whole kernel).
 template <int D>
 struct LaneOffsets {
-  int k[D / 16];  // K operand piece of k-step ks for key row `col` (add mb*32 rows)
-  int v[D / 32];  // V^T operand word for dv block db, keys 0..3 (+4 for the upper lane half) of a 16-key step
+  int k[D / 16];  // Q / K operand piece of k-step ks for tile row lane%32 (add 32 rows for the upper half)
+  int v[D / 32];  // V^T operand word for dv block db, keys 0..3 (+4 for the upper lane half) of a 16-key half-step
 };
 
 // 16-byte piece `piece` of row `row` of a row-major [rows][D] 2-byte tile, XOR-swizzled; byte offset
@@ -120,105 +126,122 @@ __device__ __forceinline__ void global_to_lds_16(const void* src, unsigned char*
 #endif
 }
 
-// One pipeline step over 32 keys.
-//   s_use  : S^T of the 32 keys being consumed (per query block nb), complete on entry
-//   s_fill : receives S^T of the next 32 keys, from the K operands kf (already in registers)
-//   kf     : on entry the K operands of this step's MFMAs; on exit those of the next step, read from
-//            rows mb_pref*32.. of the K tile k_pref
-//   v_tile : V tile of the chunk being consumed; khalf selects its keys 32*khalf..+31
-template <typename T, int D>
-__device__ __forceinline__ void pipeline_step(f32x16 (&s_use)[2], f32x16 (&s_fill)[2],
-                                              typename ElemTraits<T>::vec8 (&kf)[D / 16],
-                                              const unsigned char* k_pref, int mb_pref,
-                                              const unsigned char* v_tile, int khalf, const LaneOffsets<D>& lo,
-                                              const typename ElemTraits<T>::vec8 (&qf)[2][D / 16],
-                                              f32x16 (&acc)[D / 32][2], float (&m_run)[2], float (&l_run)[2],
-                                              float scale_log2) {
-  typedef typename ElemTraits<T>::vec8 vec8;
+// P of the 8 values of half-step H a lane holds per query block (elements 8H..8H+7 of its S^T
+// registers), rounded to T, and their sums.  m is the reference exponent (log2 units).
+template <typename T, int H>
+__device__ __forceinline__ void half_step_p(const f32x16 (&s_use)[2], const float (&m)[2], float scale_log2,
+                                            typename ElemTraits<T>::vec8 (&pn)[2], float (&sum)[2]) {
   typedef typename ElemTraits<T>::vec2 vec2;
-  constexpr int KSTEPS = D / 16;
-  constexpr int DB = D / 32;
-
-  // operands for later: V^T of this step's first 16 keys, K of the next step
-  vec8 vf[DB];
 #pragma unroll
-  for (int db = 0; db < DB; ++db) vf[db] = lds_read_vt<T>(v_tile, lo.v[db] + khalf * 32 * D * 2, D * 2);
-  vec8 kf_next[KSTEPS];
+  for (int nb = 0; nb < 2; ++nb) {
+    float acc_sum = 0.f;
 #pragma unroll
-  for (int ks = 0; ks < KSTEPS; ++ks) kf_next[ks] = lds_read_k<T>(k_pref, lo.k[ks] + mb_pref * 32 * D * 2);
+    for (int e = 0; e < 8; e += 2) {
+      const int i = H * 8 + e;
+      vec2 pp;
+      pp[0] = (T)__builtin_amdgcn_exp2f(__builtin_fmaf(s_use[nb][i], scale_log2, -m[nb]));
+      pp[1] = (T)__builtin_amdgcn_exp2f(__builtin_fmaf(s_use[nb][i + 1], scale_log2, -m[nb]));
+      acc_sum = Mfma<T>::pair_sum(pp, acc_sum);
+      pn[nb][e] = pp[0];
+      pn[nb][e + 1] = pp[1];
+    }
+    sum[nb] = acc_sum;
+  }
+}
 
-  // row maxima of the 32 keys; raise the reference maximum only when needed (wave-uniform branch)
-  float mx[2];
-  bool grow = false;
+// The rare path of a half-step: raise the reference exponents to the row maxima of the step, rescale
+// the row sums and redo the half-step's P.  The accumulators hold everything up to the previous
+// half-step (its P.V was issued in this block); they are rescaled by alpha_pend at the start of the
+// next block, before the P.V of this half-step is added.
+template <typename T, int D, int H>
+__device__ __forceinline__ void half_step_rescale(const f32x16 (&s_use)[2], float scale_log2,
+                                                  float (&alpha_pend)[2], float (&m_run)[2], float (&l_run)[2],
+                                                  typename ElemTraits<T>::vec8 (&pn)[2], float (&sum)[2]) {
+  float m_use[2];
 #pragma unroll
   for (int nb = 0; nb < 2; ++nb) {
     float v = s_use[nb][0];
 #pragma unroll
     for (int i = 1; i < 16; ++i) v = fmaxf(v, s_use[nb][i]);
     v = fmaxf(v, __shfl_xor(v, 32)) * scale_log2;
-    mx[nb] = v;
-    grow = grow || (v > m_run[nb] + RESCALE_SLACK);
+    const float m_new = fmaxf(m_run[nb], v);
+    // nothing accumulated yet under m_run = -inf; otherwise 2^(old - new) <= 1
+    const float alpha = m_run[nb] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m_run[nb] - m_new);
+    m_run[nb] = m_new;
+    l_run[nb] *= alpha;
+    alpha_pend[nb] = alpha;
+    // rows that have seen no key yet (all masked) keep m_run = -inf; their P is 2^(-inf - 0) = 0
+    m_use[nb] = m_new == -INFINITY ? 0.f : m_new;
   }
-  if (__any(grow)) {
-#pragma unroll
-    for (int nb = 0; nb < 2; ++nb) {
-      const float m_new = fmaxf(m_run[nb], mx[nb]);
-      const float alpha = __builtin_amdgcn_exp2f(m_run[nb] - m_new);
-      m_run[nb] = m_new;
-      l_run[nb] *= alpha;
-#pragma unroll
-      for (int db = 0; db < DB; ++db)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) acc[db][nb][i] *= alpha;
-    }
-  }
+  half_step_p<T, H>(s_use, m_use, scale_log2, pn, sum);
+}
 
-  // ---- straight-line block: next S^T MFMAs | exp, round, row sums | P V MFMAs ---------------------
-#pragma unroll
-  for (int nb = 0; nb < 2; ++nb)
-#pragma unroll
-    for (int i = 0; i < 16; ++i) s_fill[nb][i] = 0.f;
-#pragma unroll
-  for (int ks = 0; ks < KSTEPS; ++ks)
-#pragma unroll
-    for (int nb = 0; nb < 2; ++nb) s_fill[nb] = Mfma<T>::run(kf[ks], qf[nb][ks], s_fill[nb]);
+// One block of the pipeline: half-step H (16 keys) of the 32-key step whose S^T is s_use.
+//   MFMAs : P.V of the previous half-step (operands vf, pb, both in registers) and this half's share
+//           (k-steps H*KSTEPS/2 ..) of the next step's S^T, K rows k_row_off.. of k_tile
+//   VALU  : P of this half-step from s_use -> pb (for the next block) and the row sums
+//   LDS   : V^T of this half-step's keys (v_key_off.. of v_tile) -> vf (for the next block)
+// rescale_pend (wave-uniform) / alpha_pend: accumulator rescale left over by the previous block
+template <typename T, int D, int H>
+__device__ __forceinline__ void half_step(const f32x16 (&s_use)[2], f32x16 (&s_fill)[2],
+                                          const unsigned char* k_tile, int k_row_off,
+                                          const unsigned char* v_tile, int v_key_off, const LaneOffsets<D>& lo,
+                                          const typename ElemTraits<T>::vec8 (&qf)[2][D / 16],
+                                          f32x16 (&acc)[D / 32][2], float (&m_run)[2], float (&l_run)[2],
+                                          typename ElemTraits<T>::vec8 (&pb)[2],
+                                          typename ElemTraits<T>::vec8 (&vf)[D / 32], float scale_log2,
+                                          float (&alpha_pend)[2], bool& rescale_pend) {
+  typedef typename ElemTraits<T>::vec8 vec8;
+  constexpr int KH = D / 32;  // k-steps of this half
+  constexpr int DB = D / 32;
 
-#pragma unroll
-  for (int ks2 = 0; ks2 < 2; ++ks2) {
-    vec8 pb[2];
-#pragma unroll
-    for (int nb = 0; nb < 2; ++nb) {
-      // rows that have seen no key yet (every key so far masked) keep m_run = -inf: use 0 there
-      const float m_use = m_run[nb] == -INFINITY ? 0.f : m_run[nb];
-      float sum = l_run[nb];
-#pragma unroll
-      for (int e = 0; e < 8; e += 2) {
-        const int i = ks2 * 8 + e;
-        vec2 pp;
-        pp[0] = (T)__builtin_amdgcn_exp2f(__builtin_fmaf(s_use[nb][i], scale_log2, -m_use));
-        pp[1] = (T)__builtin_amdgcn_exp2f(__builtin_fmaf(s_use[nb][i + 1], scale_log2, -m_use));
-        sum = Mfma<T>::pair_sum(pp, sum);
-        pb[nb][e] = pp[0];
-        pb[nb][e + 1] = pp[1];
-      }
-      l_run[nb] = sum;
-    }
-    vec8 vf2[DB];
-    if (ks2 == 0) {
-#pragma unroll
-      for (int db = 0; db < DB; ++db) vf2[db] = lds_read_vt<T>(v_tile, lo.v[db] + (khalf * 32 + 16) * D * 2, D * 2);
-    }
+  if (rescale_pend) {
 #pragma unroll
     for (int db = 0; db < DB; ++db)
 #pragma unroll
-      for (int nb = 0; nb < 2; ++nb) acc[db][nb] = Mfma<T>::run(vf[db], pb[nb], acc[db][nb]);
-    if (ks2 == 0) {
+      for (int nb = 0; nb < 2; ++nb)
 #pragma unroll
-      for (int db = 0; db < DB; ++db) vf[db] = vf2[db];
-    }
+        for (int i = 0; i < 16; ++i) acc[db][nb][i] *= alpha_pend[nb];
+    rescale_pend = false;
+  }
+  vec8 kf[KH];
+#pragma unroll
+  for (int k2 = 0; k2 < KH; ++k2) kf[k2] = lds_read_k<T>(k_tile, lo.k[H * KH + k2] + k_row_off);
+  vec8 vf_next[DB];
+#pragma unroll
+  for (int db = 0; db < DB; ++db) vf_next[db] = lds_read_vt<T>(v_tile, lo.v[db] + v_key_off, D * 2);
+
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+#pragma unroll
+    for (int nb = 0; nb < 2; ++nb) acc[db][nb] = Mfma<T>::run(vf[db], pb[nb], acc[db][nb]);
+  if (H == 0) {
+#pragma unroll
+    for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) s_fill[nb][i] = 0.f;
   }
 #pragma unroll
-  for (int ks = 0; ks < KSTEPS; ++ks) kf[ks] = kf_next[ks];
+  for (int k2 = 0; k2 < KH; ++k2)
+#pragma unroll
+    for (int nb = 0; nb < 2; ++nb) s_fill[nb] = Mfma<T>::run(kf[k2], qf[nb][H * KH + k2], s_fill[nb]);
+
+  vec8 pn[2];
+  float sum[2];
+  half_step_p<T, H>(s_use, m_run, scale_log2, pn, sum);
+  // not "sum >= limit": a NaN (row that has seen nothing yet) must take the rare path too
+  const bool redo = !(sum[0] < HALF_SUM_LIMIT) || !(sum[1] < HALF_SUM_LIMIT);
+  if (__any(redo)) {
+    half_step_rescale<T, D, H>(s_use, scale_log2, alpha_pend, m_run, l_run, pn, sum);
+    rescale_pend = true;
+  }
+#pragma unroll
+  for (int nb = 0; nb < 2; ++nb) {
+    l_run[nb] += sum[nb];
+    pb[nb] = pn[nb];
+  }
+#pragma unroll
+  for (int db = 0; db < DB; ++db) vf[db] = vf_next[db];
 }
 
 }  // namespace
@@ -227,19 +250,22 @@ template <typename T, int D, bool GATHER, bool CAUSAL>
 __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_kernel(const ha_attn_kernel_params p) {
   typedef typename ElemTraits<T>::vec8 vec8;
   typedef typename ElemTraits<T>::vec4 vec4;
-  typedef typename ElemTraits<T>::vec2 vec2;
   constexpr int DV = D;
   constexpr int KSTEPS = D / 16;  // MFMA k-steps of Q.K^T
   constexpr int DB = DV / 32;     // 32-row blocks of O^T
-  constexpr int PR = D / 8;       // 16-byte pieces per K (and V) row
+  constexpr int PR = D / 8;       // 16-byte pieces per row
 
-  // Four separate LDS objects (two K tiles, two V tiles of KC rows): the compiler then knows that a
-  // tile being filled from HBM and a tile being read do not alias, and does not serialise them.
+  // Separate LDS objects (two K tiles, two V tiles of KC rows, the query rows): the compiler then
+  // knows that a tile being filled from HBM and a tile being read do not alias, and does not
+  // serialise them.  The query region (one tile per wave) is reused for the output rows at the end.
   constexpr int TILE_BYTES = KC * D * 2;
   __shared__ __attribute__((aligned(16))) unsigned char lds_k0[TILE_BYTES];
   __shared__ __attribute__((aligned(16))) unsigned char lds_k1[TILE_BYTES];
   __shared__ __attribute__((aligned(16))) unsigned char lds_v0[TILE_BYTES];
   __shared__ __attribute__((aligned(16))) unsigned char lds_v1[TILE_BYTES];
+  __shared__ __attribute__((aligned(16))) unsigned char lds_q[4 * TILE_BYTES];
+  __shared__ int lds_qrow[WG_QUERIES];   // original row of every query position (-1: past the end)
+  __shared__ float lds_w[WG_QUERIES];    // weight of the resumed partial result per query position
 
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63;
@@ -301,24 +327,26 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
   }
   const int wave_q_first = qt * WG_QUERIES + wave * 64;
 
-  // ---- tiles: HBM -> LDS without passing through registers ----------------------------------------
+  // ---- rows: HBM -> LDS without passing through registers -----------------------------------------
   // One global_load_lds moves 16 bytes per lane to 1 KB of consecutive LDS: 64/PR rows of a tile.
-  // Wave w issues loads LPW*w .. LPW*w + LPW-1 of a tile.  A lane's LDS slot is (row, physical piece
-  // lane % PR); it fetches the logical piece that the swizzle puts there.  Original row numbers are
-  // fetched one chunk ahead of the rows, so a row load never waits for an index load.
+  // Wave w issues loads LPW*w .. LPW*w + LPW-1 of a key tile and all PR loads of its own query tile.
+  // A lane's LDS slot is (row, physical piece lane % PR); it fetches the logical piece that the
+  // swizzle puts there.  Original row numbers are fetched one tile ahead of the rows, so a row load
+  // never waits for an index load.
   constexpr int ROWS_PER_LOAD = 64 / PR;
-  constexpr int LPW = PR / 4;  // loads per wave per tile
-  int rows_k[LPW], rows_v[LPW];
-  const int my_pp = lane % PR;           // physical piece of this lane's LDS slot
-  const int my_lr = lane / PR;           // row inside one load
+  constexpr int LPW = PR / 4;  // loads per wave per key tile
+  const int my_pp = lane % PR;  // physical piece of this lane's LDS slot
+  const int my_lr = lane / PR;  // row inside one load
 
-  // Original rows of the keys of chunk ci.  The source of a chunk is wave-uniform: either a run of an
-  // index array (sorted keys of the block part, or an explicit sample list) or 64 consecutive rows
-  // (default samples, exact attention).  Index arrays are read as 4-byte words at a stride of 4 or 8
-  // bytes (row numbers fit the low word of an int64).  Rows past n_k alias row 0: their scores are
-  // masked and row 0 holds finite data; chunks past the end are never loaded.
+  // Original rows of keys kk0 + j*ROWS_PER_LOAD + my_lr (j < LPW) of chunk ci.  The source of a chunk
+  // is wave-uniform: either a run of an index array (sorted keys of the block part, or an explicit
+  // sample list) or consecutive rows (default samples, exact attention).  Index arrays are read as
+  // 4-byte words at a stride of 4 or 8 bytes (row numbers fit the low word of an int64).  Keys past
+  // n_k and chunks outside 0..n_chunks-1 alias row 0: row 0 holds finite data and their scores are
+  // masked or never used.  Every branch is wave-uniform and nothing touches a loaded value here: the
+  // loads stay in flight until the row numbers are needed for the tile loads of a later iteration.
   const int idx_shift = p.idx64 ? 3 : 2;
-  auto fetch_rows = [&](int ci, int (&rows)[LPW]) {
+  auto fetch_rows = [&](int ci, int kk0, int (&rows)[LPW]) {
     const unsigned char* src = nullptr;  // index array run, or null for consecutive rows
     int64_t stride = 0;
     int first = 0;
@@ -339,18 +367,28 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
     } else {
       first = ci * KC;
     }
+    if (ci < 0 || ci >= n_chunks) {
 #pragma unroll
-    for (int j = 0; j < LPW; ++j) {
-      const int r = (wave * LPW + j) * ROWS_PER_LOAD + my_lr;
-      if (src) {
-        rows[j] = ci < n_chunks ? *reinterpret_cast<const int*>(src + r * stride) : 0;
-      } else {
-        const int row = first + r;
+      for (int j = 0; j < LPW; ++j) rows[j] = 0;
+    } else if (src) {
+#pragma unroll
+      for (int j = 0; j < LPW; ++j)
+        rows[j] = *reinterpret_cast<const int*>(src + (kk0 + j * ROWS_PER_LOAD + my_lr) * stride);
+    } else {
+#pragma unroll
+      for (int j = 0; j < LPW; ++j) {
+        const int row = first + kk0 + j * ROWS_PER_LOAD + my_lr;
         rows[j] = (GATHER || row < p.n_k) ? row : 0;
       }
     }
   };
-#define HA_FETCH_ROWS(ci, rows) fetch_rows((ci), rows);
+  // V tile c holds keys 0..63 of chunk c.  K tile c holds keys 32..63 of chunk c-1 in its rows 0..31
+  // and keys 0..31 of chunk c in its rows 32..63: waves 0,1 load the former, waves 2,3 the latter.
+  const int v_kk0 = wave * (LPW * ROWS_PER_LOAD);
+  const int k_kk0 = (v_kk0 + 32) & 63;
+  const int k_chunk_shift = (wave >> 1) - 1;
+#define HA_FETCH_ROWS_K(tile_c, rows) fetch_rows((tile_c) + k_chunk_shift, k_kk0, rows);
+#define HA_FETCH_ROWS_V(ci, rows) fetch_rows((ci), v_kk0, rows);
 #define HA_LOAD_TILE(base, stride, rows, tile)                                                           \
   _Pragma("unroll") for (int j = 0; j < LPW; ++j) {                                                      \
     const int r = (wave * LPW + j) * ROWS_PER_LOAD + my_lr;                                              \
@@ -358,37 +396,46 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
     global_to_lds_16(src, (tile) + (wave * LPW + j) * 1024);                                             \
   }
 
-  // first loads: indices of the queries and of the first key chunks, then the rows themselves
-  int qrow[2];
-#pragma unroll
-  for (int nb = 0; nb < 2; ++nb) {
-    const int pq = qt * WG_QUERIES + wave * 64 + nb * 32 + col;
-    qrow[nb] = pq >= p.n_q ? -1 : (GATHER ? ha_load_idx(p.q_idx, qidx_off + (int64_t)pq * p.qi_sn, p.idx64) : pq);
-  }
+  // ---- first loads: row numbers of the queries and of the first key tiles, then the rows ----------
+  unsigned char* const my_q = lds_q + wave * TILE_BYTES;
+  int rows_k[LPW], rows_v[LPW];
+  int qrow[2];  // original row of the query a lane's S^T / O^T columns belong to
   {
+    int q_rows[PR];  // rows of this wave's query tile, in the order of its PR loads
+#pragma unroll
+    for (int j = 0; j < PR; ++j) {
+      const int pq = wave_q_first + j * ROWS_PER_LOAD + my_lr;
+      q_rows[j] = pq >= p.n_q ? -1 : (GATHER ? ha_load_idx(p.q_idx, qidx_off + (int64_t)pq * p.qi_sn, p.idx64) : pq);
+    }
+#pragma unroll
+    for (int nb = 0; nb < 2; ++nb) {
+      const int pq = wave_q_first + nb * 32 + col;
+      qrow[nb] = pq >= p.n_q ? -1 : (GATHER ? ha_load_idx(p.q_idx, qidx_off + (int64_t)pq * p.qi_sn, p.idx64) : pq);
+    }
     int rows_k1[LPW];
-    HA_FETCH_ROWS(0, rows_k)
-    HA_FETCH_ROWS(0, rows_v)
-    HA_FETCH_ROWS(1, rows_k1)
+    HA_FETCH_ROWS_K(0, rows_k)
+    HA_FETCH_ROWS_V(0, rows_v)
+    HA_FETCH_ROWS_K(1, rows_k1)
     HA_LOAD_TILE(kb, p.k_sn, rows_k, lds_k0)
+#pragma unroll
+    for (int j = 0; j < PR; ++j) {
+      // positions past the end read row 0 (finite data; their results are never written)
+      const int r = j * ROWS_PER_LOAD + my_lr;
+      const T* src = qb + (int64_t)(q_rows[j] < 0 ? 0 : q_rows[j]) * p.q_sn + ((my_pp ^ (r & 7)) << 3);
+      global_to_lds_16(src, my_q + j * 1024);
+      if (my_pp == 0) lds_qrow[wave * 64 + r] = q_rows[j];
+    }
     HA_LOAD_TILE(vb, p.v_sn, rows_v, lds_v0)
     HA_LOAD_TILE(kb, p.k_sn, rows_k1, lds_k1)
   }
-  HA_FETCH_ROWS(2, rows_k)
-  HA_FETCH_ROWS(1, rows_v)
+  HA_FETCH_ROWS_K(2, rows_k)
+  HA_FETCH_ROWS_V(1, rows_v)
 
-  // ---- Q fragments (B operand), soft-max state, accumulators ------------------------------------
-  vec8 qf[2][KSTEPS];
-  float m_run[2], l_run[2];
+  // ---- soft-max state, accumulators ----------------------------------------------------------------
+  float m_run[2], l_run[2], m_init[2];
   f32x16 acc[DB][2];
 #pragma unroll
   for (int nb = 0; nb < 2; ++nb) {
-#pragma unroll
-    for (int ks = 0; ks < KSTEPS; ++ks) {
-      vec8 z = {};
-      if (qrow[nb] >= 0) z = *reinterpret_cast<const vec8*>(qb + (int64_t)qrow[nb] * p.q_sn + ks * 16 + hi * 8);
-      qf[nb][ks] = z;
-    }
     m_run[nb] = -INFINITY;
     l_run[nb] = 0.f;
 #pragma unroll
@@ -396,18 +443,12 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[db][nb][i] = 0.f;
     if (p.accumulate && qrow[nb] >= 0) {
-      // resume from a previous partial attention: weight exp(lse_prev) with normalised output
+      // resume from a previous partial attention: it enters with weight exp(lse_prev - m) = 1; its
+      // normalised output rows are added when the result is written
       m_run[nb] = lb[qrow[nb]] * LOG2E;
       l_run[nb] = hi == 0 ? 1.f : 0.f;
-#pragma unroll
-      for (int db = 0; db < DB; ++db)
-#pragma unroll
-        for (int q4 = 0; q4 < 4; ++q4) {
-          const vec4 o = *reinterpret_cast<const vec4*>(ob + (int64_t)qrow[nb] * p.o_sn + db * 32 + q4 * 8 + hi * 4);
-#pragma unroll
-          for (int e = 0; e < 4; ++e) acc[db][nb][q4 * 4 + e] = (float)o[e];
-        }
     }
+    m_init[nb] = m_run[nb];
   }
 
   // per-lane LDS offsets of the MFMA operand reads
@@ -425,7 +466,7 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
       lo.v[db] = tile_offset<D>(key, db * 4 + (g & 1) * 2 + (w >> 1)) + (w & 1) * 8;
   }
 
-  // every wave's part of K(0), V(0), K(1) has landed before anyone reads the tiles
+  // every wave's part of Q, K tile 0, V tile 0, K tile 1 has landed before anyone reads the tiles
   __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
   __syncthreads();
 
@@ -436,8 +477,10 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
     return (CAUSAL && k_first + KC - 1 > wave_q_first) || (k_first + KC > p.n_k);
   };
   // element i of a lane is key  first + 8*(i/4) + i%4  with first = chunk*64 + mb*32 + 4*hi; it is
-  // dead when that exceeds `limit` = min(n_k - 1, query position) (everything is dead in gather mode)
+  // dead when that exceeds `limit` = min(n_k - 1, query position).  In gather mode a masked chunk is
+  // one whose keys belong to the other half of the workgroup: everything is dead.
 #define HA_APPLY_MASK(ci, mb, s)                                                        \
+  asm volatile("" ::); /* keeps this a branch: masked chunks are the exception */       \
   _Pragma("unroll") for (int nb = 0; nb < 2; ++nb) {                                    \
     const int first = (ci) * KC + (mb) * 32 + 4 * hi;                                   \
     int limit = p.n_k - 1;                                                              \
@@ -447,17 +490,18 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
       if (8 * (i >> 2) + (i & 3) > slack) s[nb][i] = -INFINITY;                         \
   }
 
-  // ---- main loop -----------------------------------------------------------------------------------
-  // s_a / s_b hold S^T of keys 0..31 / 32..63 of the chunk being consumed.  On entry of iteration ci
-  // s_a is complete and kf holds the K operands of keys 32..63 of K(ci); step 0 consumes s_a, fills
-  // s_b and fetches the operands of keys 0..31 of K(ci+1); step 1 consumes s_b, fills s_a and fetches
-  // those of keys 32..63 of K(ci+1).  K(ci) itself is no longer read from LDS in iteration ci, so
-  // K(ci+2) streams into its buffer meanwhile, and V(ci+1) into the buffer V(ci-1) left.
-  f32x16 s_a[2], s_b[2];
-  vec8 kf[KSTEPS];
-  {
+  // ---- Q fragments (B operand), S^T of the first 32 keys ---------------------------------------
+  vec8 qf[2][KSTEPS];
 #pragma unroll
-    for (int ks = 0; ks < KSTEPS; ++ks) kf[ks] = lds_read_k<T>(lds_k0, lo.k[ks]);
+  for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) qf[nb][ks] = lds_read_k<T>(my_q, lo.k[ks] + nb * 32 * D * 2);
+  // s_a / s_b hold S^T of keys 0..31 / 32..63 of the chunk being consumed
+  f32x16 s_a[2], s_b[2];
+  {
+    vec8 kf[KSTEPS];
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) kf[ks] = lds_read_k<T>(lds_k0, lo.k[ks] + 32 * D * 2);
 #pragma unroll
     for (int nb = 0; nb < 2; ++nb)
 #pragma unroll
@@ -466,48 +510,94 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
     for (int ks = 0; ks < KSTEPS; ++ks)
 #pragma unroll
       for (int nb = 0; nb < 2; ++nb) s_a[nb] = Mfma<T>::run(kf[ks], qf[nb][ks], s_a[nb]);
-#pragma unroll
-    for (int ks = 0; ks < KSTEPS; ++ks) kf[ks] = lds_read_k<T>(lds_k0, lo.k[ks] + 32 * D * 2);
   }
-  // all waves hold their operands of K(0): its buffer may be overwritten from iteration 0 on
+  // the P.V of "the half-step before the first" adds nothing
+  vec8 pb[2], vf[DB];
+#pragma unroll
+  for (int nb = 0; nb < 2; ++nb) pb[nb] = vec8{};
+#pragma unroll
+  for (int db = 0; db < DB; ++db) vf[db] = vec8{};
+  float alpha_pend[2] = {1.f, 1.f};  // accumulator rescale owed by the last half-step, if rescale_pend
+  bool rescale_pend = false;
+  bool pending = false;  // pb/vf hold a half-step whose P.V has not been issued
+  // all waves hold their operands of K tile 0: its buffer may be overwritten from iteration 0 on
   __syncthreads();
 
-  // the loop is unrolled by two so that every tile access names its LDS object statically
-#define HA_ITERATION(ci, K_CUR, K_NXT, V_CUR, V_NXT)                                                        \
+  // ---- main loop -----------------------------------------------------------------------------------
+  // Iteration ci consumes chunk ci: its steps 0 and 1 soft-max s_a and s_b, read V tile ci, and fill
+  // s_b and (for chunk ci+1) s_a from K tile ci+1.  Meanwhile K tile ci+2 streams into the buffer K
+  // tile ci was read from during iteration ci-1, and V tile ci+1 into the buffer of V tile ci-1.
+  // The loop is unrolled by two so that every tile access names its LDS object statically.
+#define HA_PV_DRAIN()                                                                                       \
+  if (rescale_pend) {                                                                                       \
+    _Pragma("unroll") for (int db = 0; db < DB; ++db) _Pragma("unroll") for (int nb = 0; nb < 2; ++nb)      \
+        _Pragma("unroll") for (int i = 0; i < 16; ++i) acc[db][nb][i] *= alpha_pend[nb];                    \
+    rescale_pend = false;                                                                                   \
+  }                                                                                                         \
+  _Pragma("unroll") for (int db = 0; db < DB; ++db) _Pragma("unroll") for (int nb = 0; nb < 2; ++nb)        \
+      acc[db][nb] = Mfma<T>::run(vf[db], pb[nb], acc[db][nb]);
+#define HA_ITERATION(ci, K_RD, K_WR, V_CUR, V_WR)                                                           \
   {                                                                                                         \
-    if ((ci) + 2 < n_chunks) { HA_LOAD_TILE(kb, p.k_sn, rows_k, K_CUR) } /* K(ci+2) */                      \
-    if ((ci) + 1 < n_chunks) { HA_LOAD_TILE(vb, p.v_sn, rows_v, V_NXT) } /* V(ci+1) */                      \
-    HA_FETCH_ROWS((ci) + 3, rows_k)                                                                         \
-    HA_FETCH_ROWS((ci) + 2, rows_v)                                                                         \
+    if ((ci) + 2 <= n_chunks) { HA_LOAD_TILE(kb, p.k_sn, rows_k, K_WR) } /* K tile ci+2 */                  \
+    if ((ci) + 1 < n_chunks) { HA_LOAD_TILE(vb, p.v_sn, rows_v, V_WR) }  /* V tile ci+1 */                  \
+    HA_FETCH_ROWS_K((ci) + 3, rows_k)                                                                       \
+    HA_FETCH_ROWS_V((ci) + 2, rows_v)                                                                       \
     /* causal: once a chunk lies wholly above this wave's queries, so do all later ones */                  \
     if (!(CAUSAL && (ci) * KC > wave_q_first + 63)) {                                                       \
       const bool masked = chunk_masked(ci);                                                                 \
       if (masked) { HA_APPLY_MASK(ci, 0, s_a) }                                                             \
-      pipeline_step<T, D>(s_a, s_b, kf, K_NXT, 0, V_CUR, 0, lo, qf, acc, m_run, l_run, p.scale_log2);       \
+      half_step<T, D, 0>(s_a, s_b, K_RD, 0, V_CUR, 0, lo, qf, acc, m_run, l_run, pb, vf,                    \
+                         p.scale_log2, alpha_pend, rescale_pend);                                           \
+      half_step<T, D, 1>(s_a, s_b, K_RD, 0, V_CUR, 16 * D * 2, lo, qf, acc, m_run, l_run, pb, vf,           \
+                         p.scale_log2, alpha_pend, rescale_pend);                                           \
       if (masked) { HA_APPLY_MASK(ci, 1, s_b) }                                                             \
-      pipeline_step<T, D>(s_b, s_a, kf, K_NXT, 1, V_CUR, 1, lo, qf, acc, m_run, l_run, p.scale_log2);       \
+      half_step<T, D, 0>(s_b, s_a, K_RD, 32 * D * 2, V_CUR, 32 * D * 2, lo, qf, acc, m_run, l_run, pb, vf,  \
+                         p.scale_log2, alpha_pend, rescale_pend);                                           \
+      half_step<T, D, 1>(s_b, s_a, K_RD, 32 * D * 2, V_CUR, 48 * D * 2, lo, qf, acc, m_run, l_run, pb, vf,  \
+                         p.scale_log2, alpha_pend, rescale_pend);                                           \
+      pending = true;                                                                                       \
+    } else if (pending) {                                                                                   \
+      HA_PV_DRAIN()                                                                                         \
+      pending = false;                                                                                      \
     }                                                                                                       \
-    __builtin_amdgcn_s_waitcnt(0x0F70); /* this wave's parts of K(ci+2), V(ci+1) have landed */             \
+    __builtin_amdgcn_s_waitcnt(0x0F70); /* this wave's parts of K tile ci+2, V tile ci+1 have landed */     \
     __syncthreads();                                                                                        \
   }
   for (int ci = 0; ci < n_chunks; ci += 2) {
-    HA_ITERATION(ci, lds_k0, lds_k1, lds_v0, lds_v1)
-    if (ci + 1 < n_chunks) HA_ITERATION(ci + 1, lds_k1, lds_k0, lds_v1, lds_v0)
+    HA_ITERATION(ci, lds_k1, lds_k0, lds_v0, lds_v1)
+    if (ci + 1 < n_chunks) HA_ITERATION(ci + 1, lds_k0, lds_k1, lds_v1, lds_v0)
   }
+  if (pending) { HA_PV_DRAIN() }
 #undef HA_ITERATION
+#undef HA_PV_DRAIN
 
   // ---- epilogue: normalise, stage O through LDS, write whole rows ---------------------------------
-  // A wave's 64 output rows are exactly one tile (64 rows of DV elements): wave w stages them in tile
-  // object w and writes them out itself, so no further workgroup barrier is needed.
-  unsigned char* const lds_o_raw = wave == 0 ? lds_k0 : (wave == 1 ? lds_k1 : (wave == 2 ? lds_v0 : lds_v1));
-  T* const lds_o = reinterpret_cast<T*>(lds_o_raw);
+  // A wave's 64 output rows are exactly one tile (64 rows of DV elements): it stages them in its
+  // query tile and writes them out itself, so no further workgroup barrier is needed.  Piece j of a
+  // lane belongs to the row its j-th query load fetched.
+  constexpr int OUT_PIECES = PR;  // 16-byte pieces per lane
+  int out_row[OUT_PIECES];
+  vec8 prev[OUT_PIECES];
+#pragma unroll
+  for (int j = 0; j < OUT_PIECES; ++j) out_row[j] = lds_qrow[wave * 64 + j * ROWS_PER_LOAD + my_lr];
+  if (p.accumulate) {
+#pragma unroll
+    for (int j = 0; j < OUT_PIECES; ++j) {
+      prev[j] = vec8{};
+      if (out_row[j] >= 0) prev[j] = *reinterpret_cast<const vec8*>(ob + (int64_t)out_row[j] * p.o_sn + my_pp * 8);
+    }
+  }
+  T* const lds_o = reinterpret_cast<T*>(my_q);
 #pragma unroll
   for (int nb = 0; nb < 2; ++nb) {
     const float l_tot = l_run[nb] + __shfl_xor(l_run[nb], 32);
     const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
     const int lrow = nb * 32 + col;
-    if (hi == 0 && qrow[nb] >= 0)
-      lb[qrow[nb]] = l_tot > 0.f ? (m_run[nb] + __builtin_amdgcn_logf(l_tot)) * LN2 : -INFINITY;
+    if (hi == 0) {
+      if (qrow[nb] >= 0) lb[qrow[nb]] = l_tot > 0.f ? (m_run[nb] + __builtin_amdgcn_logf(l_tot)) * LN2 : -INFINITY;
+      // weight of the resumed rows: exp(lse_prev - m_final) / l_tot
+      lds_w[wave * 64 + lrow] = m_init[nb] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m_init[nb] - m_run[nb]) * inv;
+    }
 #pragma unroll
     for (int db = 0; db < DB; ++db)
 #pragma unroll
@@ -522,17 +612,20 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
   __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): this wave's LDS writes are done
   __builtin_amdgcn_wave_barrier();
 #pragma unroll
-  for (int j = 0; j < 64 * PR / HA_WAVE; ++j) {
-    const int i = lane + j * HA_WAVE;
-    const int lrow = i / PR, pc = i % PR;
-    const int pq = qt * WG_QUERIES + wave * 64 + lrow;
-    if (pq < p.n_q) {
-      const int row = GATHER ? ha_load_idx(p.q_idx, qidx_off + (int64_t)pq * p.qi_sn, p.idx64) : pq;
-      const vec8 o = *reinterpret_cast<const vec8*>(&lds_o[lrow * DV + ((pc ^ (lrow & 7)) * 8)]);
-      *reinterpret_cast<vec8*>(ob + (int64_t)row * p.o_sn + pc * 8) = o;
+  for (int j = 0; j < OUT_PIECES; ++j) {
+    const int lrow = j * ROWS_PER_LOAD + my_lr;
+    if (out_row[j] >= 0) {
+      vec8 o = *reinterpret_cast<const vec8*>(&lds_o[lrow * DV + ((my_pp ^ (lrow & 7)) * 8)]);
+      if (p.accumulate) {
+        const float w = lds_w[wave * 64 + lrow];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) o[e] = (T)__builtin_fmaf(w, (float)prev[j][e], (float)o[e]);
+      }
+      *reinterpret_cast<vec8*>(ob + (int64_t)out_row[j] * p.o_sn + my_pp * 8) = o;
     }
   }
-#undef HA_FETCH_ROWS
+#undef HA_FETCH_ROWS_K
+#undef HA_FETCH_ROWS_V
 #undef HA_LOAD_TILE
 #undef HA_APPLY_MASK
 }

@@ -68,5 +68,7 @@ __device__ __forceinline__ float ha_to_float(bf16_t v) { return (float)v; }
 
 // index loads of either width
 __device__ __forceinline__ int ha_load_idx(const void* base, int64_t off, int is64) {
-  return is64 ? (int)((const int64_t*)base)[off] : ((const int32_t*)base)[off];
+  // one load either way (row numbers fit the low word of a little-endian int64), so that the value
+  // is not consumed by a select right behind the load
+  return *reinterpret_cast<const int32_t*>(static_cast<const char*>(base) + (off << (is64 ? 3 : 2)));
 }
