@@ -210,6 +210,9 @@ __device__ __forceinline__ void half_step(const f32x16 (&s_use)[2], f32x16 (&s_f
   vec8 vf_next[DB];
 #pragma unroll
   for (int db = 0; db < DB; ++db) vf_next[db] = lds_read_vt<T>(v_tile, lo.v[db] + v_key_off, D * 2);
+  // the LDS reads stay at the head of the block: their latency hides behind the P.V MFMAs and the
+  // exponentials instead of being waited for where the compiler would sink them to
+  __builtin_amdgcn_sched_barrier(0);
 
 #pragma unroll
   for (int db = 0; db < DB; ++db)
@@ -345,8 +348,16 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
   // n_k and chunks outside 0..n_chunks-1 alias row 0: row 0 holds finite data and their scores are
   // masked or never used.  Every branch is wave-uniform and nothing touches a loaded value here: the
   // loads stay in flight until the row numbers are needed for the tile loads of a later iteration.
+  // Loaded row numbers live in registers that only loads write (rows); consecutive rows are kept as
+  // their wave-uniform first row and turned into per-lane numbers where they are used, so a register
+  // with a load in flight is never overwritten by a vector instruction (which would have to wait).
   const int idx_shift = p.idx64 ? 3 : 2;
-  auto fetch_rows = [&](int ci, int kk0, int (&rows)[LPW]) {
+  constexpr int ROWS_LOADED = -1, ROWS_NONE = -2;  // values of RowSource::first
+  struct RowSource {
+    int rows[LPW];  // valid when first == ROWS_LOADED
+    int first;      // >= 0: rows first + key number; ROWS_NONE: chunk out of range (row 0)
+  };
+  auto fetch_rows = [&](int ci, int kk0, RowSource& rs) {
     const unsigned char* src = nullptr;  // index array run, or null for consecutive rows
     int64_t stride = 0;
     int first = 0;
@@ -368,18 +379,14 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
       first = ci * KC;
     }
     if (ci < 0 || ci >= n_chunks) {
-#pragma unroll
-      for (int j = 0; j < LPW; ++j) rows[j] = 0;
+      rs.first = ROWS_NONE;
     } else if (src) {
+      rs.first = ROWS_LOADED;
 #pragma unroll
       for (int j = 0; j < LPW; ++j)
-        rows[j] = *reinterpret_cast<const int*>(src + (kk0 + j * ROWS_PER_LOAD + my_lr) * stride);
+        rs.rows[j] = *reinterpret_cast<const int*>(src + (kk0 + j * ROWS_PER_LOAD + my_lr) * stride);
     } else {
-#pragma unroll
-      for (int j = 0; j < LPW; ++j) {
-        const int row = first + kk0 + j * ROWS_PER_LOAD + my_lr;
-        rows[j] = (GATHER || row < p.n_k) ? row : 0;
-      }
+      rs.first = first;
     }
   };
   // V tile c holds keys 0..63 of chunk c.  K tile c holds keys 32..63 of chunk c-1 in its rows 0..31
@@ -387,36 +394,52 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
   const int v_kk0 = wave * (LPW * ROWS_PER_LOAD);
   const int k_kk0 = (v_kk0 + 32) & 63;
   const int k_chunk_shift = (wave >> 1) - 1;
-#define HA_FETCH_ROWS_K(tile_c, rows) fetch_rows((tile_c) + k_chunk_shift, k_kk0, rows);
-#define HA_FETCH_ROWS_V(ci, rows) fetch_rows((ci), v_kk0, rows);
-#define HA_LOAD_TILE(base, stride, rows, tile)                                                           \
+#define HA_FETCH_ROWS_K(tile_c, rs) fetch_rows((tile_c) + k_chunk_shift, k_kk0, rs);
+#define HA_FETCH_ROWS_V(ci, rs) fetch_rows((ci), v_kk0, rs);
+#define HA_LOAD_TILE(base, stride, rs, kk0, tile)                                                        \
   _Pragma("unroll") for (int j = 0; j < LPW; ++j) {                                                      \
     const int r = (wave * LPW + j) * ROWS_PER_LOAD + my_lr;                                              \
-    const T* src = (base) + (int64_t)rows[j] * (stride) + ((my_pp ^ (r & 7)) << 3);                      \
+    int row = rs.first + (kk0) + j * ROWS_PER_LOAD + my_lr; /* consecutive rows */                       \
+    if (!GATHER && row >= p.n_k) row = 0;                                                                \
+    if (GATHER && rs.first == ROWS_LOADED) row = rs.rows[j];                                             \
+    if (rs.first == ROWS_NONE) row = 0;                                                                  \
+    const T* src = (base) + (int64_t)row * (stride) + ((my_pp ^ (r & 7)) << 3);                          \
     global_to_lds_16(src, (tile) + (wave * LPW + j) * 1024);                                             \
   }
 
   // ---- first loads: row numbers of the queries and of the first key tiles, then the rows ----------
   unsigned char* const my_q = lds_q + wave * TILE_BYTES;
-  int rows_k[LPW], rows_v[LPW];
+  RowSource rows_k, rows_v;
+#pragma unroll
+  for (int j = 0; j < LPW; ++j) rows_k.rows[j] = rows_v.rows[j] = 0;
   int qrow[2];  // original row of the query a lane's S^T / O^T columns belong to
   {
     int q_rows[PR];  // rows of this wave's query tile, in the order of its PR loads
 #pragma unroll
     for (int j = 0; j < PR; ++j) {
+      // positions past the end load the index of position 0 (replaced by -1 below, once all the
+      // index loads of this prologue are in flight)
       const int pq = wave_q_first + j * ROWS_PER_LOAD + my_lr;
-      q_rows[j] = pq >= p.n_q ? -1 : (GATHER ? ha_load_idx(p.q_idx, qidx_off + (int64_t)pq * p.qi_sn, p.idx64) : pq);
+      q_rows[j] = GATHER ? ha_load_idx(p.q_idx, qidx_off + (int64_t)(pq < p.n_q ? pq : 0) * p.qi_sn, p.idx64) : pq;
     }
 #pragma unroll
     for (int nb = 0; nb < 2; ++nb) {
       const int pq = wave_q_first + nb * 32 + col;
-      qrow[nb] = pq >= p.n_q ? -1 : (GATHER ? ha_load_idx(p.q_idx, qidx_off + (int64_t)pq * p.qi_sn, p.idx64) : pq);
+      qrow[nb] = GATHER ? ha_load_idx(p.q_idx, qidx_off + (int64_t)(pq < p.n_q ? pq : 0) * p.qi_sn, p.idx64) : pq;
     }
-    int rows_k1[LPW];
+    RowSource rows_k1;
+#pragma unroll
+    for (int j = 0; j < LPW; ++j) rows_k1.rows[j] = 0;
     HA_FETCH_ROWS_K(0, rows_k)
     HA_FETCH_ROWS_V(0, rows_v)
     HA_FETCH_ROWS_K(1, rows_k1)
-    HA_LOAD_TILE(kb, p.k_sn, rows_k, lds_k0)
+#pragma unroll
+    for (int j = 0; j < PR; ++j)
+      if (wave_q_first + j * ROWS_PER_LOAD + my_lr >= p.n_q) q_rows[j] = -1;
+#pragma unroll
+    for (int nb = 0; nb < 2; ++nb)
+      if (wave_q_first + nb * 32 + col >= p.n_q) qrow[nb] = -1;
+    HA_LOAD_TILE(kb, p.k_sn, rows_k, k_kk0, lds_k0)
 #pragma unroll
     for (int j = 0; j < PR; ++j) {
       // positions past the end read row 0 (finite data; their results are never written)
@@ -425,8 +448,8 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
       global_to_lds_16(src, my_q + j * 1024);
       if (my_pp == 0) lds_qrow[wave * 64 + r] = q_rows[j];
     }
-    HA_LOAD_TILE(vb, p.v_sn, rows_v, lds_v0)
-    HA_LOAD_TILE(kb, p.k_sn, rows_k1, lds_k1)
+    HA_LOAD_TILE(vb, p.v_sn, rows_v, v_kk0, lds_v0)
+    HA_LOAD_TILE(kb, p.k_sn, rows_k1, k_kk0, lds_k1)
   }
   HA_FETCH_ROWS_K(2, rows_k)
   HA_FETCH_ROWS_V(1, rows_v)
@@ -538,8 +561,8 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
       acc[db][nb] = Mfma<T>::run(vf[db], pb[nb], acc[db][nb]);
 #define HA_ITERATION(ci, K_RD, K_WR, V_CUR, V_WR)                                                           \
   {                                                                                                         \
-    if ((ci) + 2 <= n_chunks) { HA_LOAD_TILE(kb, p.k_sn, rows_k, K_WR) } /* K tile ci+2 */                  \
-    if ((ci) + 1 < n_chunks) { HA_LOAD_TILE(vb, p.v_sn, rows_v, V_WR) }  /* V tile ci+1 */                  \
+    if ((ci) + 2 <= n_chunks) { HA_LOAD_TILE(kb, p.k_sn, rows_k, k_kk0, K_WR) } /* K tile ci+2 */           \
+    if ((ci) + 1 < n_chunks) { HA_LOAD_TILE(vb, p.v_sn, rows_v, v_kk0, V_WR) }  /* V tile ci+1 */           \
     HA_FETCH_ROWS_K((ci) + 3, rows_k)                                                                       \
     HA_FETCH_ROWS_V((ci) + 2, rows_v)                                                                       \
     /* causal: once a chunk lies wholly above this wave's queries, so do all later ones */                  \
