@@ -278,7 +278,8 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
   const int wg = xcd_contiguous_id(blockIdx.x, gridDim.x);
   const int qtiles = (p.n_q + WG_QUERIES - 1) / WG_QUERIES;
   const int vhead = wg / qtiles;
-  const int qt = wg % qtiles;
+  // causal: the tiles with the most keys go first, so that the last workgroups of the grid are short
+  const int qt = CAUSAL ? qtiles - 1 - wg % qtiles : wg % qtiles;
   const int seg = vhead % p.segs;
   const int bh = vhead / p.segs;
   const int b = bh / p.heads, h = bh % p.heads;
