@@ -29,6 +29,9 @@ sys.path.insert(0, ROOT)
 METRIC = "HyperAttention fwd ms + MFMA util at seq 131k, 32 heads, d=64, fp16 causal"
 MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense fp16/bf16
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per launch of the gathered attention kernel, measured with rocprofv3 --pmc (see the
+# summary of that run under profiles/); only the workload that was measured has a figure
+MEASURED_TRAFFIC_BYTES = {"c3": 1.3936e9}
 
 WORKLOADS = {
     # name: batch, q heads, kv heads, n, d, dtype, causal, block, sample, min_seq_len, smooth
@@ -235,15 +238,28 @@ def main():
 
     blk_avg = sum(blk_ms) / len(blk_ms)
     blk_flops = per_level[0]
+    # algorithmic HBM bytes of one launch: Q rows, the gathered K and V rows of the blocks, output rows and
+    # lse, the sorted index arrays, and (causal: resumed partial result) the previous rows and lse; the
+    # sampled rows are shared by all query blocks of a head
+    lvl_q = b * h * (n // 2 if w["causal"] else n)
+    lvl_k = lvl_q  # one key block per query block
+    row_b = d * 2
+    blk_bytes = lvl_q * row_b + 2 * lvl_k * row_b + lvl_q * (row_b + 4) + (lvl_q + lvl_k) * 4
+    if w["causal"]:
+        blk_bytes += lvl_q * (row_b + 4)
     achieved = blk_flops / blk_avg / 1e9  # TFLOP/s
     roofline = {"kernel": "attn_fwd_kernel<gather> (block-diagonal + sampled attention)", "bound": "mfma",
                 "achieved": round(achieved, 1), "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
-                "frac": round(achieved / MFMA_PEAK_TFLOPS, 4), "traffic": None,
+                "frac": round(achieved / MFMA_PEAK_TFLOPS, 4),
+                # HBM bytes per launch from the FETCH_SIZE / WRITE_SIZE counter runs of this workload
+                # (fetch counter x 2.000, write counter x 1.000, factors from a plain copy of known size)
+                "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+                "algorithmic_bytes": blk_bytes,
                 "flops_per_launch": blk_flops, "avg_launch_ms": round(blk_avg, 4),
                 "launch_ms_by_level": [round(x, 4) for x in blk_ms]}
     sort_elems = sum((rows_q // 2 + rows_k // 2) if w["causal"] else (rows_q + rows_k) for _ in halves)
     sort_total = sum(sort_ms)
-    kernels["bucket_argsort(all levels)"] = {"ms": round(sort_total, 4), "bound": "hbm", "bytes": sort_elems * 8,
+    kernels["bucket_argsort(one launch per level and side)"] = {"ms": round(sort_total, 4), "bound": "hbm", "bytes": sort_elems * 8,
                                              "achieved_GBs": round(sort_elems * 8 / sort_total / 1e6, 1),
                                              "frac": round(sort_elems * 8 / sort_total / 1e6 / HBM_PEAK_GBS, 4)}
     if leaf is not None:
