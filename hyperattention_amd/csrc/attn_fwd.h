@@ -27,6 +27,9 @@ struct ha_attn_kernel_params {
   int sample_chunks;  // sample_size / 64
   int smooth, accumulate, idx64;
   float scale_log2;   // softmax scale * log2(e)
+  // log2 of the divisors of the workgroup -> (head, segment, tile) decomposition when they are powers
+  // of two, else -1 (filled by ha_attn_launch): the kernel then shifts instead of dividing
+  int qtiles_shift, segs_shift, heads_shift, kv_group_shift, block_tiles_shift;
 };
 
 int ha_attn_launch(const ha_attn_kernel_params& p, int d, int dtype, bool gather, bool causal, hipStream_t stream);

@@ -84,6 +84,9 @@ __device__ __forceinline__ int xcd_contiguous_id(int linear, int total) {
   return xcd * q + (xcd < r ? xcd : r) + k;
 }
 
+// x / y for non-negative x; shift = log2(y) when y is a power of two, else -1
+__device__ __forceinline__ int fast_div(int x, int y, int shift) { return shift >= 0 ? x >> shift : x / y; }
+
 // LDS byte offsets of one lane's operand reads, relative to a tile base (fixed for the whole kernel).
 template <int D>
 struct LaneOffsets {
@@ -277,13 +280,14 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
   // ---- which (virtual) head and query tile -----------------------------------------------------
   const int wg = xcd_contiguous_id(blockIdx.x, gridDim.x);
   const int qtiles = (p.n_q + WG_QUERIES - 1) / WG_QUERIES;
-  const int vhead = wg / qtiles;
+  const int vhead = fast_div(wg, qtiles, p.qtiles_shift);
   // causal: the tiles with the most keys go first, so that the last workgroups of the grid are short
-  const int qt = CAUSAL ? qtiles - 1 - wg % qtiles : wg % qtiles;
-  const int seg = vhead % p.segs;
-  const int bh = vhead / p.segs;
-  const int b = bh / p.heads, h = bh % p.heads;
-  const int hk = h / p.kv_group;
+  const int qt_fwd = wg - vhead * qtiles;
+  const int qt = CAUSAL ? qtiles - 1 - qt_fwd : qt_fwd;
+  const int bh = fast_div(vhead, p.segs, p.segs_shift);
+  const int seg = vhead - bh * p.segs;
+  const int b = fast_div(bh, p.heads, p.heads_shift), h = bh - b * p.heads;
+  const int hk = fast_div(h, p.kv_group, p.kv_group_shift);
 
   const T* qb = (const T*)p.q + b * p.q_sb + h * p.q_sh + (p.q_seg_off + (int64_t)seg * p.seg_stride) * p.q_sn;
   const T* kb = (const T*)p.k + b * p.k_sb + hk * p.k_sh + (p.k_seg_off + (int64_t)seg * p.seg_stride) * p.k_sn;
@@ -303,14 +307,14 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
 #pragma unroll
     for (int t2 = 0; t2 < 2; ++t2) {
       const int t = qt * 2 + t2;  // reference query tile of 128
-      const int block_id = t / p.block_tiles;
+      const int block_id = fast_div(t, p.block_tiles, p.block_tiles_shift);
       const int first = block_id * p.block_tiles * 128;
       int last = (block_id + 1) * p.block_tiles * 128;
       last = last < p.n_k ? last : p.n_k;
       int cnt = last > first ? (last - first) / KC : 0;
       if (t * 128 >= p.n_q) cnt = 0;
       int s = first / KC;
-      if (p.smooth) s = (first + p.n_k + (t % p.block_tiles) * 128 - ((p.block_tiles - 1) * 128) / 2) / KC;
+      if (p.smooth) s = (first + p.n_k + (t - block_id * p.block_tiles) * 128 - ((p.block_tiles - 1) * 128) / 2) / KC;
       start[t2] = s;
       end[t2] = s + cnt;
     }
@@ -671,8 +675,21 @@ int launch_variant(const ha_attn_kernel_params& p, int grid, bool gather, bool c
 
 }  // namespace
 
-int ha_attn_launch(const ha_attn_kernel_params& p, int d, int dtype, bool gather, bool causal, hipStream_t stream) {
+static int log2_if_pow2(int64_t v) {
+  if (v <= 0 || (v & (v - 1))) return -1;
+  int s = 0;
+  while ((int64_t(1) << s) < v) ++s;
+  return s;
+}
+
+int ha_attn_launch(const ha_attn_kernel_params& params, int d, int dtype, bool gather, bool causal, hipStream_t stream) {
+  ha_attn_kernel_params p = params;
   const int64_t qtiles = (p.n_q + WG_QUERIES - 1) / WG_QUERIES;
+  p.qtiles_shift = log2_if_pow2(qtiles);
+  p.segs_shift = log2_if_pow2(p.segs);
+  p.heads_shift = log2_if_pow2(p.heads);
+  p.kv_group_shift = log2_if_pow2(p.kv_group);
+  p.block_tiles_shift = log2_if_pow2(p.block_tiles);
   const int64_t grid = qtiles * p.batch * p.heads * p.segs;
   if (grid <= 0 || grid >= (1ll << 31)) return ha_fail(HA_ERR_SHAPE, "attention: grid of %lld workgroups", (long long)grid);
   if (dtype == HA_F16) {
