@@ -129,11 +129,14 @@ def _operands(q, k, v, out, lse, scale, *, layout_bnhd: bool, lse_row_stride: in
 
 
 def hyper_attn_func(q, k, v, q_sort_idx, k_sort_idx, block_size, sample_size=0, softmax_scale=None,
-                    smooth_block=False, *, sampled_idx=None):
+                    smooth_block=False, *, sampled_idx=None, resume=None):
     """q, k: (batch, seqlen, nheads, headdim); v: (batch, seqlen, nheads, v_headdim);
     q_sort_idx, k_sort_idx: (batch, seqlen, nheads) permutations; returns o (batch, seqlen, nheads,
     v_headdim) and lse (batch, nheads, seqlen) fp32.  `sampled_idx` (keyword only, not in the
-    reference) lists the sampled key rows, shape (sample_size,); default 0..sample_size-1."""
+    reference) lists the sampled key rows, shape (sample_size,); default 0..sample_size-1.
+    `resume` (keyword only, not in the reference) is a pair (o, lse) of a previous partial attention
+    over other keys, shaped like the results: the kernel continues from it and updates both in place,
+    which equals add_self_attentions(previous, this call) in fp32."""
     q, k, v = [x if x.stride(-1) == 1 else x.contiguous() for x in [q, k, v]]
     assert sample_size % 128 == 0
     batch, seqlen_q, nheads, d = q.shape
@@ -148,8 +151,14 @@ def hyper_attn_func(q, k, v, q_sort_idx, k_sort_idx, block_size, sample_size=0, 
     assert q.is_cuda and k.is_cuda and v.is_cuda and q_sort_idx.is_cuda and k_sort_idx.is_cuda
     assert q_sort_idx.dtype == k_sort_idx.dtype
     softmax_scale = softmax_scale or 1.0 / math.sqrt(d)
-    lse = torch.empty((batch, nheads, seqlen_q), device=q.device, dtype=torch.float32)
-    o = torch.empty((batch, seqlen_q, nheads, v.shape[-1]), device=q.device, dtype=q.dtype)
+    if resume is None:
+        lse = torch.empty((batch, nheads, seqlen_q), device=q.device, dtype=torch.float32)
+        o = torch.empty((batch, seqlen_q, nheads, v.shape[-1]), device=q.device, dtype=q.dtype)
+    else:
+        o, lse = resume
+        assert o.shape == (batch, seqlen_q, nheads, v.shape[-1]) and o.dtype == q.dtype and o.is_cuda
+        assert lse.shape == (batch, nheads, seqlen_q) and lse.dtype == torch.float32 and lse.is_contiguous()
+        assert o.stride(-1) == 1
     assert seqlen_k % 128 == 0, "keys sequence length must be divisible by 128"
 
     a = BlockAttnArgs()
@@ -165,7 +174,7 @@ def hyper_attn_func(q, k, v, q_sort_idx, k_sort_idx, block_size, sample_size=0, 
         a.sampled_idx = keep.data_ptr()
     a.sampled_stride_b = a.sampled_stride_h = 0
     a.block_size, a.sample_size = block_size, sample_size
-    a.smooth_block, a.accumulate = int(bool(smooth_block)), 0
+    a.smooth_block, a.accumulate = int(bool(smooth_block)), int(resume is not None)
     with torch.cuda.device(q.device):
         _lib.check(_lib.lib().ha_block_attn_fwd(ctypes.byref(a), _stream(q)))
     return o, lse

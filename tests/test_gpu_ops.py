@@ -138,6 +138,25 @@ def test_flash_attention_different_lengths_and_scale(ha):
     assert_close(lse[:, :, :300], rl, "flash lse")
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("causal", [False, True])
+def test_flash_attention_wide_logit_range(ha, dtype, causal):
+    """Scores spanning ~100 log2 units whose row maxima keep growing along the key sequence: the
+    kernel's reference exponent has to be raised again and again (its rare path), late keys dominate."""
+    b, h, n, d = 1, 2, 1536, 64
+    q, k, v = (_randn((b, n, h, d), s, dtype) for s in (61, 62, 63))
+    direction = torch.nn.functional.normalize(_randn((d,), 64, torch.float32), dim=0)
+    ramp = torch.linspace(-4.0, 4.0, n).view(1, n, 1, 1)           # keys drift along `direction`
+    k = (k.float() + ramp * direction * 16.0).to(dtype)
+    q = (q.float() * 0.5 + direction * 4.0 * torch.sign(_randn((b, n, h, 1), 65, torch.float32))).to(dtype)
+    o, lse = ha.flash_attn_func(q.cuda(), k.cuda(), v.cuda(), None, causal, None)
+    ro, rl = O.exact_attention(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), None, causal)
+    spread = (q.float().transpose(1, 2) @ k.float().transpose(1, 2).transpose(-1, -2) / 8.0)
+    assert (spread.max() - spread.min()) * 1.4427 > 60, "the case must span many powers of two"
+    assert_close(o.transpose(1, 2), ro, "flash out", dtype)
+    assert_close(lse[:, :, :n], rl, "flash lse")
+
+
 def test_flash_rejects_bias_and_bad_types(ha):
     q = torch.zeros((1, 128, 1, 64), dtype=torch.float16, device="cuda")
     with pytest.raises(NotImplementedError):
@@ -206,6 +225,37 @@ def test_block_attention_full_block_is_exact_attention(ha):
     ro, rl = O.exact_attention(q, k, v)
     assert_close(o, ro, "hyper out", torch.float16)
     assert_close(lse, rl, "hyper lse")
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("shift", [-30.0, 0.0, 30.0])
+def test_block_attention_resumes_partial_result(ha, dtype, shift):
+    """resume=(o, lse): the kernel continues a partial attention over other keys (add_self_attentions,
+    src/attn_utils.py:6-50, folded into the kernel).  `shift` moves the previous part's scores far below
+    / above the new ones; some rows have an empty previous part (lse = -inf)."""
+    b, h, n, d = 1, 2, 512, 64
+    q, k, v, qi, ki = _sorted_inputs(b, h, n, d, dtype, 70)
+    k_prev, v_prev = (_randn((b, h, 256, d), s, dtype) for s in (74, 75))
+    scale = d ** -0.5
+    s_prev = q.double() @ k_prev.double().transpose(-1, -2) * scale + shift
+    s_new = q.double() @ k.double().transpose(-1, -2) * scale
+    l_prev = torch.logsumexp(s_prev, dim=-1)
+    o_prev = torch.softmax(s_prev, dim=-1) @ v_prev.double()
+    l_prev[:, :, ::7] = float("-inf")          # rows without a previous part
+    o_prev[:, :, ::7] = 0.0
+    o_dev = o_prev.to(dtype).cuda().transpose(1, 2).contiguous()       # (b, n, h, d)
+    l_dev = l_prev.float().cuda().contiguous()
+    c = lambda t: t.cuda()
+    o, lse = ha.hyper_attn_func(c(q).transpose(1, 2), c(k).transpose(1, 2), c(v).transpose(1, 2),
+                                c(qi).transpose(1, 2), c(ki).transpose(1, 2), n, 0, None, False,
+                                resume=(o_dev, l_dev))
+    assert o.data_ptr() == o_dev.data_ptr() and lse.data_ptr() == l_dev.data_ptr()
+    # expected: exact attention over the union, the previous part entering through its ROUNDED rows
+    w_prev = torch.exp(l_prev.float().double() - torch.logaddexp(l_prev.float().double(), torch.logsumexp(s_new, -1)))
+    want = w_prev.unsqueeze(-1) * o_prev.to(dtype).double() + (1 - w_prev).unsqueeze(-1) * (torch.softmax(s_new, -1) @ v.double())
+    want_lse = torch.logaddexp(l_prev.float().double(), torch.logsumexp(s_new, -1))
+    assert_close(o.transpose(1, 2), want, "resumed out", dtype)
+    assert_close(lse, want_lse, "resumed lse")
 
 
 def test_block_attention_argument_errors(ha):
