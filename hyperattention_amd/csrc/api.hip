@@ -23,7 +23,8 @@ int check_operands(const ha_attn_operands& t, const char* who) {
   HA_REQUIRE(t.q && t.k && t.v && t.out && t.lse, HA_ERR_NULL, "%s: null tensor pointer", who);
   HA_REQUIRE(t.dtype == HA_F16 || t.dtype == HA_BF16, HA_ERR_DTYPE, "%s: Only support fp16 and bf16", who);
   HA_REQUIRE(t.batch > 0 && t.heads > 0 && t.n_q > 0 && t.n_k > 0, HA_ERR_SHAPE, "%s: sizes must be positive", who);
-  HA_REQUIRE(t.n_q < (1ll << 30) && t.n_k < (1ll << 30), HA_ERR_SHAPE, "%s: sequence too long", who);
+  // the kernels address a row as a per-head base plus a 32-bit byte offset computed with a 24-bit multiply
+  HA_REQUIRE(t.n_q < (1ll << 24) && t.n_k < (1ll << 24), HA_ERR_SHAPE, "%s: sequence too long (2^24 rows at most)", who);
   HA_REQUIRE(t.d <= 128, HA_ERR_HEADDIM, "%s: FlashAttention only support head dimensions up to 128", who);
   HA_REQUIRE(t.d == 64 || t.d == 128, HA_ERR_UNSUPPORTED, "%s: head dim %lld not built (64 and 128 are)", who,
              (long long)t.d);
@@ -37,6 +38,14 @@ int check_operands(const ha_attn_operands& t, const char* who) {
   HA_REQUIRE(((uintptr_t)t.q % 16) == 0 && ((uintptr_t)t.k % 16) == 0 && ((uintptr_t)t.v % 16) == 0 &&
                  ((uintptr_t)t.out % 16) == 0,
              HA_ERR_SHAPE, "%s: tensors must be 16-byte aligned", who);
+  const int64_t row_strides[] = {t.q_stride_n, t.k_stride_n, t.v_stride_n, t.o_stride_n};
+  const int64_t row_counts[] = {t.n_q, t.n_k, t.n_k, t.n_q};
+  for (int i = 0; i < 4; ++i) {
+    HA_REQUIRE(row_strides[i] > 0 && row_strides[i] * 2 < (1ll << 24), HA_ERR_UNSUPPORTED,
+               "%s: row strides must be positive and below 16 MiB", who);
+    HA_REQUIRE((row_counts[i] - 1) * row_strides[i] * 2 + t.d * 2 <= (1ll << 32), HA_ERR_UNSUPPORTED,
+               "%s: one head of a tensor may span 4 GiB at most", who);
+  }
   return HA_OK;
 }
 
@@ -70,6 +79,13 @@ int block_attn(const ha_block_attn_args& a, hipStream_t stream) {
   HA_REQUIRE(a.block_size > 0, HA_ERR_SHAPE, "ha_block_attn_fwd: block_size must be positive");
   HA_REQUIRE(a.sampled_idx || a.sample_size <= a.t.n_k, HA_ERR_SHAPE,
              "ha_block_attn_fwd: default sampled rows 0..sample_size-1 exceed the key length");
+  {
+    const int64_t esz = a.idx_type == HA_IDX_I64 ? 8 : 4;
+    HA_REQUIRE(a.q_idx_stride_n > 0 && a.k_idx_stride_n > 0 && a.q_idx_stride_n * esz < (1ll << 24) &&
+                   a.k_idx_stride_n * esz < (1ll << 24) && (a.t.n_q - 1) * a.q_idx_stride_n * esz < (1ll << 32) &&
+                   (a.t.n_k - 1) * a.k_idx_stride_n * esz < (1ll << 32),
+               HA_ERR_UNSUPPORTED, "ha_block_attn_fwd: index strides must be positive, below 16 MiB, and span 4 GiB at most");
+  }
   ha_attn_kernel_params p;
   fill_params(a.t, p);
   p.q_idx = a.q_idx; p.k_idx = a.k_idx; p.sampled_idx = a.sampled_idx;

@@ -87,6 +87,14 @@ __device__ __forceinline__ int xcd_contiguous_id(int linear, int total) {
 // x / y for non-negative x; shift = log2(y) when y is a power of two, else -1
 __device__ __forceinline__ int fast_div(int x, int y, int shift) { return shift >= 0 ? x >> shift : x / y; }
 
+// Address of 16-byte piece `piece_bytes` of row `row`: a wave-uniform base plus a 32-bit byte offset,
+// so that a lane spends one 24-bit multiply-add on it instead of a 64-bit multiplication.  The entry
+// points check that row numbers and row strides in bytes stay below 2^24 and their products below 2^32.
+__device__ __forceinline__ const unsigned char* row_address(const unsigned char* base, int row, uint32_t stride_bytes,
+                                                            uint32_t piece_bytes) {
+  return base + (uint32_t)(__umul24((uint32_t)row, stride_bytes) + piece_bytes);
+}
+
 // LDS byte offsets of one lane's operand reads, relative to a tile base (fixed for the whole kernel).
 template <int D>
 struct LaneOffsets {
@@ -289,10 +297,12 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
   const int b = fast_div(bh, p.heads, p.heads_shift), h = bh - b * p.heads;
   const int hk = fast_div(h, p.kv_group, p.kv_group_shift);
 
-  const T* qb = (const T*)p.q + b * p.q_sb + h * p.q_sh + (p.q_seg_off + (int64_t)seg * p.seg_stride) * p.q_sn;
-  const T* kb = (const T*)p.k + b * p.k_sb + hk * p.k_sh + (p.k_seg_off + (int64_t)seg * p.seg_stride) * p.k_sn;
-  const T* vb = (const T*)p.v + b * p.v_sb + hk * p.v_sh + (p.k_seg_off + (int64_t)seg * p.seg_stride) * p.v_sn;
-  T* ob = (T*)p.out + b * p.o_sb + h * p.o_sh + (p.q_seg_off + (int64_t)seg * p.seg_stride) * p.o_sn;
+  // bases of this (virtual) head as byte pointers, row strides in bytes
+  const unsigned char* qb = (const unsigned char*)((const T*)p.q + b * p.q_sb + h * p.q_sh + (p.q_seg_off + (int64_t)seg * p.seg_stride) * p.q_sn);
+  const unsigned char* kb = (const unsigned char*)((const T*)p.k + b * p.k_sb + hk * p.k_sh + (p.k_seg_off + (int64_t)seg * p.seg_stride) * p.k_sn);
+  const unsigned char* vb = (const unsigned char*)((const T*)p.v + b * p.v_sb + hk * p.v_sh + (p.k_seg_off + (int64_t)seg * p.seg_stride) * p.v_sn);
+  unsigned char* ob = (unsigned char*)((T*)p.out + b * p.o_sb + h * p.o_sh + (p.q_seg_off + (int64_t)seg * p.seg_stride) * p.o_sn);
+  const uint32_t q_rb = (uint32_t)p.q_sn * 2, k_rb = (uint32_t)p.k_sn * 2, v_rb = (uint32_t)p.v_sn * 2, o_rb = (uint32_t)p.o_sn * 2;
   float* lb = p.lse + b * p.lse_sb + h * p.lse_sh + p.q_seg_off + (int64_t)seg * p.seg_stride;
   const int64_t qidx_off = b * p.qi_sb + h * p.qi_sh + (int64_t)seg * p.n_q * p.qi_sn;
   const int64_t kidx_off = b * p.ki_sb + hk * p.ki_sh + (int64_t)seg * p.n_k * p.ki_sn;
@@ -364,7 +374,7 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
   };
   auto fetch_rows = [&](int ci, int kk0, RowSource& rs) {
     const unsigned char* src = nullptr;  // index array run, or null for consecutive rows
-    int64_t stride = 0;
+    uint32_t stride = 0;                 // bytes between its entries
     int first = 0;
     if (GATHER) {
       if (ci < n_blk_chunks) {
@@ -372,12 +382,12 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
         u -= u >= nk_chunks ? nk_chunks : 0;
         u -= u >= nk_chunks ? nk_chunks : 0;
         src = (const unsigned char*)p.k_idx + ((kidx_off + (int64_t)u * KC * p.ki_sn) << idx_shift);
-        stride = p.ki_sn << idx_shift;
+        stride = (uint32_t)p.ki_sn << idx_shift;
       } else {
         first = (ci - n_blk_chunks) * KC;
         if (p.sampled_idx) {
           src = (const unsigned char*)p.sampled_idx + ((sidx_off + first) << idx_shift);
-          stride = (int64_t)1 << idx_shift;
+          stride = 1u << idx_shift;
         }
       }
     } else {
@@ -389,7 +399,7 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
       rs.first = ROWS_LOADED;
 #pragma unroll
       for (int j = 0; j < LPW; ++j)
-        rs.rows[j] = *reinterpret_cast<const int*>(src + (kk0 + j * ROWS_PER_LOAD + my_lr) * stride);
+        rs.rows[j] = *reinterpret_cast<const int*>(row_address(src, kk0 + j * ROWS_PER_LOAD + my_lr, stride, 0));
     } else {
       rs.first = first;
     }
@@ -408,8 +418,7 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
     if (!GATHER && row >= p.n_k) row = 0;                                                                \
     if (GATHER && rs.first == ROWS_LOADED) row = rs.rows[j];                                             \
     if (rs.first == ROWS_NONE) row = 0;                                                                  \
-    const T* src = (base) + (int64_t)row * (stride) + ((my_pp ^ (r & 7)) << 3);                          \
-    global_to_lds_16(src, (tile) + (wave * LPW + j) * 1024);                                             \
+    global_to_lds_16(row_address(base, row, stride, (my_pp ^ (r & 7)) << 4), (tile) + (wave * LPW + j) * 1024); \
   }
 
   // ---- first loads: row numbers of the queries and of the first key tiles, then the rows ----------
@@ -418,6 +427,9 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
 #pragma unroll
   for (int j = 0; j < LPW; ++j) rows_k.rows[j] = rows_v.rows[j] = 0;
   int qrow[2];  // original row of the query a lane's S^T / O^T columns belong to
+  // sorted query positions of this head: entries of 4 or 8 bytes, the row number in the low word
+  const unsigned char* const q_idx_base = (const unsigned char*)p.q_idx + (qidx_off << idx_shift);
+  const uint32_t qi_rb = (uint32_t)p.qi_sn << idx_shift;
   {
     int q_rows[PR];  // rows of this wave's query tile, in the order of its PR loads
 #pragma unroll
@@ -425,12 +437,12 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
       // positions past the end load the index of position 0 (replaced by -1 below, once all the
       // index loads of this prologue are in flight)
       const int pq = wave_q_first + j * ROWS_PER_LOAD + my_lr;
-      q_rows[j] = GATHER ? ha_load_idx(p.q_idx, qidx_off + (int64_t)(pq < p.n_q ? pq : 0) * p.qi_sn, p.idx64) : pq;
+      q_rows[j] = GATHER ? *reinterpret_cast<const int*>(row_address(q_idx_base, pq < p.n_q ? pq : 0, qi_rb, 0)) : pq;
     }
 #pragma unroll
     for (int nb = 0; nb < 2; ++nb) {
       const int pq = wave_q_first + nb * 32 + col;
-      qrow[nb] = GATHER ? ha_load_idx(p.q_idx, qidx_off + (int64_t)(pq < p.n_q ? pq : 0) * p.qi_sn, p.idx64) : pq;
+      qrow[nb] = GATHER ? *reinterpret_cast<const int*>(row_address(q_idx_base, pq < p.n_q ? pq : 0, qi_rb, 0)) : pq;
     }
     RowSource rows_k1;
 #pragma unroll
@@ -444,17 +456,16 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
 #pragma unroll
     for (int nb = 0; nb < 2; ++nb)
       if (wave_q_first + nb * 32 + col >= p.n_q) qrow[nb] = -1;
-    HA_LOAD_TILE(kb, p.k_sn, rows_k, k_kk0, lds_k0)
+    HA_LOAD_TILE(kb, k_rb, rows_k, k_kk0, lds_k0)
 #pragma unroll
     for (int j = 0; j < PR; ++j) {
       // positions past the end read row 0 (finite data; their results are never written)
       const int r = j * ROWS_PER_LOAD + my_lr;
-      const T* src = qb + (int64_t)(q_rows[j] < 0 ? 0 : q_rows[j]) * p.q_sn + ((my_pp ^ (r & 7)) << 3);
-      global_to_lds_16(src, my_q + j * 1024);
+      global_to_lds_16(row_address(qb, q_rows[j] < 0 ? 0 : q_rows[j], q_rb, (my_pp ^ (r & 7)) << 4), my_q + j * 1024);
       if (my_pp == 0) lds_qrow[wave * 64 + r] = q_rows[j];
     }
-    HA_LOAD_TILE(vb, p.v_sn, rows_v, v_kk0, lds_v0)
-    HA_LOAD_TILE(kb, p.k_sn, rows_k1, k_kk0, lds_k1)
+    HA_LOAD_TILE(vb, v_rb, rows_v, v_kk0, lds_v0)
+    HA_LOAD_TILE(kb, k_rb, rows_k1, k_kk0, lds_k1)
   }
   HA_FETCH_ROWS_K(2, rows_k)
   HA_FETCH_ROWS_V(1, rows_v)
@@ -566,8 +577,8 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
       acc[db][nb] = Mfma<T>::run(vf[db], pb[nb], acc[db][nb]);
 #define HA_ITERATION(ci, K_RD, K_WR, V_CUR, V_WR)                                                           \
   {                                                                                                         \
-    if ((ci) + 2 <= n_chunks) { HA_LOAD_TILE(kb, p.k_sn, rows_k, k_kk0, K_WR) } /* K tile ci+2 */           \
-    if ((ci) + 1 < n_chunks) { HA_LOAD_TILE(vb, p.v_sn, rows_v, v_kk0, V_WR) }  /* V tile ci+1 */           \
+    if ((ci) + 2 <= n_chunks) { HA_LOAD_TILE(kb, k_rb, rows_k, k_kk0, K_WR) } /* K tile ci+2 */             \
+    if ((ci) + 1 < n_chunks) { HA_LOAD_TILE(vb, v_rb, rows_v, v_kk0, V_WR) }  /* V tile ci+1 */             \
     HA_FETCH_ROWS_K((ci) + 3, rows_k)                                                                       \
     HA_FETCH_ROWS_V((ci) + 2, rows_v)                                                                       \
     /* causal: once a chunk lies wholly above this wave's queries, so do all later ones */                  \
@@ -612,7 +623,7 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
 #pragma unroll
     for (int j = 0; j < OUT_PIECES; ++j) {
       prev[j] = vec8{};
-      if (out_row[j] >= 0) prev[j] = *reinterpret_cast<const vec8*>(ob + (int64_t)out_row[j] * p.o_sn + my_pp * 8);
+      if (out_row[j] >= 0) prev[j] = *reinterpret_cast<const vec8*>(row_address(ob, out_row[j], o_rb, my_pp * 16));
     }
   }
   T* const lds_o = reinterpret_cast<T*>(my_q);
@@ -649,7 +660,7 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
 #pragma unroll
         for (int e = 0; e < 8; ++e) o[e] = (T)__builtin_fmaf(w, (float)prev[j][e], (float)o[e]);
       }
-      *reinterpret_cast<vec8*>(ob + (int64_t)out_row[j] * p.o_sn + my_pp * 8) = o;
+      *reinterpret_cast<vec8*>(const_cast<unsigned char*>(row_address(ob, out_row[j], o_rb, my_pp * 16))) = o;
     }
   }
 #undef HA_FETCH_ROWS_K
