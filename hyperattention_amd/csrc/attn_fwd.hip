@@ -283,6 +283,9 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
 
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63;
+  // the same number, known to the compiler to be wave-uniform: what the tile loads derive from it
+  // (chunk numbers, index array addresses, LDS destinations) then stays in scalar registers
+  const int wave_s = __builtin_amdgcn_readfirstlane(wave);
   const int hi = lane >> 5, col = lane & 31;
 
   // ---- which (virtual) head and query tile -----------------------------------------------------
@@ -332,8 +335,8 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
     uni_start = start[0];
     const int uni_end = end[1] > end[0] ? end[1] : end[0];
     n_blk_chunks = uni_end - uni_start;
-    my_lo = start[wave >> 1];
-    my_hi = end[wave >> 1];
+    my_lo = start[wave_s >> 1];
+    my_hi = end[wave_s >> 1];
     n_chunks = n_blk_chunks + p.sample_chunks;
   } else {
     int kend = p.n_k;
@@ -406,19 +409,19 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
   };
   // V tile c holds keys 0..63 of chunk c.  K tile c holds keys 32..63 of chunk c-1 in its rows 0..31
   // and keys 0..31 of chunk c in its rows 32..63: waves 0,1 load the former, waves 2,3 the latter.
-  const int v_kk0 = wave * (LPW * ROWS_PER_LOAD);
+  const int v_kk0 = wave_s * (LPW * ROWS_PER_LOAD);
   const int k_kk0 = (v_kk0 + 32) & 63;
-  const int k_chunk_shift = (wave >> 1) - 1;
+  const int k_chunk_shift = (wave_s >> 1) - 1;
 #define HA_FETCH_ROWS_K(tile_c, rs) fetch_rows((tile_c) + k_chunk_shift, k_kk0, rs);
 #define HA_FETCH_ROWS_V(ci, rs) fetch_rows((ci), v_kk0, rs);
 #define HA_LOAD_TILE(base, stride, rs, kk0, tile)                                                        \
   _Pragma("unroll") for (int j = 0; j < LPW; ++j) {                                                      \
-    const int r = (wave * LPW + j) * ROWS_PER_LOAD + my_lr;                                              \
+    const int r = (wave_s * LPW + j) * ROWS_PER_LOAD + my_lr;                                            \
     int row = rs.first + (kk0) + j * ROWS_PER_LOAD + my_lr; /* consecutive rows */                       \
     if (!GATHER && row >= p.n_k) row = 0;                                                                \
     if (GATHER && rs.first == ROWS_LOADED) row = rs.rows[j];                                             \
     if (rs.first == ROWS_NONE) row = 0;                                                                  \
-    global_to_lds_16(row_address(base, row, stride, (my_pp ^ (r & 7)) << 4), (tile) + (wave * LPW + j) * 1024); \
+    global_to_lds_16(row_address(base, row, stride, (my_pp ^ (r & 7)) << 4), (tile) + (wave_s * LPW + j) * 1024); \
   }
 
   // ---- first loads: row numbers of the queries and of the first key tiles, then the rows ----------
