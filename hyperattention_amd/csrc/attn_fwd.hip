@@ -625,8 +625,8 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
   if (p.accumulate) {
 #pragma unroll
     for (int j = 0; j < OUT_PIECES; ++j) {
-      prev[j] = vec8{};
-      if (out_row[j] >= 0) prev[j] = *reinterpret_cast<const vec8*>(row_address(ob, out_row[j], o_rb, my_pp * 16));
+      // positions past the end read row 0 (never written back): an unconditional load needs no zero fill
+      prev[j] = *reinterpret_cast<const vec8*>(row_address(ob, out_row[j] < 0 ? 0 : out_row[j], o_rb, my_pp * 16));
     }
   }
   T* const lds_o = reinterpret_cast<T*>(my_q);
