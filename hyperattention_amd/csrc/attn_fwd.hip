@@ -102,10 +102,20 @@ struct LaneOffsets {
   int v[D / 32];  // V^T operand word for dv block db, keys 0..3 (+4 for the upper lane half) of a 16-key half-step
 };
 
-// 16-byte piece `piece` of row `row` of a row-major [rows][D] 2-byte tile, XOR-swizzled; byte offset
+// 16-byte piece `piece` of row `row` of a row-major [rows][D] 2-byte tile, XOR-swizzled; byte offset.
+// Q and K tiles (read 16 bytes per lane, 8 consecutive rows at a time) move a piece by the row number
+// mod 8.  V tiles are read by the transposing loads, 16 lanes at a time: 4 consecutive rows x 32
+// bytes; they move a PAIR of pieces by the row number mod 4, so that the four rows fall into four
+// different 32-byte bank groups.
+__device__ __forceinline__ int k_swizzle(int row) { return row & 7; }
+__device__ __forceinline__ int v_swizzle(int row) { return (row & 3) << 1; }
 template <int D>
 __device__ __forceinline__ int tile_offset(int row, int piece) {
-  return row * D * 2 + ((piece ^ (row & 7)) << 4);
+  return row * D * 2 + ((piece ^ k_swizzle(row)) << 4);
+}
+template <int D>
+__device__ __forceinline__ int v_tile_offset(int row, int piece) {
+  return row * D * 2 + ((piece ^ v_swizzle(row)) << 4);
 }
 
 template <typename T>
@@ -414,14 +424,14 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
   const int k_chunk_shift = (wave_s >> 1) - 1;
 #define HA_FETCH_ROWS_K(tile_c, rs) fetch_rows((tile_c) + k_chunk_shift, k_kk0, rs);
 #define HA_FETCH_ROWS_V(ci, rs) fetch_rows((ci), v_kk0, rs);
-#define HA_LOAD_TILE(base, stride, rs, kk0, tile)                                                        \
+#define HA_LOAD_TILE(base, stride, rs, kk0, tile, SWZ)                                                   \
   _Pragma("unroll") for (int j = 0; j < LPW; ++j) {                                                      \
     const int r = (wave_s * LPW + j) * ROWS_PER_LOAD + my_lr;                                            \
     int row = rs.first + (kk0) + j * ROWS_PER_LOAD + my_lr; /* consecutive rows */                       \
     if (!GATHER && row >= p.n_k) row = 0;                                                                \
     if (GATHER && rs.first == ROWS_LOADED) row = rs.rows[j];                                             \
     if (rs.first == ROWS_NONE) row = 0;                                                                  \
-    global_to_lds_16(row_address(base, row, stride, (my_pp ^ (r & 7)) << 4), (tile) + (wave_s * LPW + j) * 1024); \
+    global_to_lds_16(row_address(base, row, stride, (my_pp ^ SWZ(r)) << 4), (tile) + (wave_s * LPW + j) * 1024); \
   }
 
   // ---- first loads: row numbers of the queries and of the first key tiles, then the rows ----------
@@ -459,7 +469,7 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
 #pragma unroll
     for (int nb = 0; nb < 2; ++nb)
       if (wave_q_first + nb * 32 + col >= p.n_q) qrow[nb] = -1;
-    HA_LOAD_TILE(kb, k_rb, rows_k, k_kk0, lds_k0)
+    HA_LOAD_TILE(kb, k_rb, rows_k, k_kk0, lds_k0, k_swizzle)
 #pragma unroll
     for (int j = 0; j < PR; ++j) {
       // positions past the end read row 0 (finite data; their results are never written)
@@ -467,8 +477,8 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
       global_to_lds_16(row_address(qb, q_rows[j] < 0 ? 0 : q_rows[j], q_rb, (my_pp ^ (r & 7)) << 4), my_q + j * 1024);
       if (my_pp == 0) lds_qrow[wave * 64 + r] = q_rows[j];
     }
-    HA_LOAD_TILE(vb, v_rb, rows_v, v_kk0, lds_v0)
-    HA_LOAD_TILE(kb, k_rb, rows_k1, k_kk0, lds_k1)
+    HA_LOAD_TILE(vb, v_rb, rows_v, v_kk0, lds_v0, v_swizzle)
+    HA_LOAD_TILE(kb, k_rb, rows_k1, k_kk0, lds_k1, k_swizzle)
   }
   HA_FETCH_ROWS_K(2, rows_k)
   HA_FETCH_ROWS_V(1, rows_v)
@@ -505,7 +515,7 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
     const int w = sl & 3;
 #pragma unroll
     for (int db = 0; db < DB; ++db)
-      lo.v[db] = tile_offset<D>(key, db * 4 + (g & 1) * 2 + (w >> 1)) + (w & 1) * 8;
+      lo.v[db] = v_tile_offset<D>(key, db * 4 + (g & 1) * 2 + (w >> 1)) + (w & 1) * 8;
   }
 
   // every wave's part of Q, K tile 0, V tile 0, K tile 1 has landed before anyone reads the tiles
@@ -580,8 +590,8 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
       acc[db][nb] = Mfma<T>::run(vf[db], pb[nb], acc[db][nb]);
 #define HA_ITERATION(ci, K_RD, K_WR, V_CUR, V_WR)                                                           \
   {                                                                                                         \
-    if ((ci) + 2 <= n_chunks) { HA_LOAD_TILE(kb, k_rb, rows_k, k_kk0, K_WR) } /* K tile ci+2 */             \
-    if ((ci) + 1 < n_chunks) { HA_LOAD_TILE(vb, v_rb, rows_v, v_kk0, V_WR) }  /* V tile ci+1 */             \
+    if ((ci) + 2 <= n_chunks) { HA_LOAD_TILE(kb, k_rb, rows_k, k_kk0, K_WR, k_swizzle) } /* K tile ci+2 */  \
+    if ((ci) + 1 < n_chunks) { HA_LOAD_TILE(vb, v_rb, rows_v, v_kk0, V_WR, v_swizzle) }  /* V tile ci+1 */  \
     HA_FETCH_ROWS_K((ci) + 3, rows_k)                                                                       \
     HA_FETCH_ROWS_V((ci) + 2, rows_v)                                                                       \
     /* causal: once a chunk lies wholly above this wave's queries, so do all later ones */                  \
