@@ -137,3 +137,14 @@ def test_python_layer_fails_loudly_without_library(monkeypatch, tmp_path):
     monkeypatch.setattr(_lib, "_lib", None)
     with pytest.raises(RuntimeError, match="no fallback"):
         _lib.lib()
+
+
+def test_sweep_script_command_line():
+    """The sweep keeps the reference's options (benchmark_single_attention.py:14-22); the modes that
+    need a backward pass stop before touching the GPU."""
+    from hyperattention_amd import benchmark_single_attention as sweep
+    args = sweep.get_arguments(["--no_causal", "--smooth_block", "--mode", "fwd", "--attn_method", "hyper"])
+    assert args.no_causal and args.smooth_block and args.mode == "fwd" and args.attn_method == "hyper"
+    for mode in ("bwd", "fwd+bwd"):
+        with pytest.raises(SystemExit):
+            sweep.main(["--mode", mode, "--attn_method", "hyper"])
