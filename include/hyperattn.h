@@ -91,6 +91,8 @@ int ha_gather_rows(const void* x, const void* idx, int idx_type, void* out,
  * k_seg_offset + g*seg_stride_rows.  This is the halves-as-heads view of hyper_attention.py:67-69
  * and the half slicing of :82-84 expressed as index arithmetic.  segs == 1 with zero offsets is the
  * plain case.
+ * Limits (HA_ERR_SHAPE / HA_ERR_UNSUPPORTED otherwise): n_q, n_k < 2^24; row strides positive, multiples
+ * of 8 elements and below 16 MiB; (n - 1) rows of one head within 4 GiB; tensors 16-byte aligned.
  */
 typedef struct {
   const void* q;
