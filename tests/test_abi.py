@@ -98,9 +98,16 @@ def test_attention_argument_errors(lib):
     assert lib.ha_flash_attn_fwd(ctypes.byref(_operands(d=32, dv=32)), 0, None) == -5
     assert lib.ha_flash_attn_fwd(ctypes.byref(_operands(scale=0.0)), 0, None) == -3
     assert lib.ha_flash_attn_fwd(ctypes.byref(_operands(q_stride_n=60)), 0, None) == -3
+    # addressing limits: 2^24 rows, row strides below 16 MiB, one head within 4 GiB
+    assert lib.ha_flash_attn_fwd(ctypes.byref(_operands(n_k=1 << 24)), 0, None) == -3
+    assert lib.ha_flash_attn_fwd(ctypes.byref(_operands(k_stride_n=1 << 23)), 0, None) == -5
+    assert lib.ha_flash_attn_fwd(ctypes.byref(_operands(n_q=1 << 20, q_stride_n=4096)), 0, None) == -5
+    assert b"4 GiB" in lib.ha_last_error()
+    assert lib.ha_flash_attn_fwd(ctypes.byref(_operands(v_stride_n=-64)), 0, None) == -5
     a = _lib.BlockAttnArgs()
     a.t = _operands()
     a.q_idx = a.k_idx = 16
+    a.q_idx_stride_n = a.k_idx_stride_n = 1
     a.block_size, a.sample_size = 256, 100
     assert lib.ha_block_attn_fwd(ctypes.byref(a), None) == -3  # sample_size % 128
     a.sample_size = 0
@@ -108,6 +115,9 @@ def test_attention_argument_errors(lib):
     assert lib.ha_block_attn_fwd(ctypes.byref(a), None) == -3
     assert b"divisible by 128" in lib.ha_last_error()
     a.t = _operands()
+    a.k_idx_stride_n = 0
+    assert lib.ha_block_attn_fwd(ctypes.byref(a), None) == -5
+    a.k_idx_stride_n = 1
     a.q_idx = None
     assert lib.ha_block_attn_fwd(ctypes.byref(a), None) == -1
 
