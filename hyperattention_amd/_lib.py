@@ -106,6 +106,9 @@ class ForwardArgs(ctypes.Structure):
         ("smooth_block", ctypes.c_int), ("causal", ctypes.c_int),
         ("scale", ctypes.c_float), ("dtype", ctypes.c_int),
         ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_int64),
+        ("q_stride_b", ctypes.c_int64), ("q_stride_h", ctypes.c_int64), ("q_stride_n", ctypes.c_int64),
+        ("k_stride_b", ctypes.c_int64), ("k_stride_h", ctypes.c_int64), ("k_stride_n", ctypes.c_int64),
+        ("v_stride_b", ctypes.c_int64), ("v_stride_h", ctypes.c_int64), ("v_stride_n", ctypes.c_int64),
     ]
 
 
@@ -148,7 +151,7 @@ def lib():
                 "(hipcc, gfx950). There is no fallback path.")
         loaded = ctypes.CDLL(LIB_PATH)
         _declare(loaded)
-        if loaded.ha_abi_version() != 1:
+        if loaded.ha_abi_version() != 2:
             raise RuntimeError("libhyperattn.so: ABI version mismatch")
         _lib = loaded
     return _lib

@@ -239,7 +239,7 @@ extern "C" int ha_forward(const ha_forward_args* args, void* stream_) {
   unsigned char* ws = (unsigned char*)a.workspace;
   const int64_t group = a.heads / a.kv_heads;
 
-  // operands shared by every launch: contiguous (batch, heads, n, d) tensors
+  // operands shared by every launch: (batch, heads, n, d) tensors, contiguous unless strides are given
   ha_attn_operands t;
   t.q = a.q; t.k = a.k; t.v = a.v; t.out = a.out; t.lse = a.lse;
   t.batch = a.batch; t.heads = a.heads; t.d = a.d; t.dv = a.dv;
@@ -247,6 +247,15 @@ extern "C" int ha_forward(const ha_forward_args* args, void* stream_) {
   t.k_stride_b = a.kv_heads * a.n * a.d; t.k_stride_h = a.n * a.d; t.k_stride_n = a.d;
   t.v_stride_b = a.kv_heads * a.n * a.dv; t.v_stride_h = a.n * a.dv; t.v_stride_n = a.dv;
   t.o_stride_b = a.heads * a.n * a.dv; t.o_stride_h = a.n * a.dv; t.o_stride_n = a.dv;
+  if (a.q_stride_b || a.q_stride_h || a.q_stride_n) {
+    t.q_stride_b = a.q_stride_b; t.q_stride_h = a.q_stride_h; t.q_stride_n = a.q_stride_n;
+  }
+  if (a.k_stride_b || a.k_stride_h || a.k_stride_n) {
+    t.k_stride_b = a.k_stride_b; t.k_stride_h = a.k_stride_h; t.k_stride_n = a.k_stride_n;
+  }
+  if (a.v_stride_b || a.v_stride_h || a.v_stride_n) {
+    t.v_stride_b = a.v_stride_b; t.v_stride_h = a.v_stride_h; t.v_stride_n = a.v_stride_n;
+  }
   t.lse_stride_b = a.heads * a.n; t.lse_stride_h = a.n;
   t.kv_group = group;
   t.scale = a.scale;

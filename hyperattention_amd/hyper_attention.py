@@ -47,9 +47,8 @@ class HyperAttention(torch.nn.Module):
             - attn: (approximation of) the attention output (batch, heads, seq_len, dim_v)
             - lse: (approximation of) log-sum-exp of the scaled qk matrix, (batch, heads, seq_len, 1)
         """
-        query = query.contiguous()
-        key = key.contiguous()
-        value = value.contiguous()
+        # permuted views (e.g. (sq, b, np, hn) tensors seen as (b, np, sq, hn)) are read in place
+        query, key, value = [x if x.stride(-1) == 1 else x.contiguous() for x in (query, key, value)]
 
         n_query = query.shape[2]
         batch_size, n_heads, n_key, dim = key.shape
@@ -68,7 +67,7 @@ class HyperAttention(torch.nn.Module):
             else:
                 lse = lse.unsqueeze(-1)
         else:
-            attn, lse = self._forward_composed(query, key, value, scale, causal)
+            attn, lse = self._forward_composed(query.contiguous(), key.contiguous(), value.contiguous(), scale, causal)
 
         if not return_lse:
             return attn

@@ -237,9 +237,10 @@ def forward_plan_supported(n: int, min_seq_len: int, causal: bool, lsh_num_projs
 
 def hyper_forward(q, k, v, proj, *, scale, causal, lsh_num_projs, block_size, sample_size, min_seq_len,
                   smooth_block, sampled_idx=None):
-    """One-call forward for contiguous (b,h,n,d) q and (b,h_kv,n,d) k, v.  Returns out (b,h,n,dv) and
-    lse (b,h,n) fp32."""
-    assert q.is_cuda and k.is_cuda and v.is_cuda and q.is_contiguous() and k.is_contiguous() and v.is_contiguous()
+    """One-call forward for (b,h,n,d) q and (b,h_kv,n,d) k, v of any strides with a contiguous last
+    dimension (permuted views are read in place).  Returns contiguous out (b,h,n,dv) and lse (b,h,n) fp32."""
+    assert q.is_cuda and k.is_cuda and v.is_cuda
+    assert q.stride(-1) == 1 and k.stride(-1) == 1 and v.stride(-1) == 1
     assert q.dtype == k.dtype == v.dtype, "All tensors must have the same type"
     b, h, n, d = q.shape
     hk = k.shape[1]
@@ -263,6 +264,9 @@ def hyper_forward(q, k, v, proj, *, scale, causal, lsh_num_projs, block_size, sa
     a.smooth_block, a.causal = int(bool(smooth_block)), int(bool(causal))
     a.scale = scale
     a.dtype = _dtype_code(q)
+    a.q_stride_b, a.q_stride_h, a.q_stride_n = q.stride(0), q.stride(1), q.stride(2)
+    a.k_stride_b, a.k_stride_h, a.k_stride_n = k.stride(0), k.stride(1), k.stride(2)
+    a.v_stride_b, a.v_stride_h, a.v_stride_n = v.stride(0), v.stride(1), v.stride(2)
     L = _lib.lib()
     ws_bytes = L.ha_forward_workspace_bytes(ctypes.byref(a))
     if ws_bytes < 0:

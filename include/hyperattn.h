@@ -21,7 +21,7 @@
 extern "C" {
 #endif
 
-#define HA_ABI_VERSION 1
+#define HA_ABI_VERSION 2
 
 typedef enum {
   HA_OK = 0,
@@ -158,7 +158,7 @@ int ha_lse_merge(const void* attn1, const float* lse1, const void* attn2, const 
                  int dtype, void* stream);
 
 /* ---------------------------------------------------------------------------------------------
- * Whole forward pass of the module for contiguous (batch, heads, n, d) tensors, one call, no host
+ * Whole forward pass of the module for (batch, heads, n, d) tensors, one call, no host
  * synchronisation and no tensor copies.
  * replaces: HyperAttention.forward / forward_no_causal_mask (hyper_attention.py:25-132) for the
  * shapes where every recursion level has an even length (n = leaf_len * 2^levels); other shapes
@@ -167,6 +167,9 @@ int ha_lse_merge(const void* attn1, const float* lse1, const void* attn2, const 
  * sample_size rows), shared by all heads and levels.  out (batch,heads,n,dv) dtype, lse
  * (batch,heads,n) fp32.  kv_heads divides heads (grouped-query: q head h reads kv head
  * h / (heads/kv_heads)); k and v are (batch, kv_heads, n, d).
+ * q/k/v strides in elements, last dim contiguous; a tensor whose three strides are all zero is
+ * contiguous.  This takes the permuted views of the reference's callers
+ * (chatglm_fast_attention.py:42-58: (sq, b, np, hn) tensors seen as (b, np, sq, hn)) without a copy.
  */
 typedef struct {
   const void* q;
@@ -184,6 +187,9 @@ typedef struct {
   int dtype;
   void* workspace;
   int64_t workspace_bytes;
+  int64_t q_stride_b, q_stride_h, q_stride_n;
+  int64_t k_stride_b, k_stride_h, k_stride_n;
+  int64_t v_stride_b, v_stride_h, v_stride_n;
 } ha_forward_args;
 
 int64_t ha_forward_workspace_bytes(const ha_forward_args* args);

@@ -32,7 +32,7 @@ def test_every_declared_symbol_is_exported(lib):
     assert declared == sorted(_lib.SYMBOLS)
     for name in declared:
         assert hasattr(lib, name), f"{name} declared in hyperattn.h but not exported"
-    assert lib.ha_abi_version() == 1
+    assert lib.ha_abi_version() == 2
 
 
 def test_struct_layouts_match_the_header(tmp_path):
@@ -46,7 +46,8 @@ int main(void) {
   printf("%zu %zu %zu\n", sizeof(ha_attn_operands), sizeof(ha_block_attn_args), sizeof(ha_forward_args));
   printf("%zu %zu %zu\n", offsetof(ha_attn_operands, scale), offsetof(ha_block_attn_args, accumulate),
          offsetof(ha_forward_args, workspace_bytes));
-  printf("%zu %zu\n", offsetof(ha_block_attn_args, q_idx), offsetof(ha_forward_args, scale));
+  printf("%zu %zu %zu\n", offsetof(ha_block_attn_args, q_idx), offsetof(ha_forward_args, scale),
+         offsetof(ha_forward_args, v_stride_n));
   return 0;
 }''')
     exe = tmp_path / "layout"
@@ -55,7 +56,8 @@ int main(void) {
     got = [int(x) for x in out]
     want = [ctypes.sizeof(_lib.AttnOperands), ctypes.sizeof(_lib.BlockAttnArgs), ctypes.sizeof(_lib.ForwardArgs),
             _lib.AttnOperands.scale.offset, _lib.BlockAttnArgs.accumulate.offset,
-            _lib.ForwardArgs.workspace_bytes.offset, _lib.BlockAttnArgs.q_idx.offset, _lib.ForwardArgs.scale.offset]
+            _lib.ForwardArgs.workspace_bytes.offset, _lib.BlockAttnArgs.q_idx.offset, _lib.ForwardArgs.scale.offset,
+            _lib.ForwardArgs.v_stride_n.offset]
     assert got == want
 
 

@@ -115,6 +115,21 @@ def test_causal_composed_path_equals_fused_path(ha):
     assert_close(lse_c, lse_f, "composed vs fused lse")
 
 
+@pytest.mark.parametrize("causal", [False, True])
+def test_permuted_views_are_read_in_place(ha, causal):
+    """(sq, b, np, hn) tensors seen as (b, np, sq, hn), the layout of the reference's ChatGLM caller
+    (chatglm_fast_attention.py:42-58), and grouped-query k/v: same bits as from contiguous copies."""
+    n, b, h, hk, d = 2048, 2, 4, 2, 64
+    q_s = _randn((n, b, h, d), 170, torch.float16).cuda()
+    k_s, v_s = (_randn((n, b, hk, d), s, torch.float16).cuda() for s in (171, 172))
+    q, k, v = (x.permute(1, 2, 0, 3) for x in (q_s, k_s, v_s))
+    assert not q.is_contiguous()
+    m, _ = _module(ha, d, torch.float16, 173, min_seq_len=512)
+    got, lse = m(q, k, v, causal=causal, return_lse=True)
+    want, wlse = m(q.contiguous(), k.contiguous(), v.contiguous(), causal=causal, return_lse=True)
+    assert got.is_contiguous() and torch.equal(got, want) and torch.equal(lse, wlse)
+
+
 def test_module_argument_errors(ha):
     m, _ = _module(ha, 64, torch.float16, 160)
     q = torch.zeros((1, 1, 256, 64), dtype=torch.float16, device="cuda")
