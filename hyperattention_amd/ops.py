@@ -139,6 +139,19 @@ def hyper_attn_func(q, k, v, q_sort_idx, k_sort_idx, block_size, sample_size=0, 
     which equals add_self_attentions(previous, this call) in fp32."""
     q, k, v = [x if x.stride(-1) == 1 else x.contiguous() for x in [q, k, v]]
     assert sample_size % 128 == 0
+    if v.shape[-1] != q.shape[-1]:
+        # A value head dim different from the q/k head dim (src/hyper_attn_triton.py:679,692-693;
+        # unit_tests/test_hyper_attention.py:120-133).  The kernels are built for equal dims, so the
+        # narrower side is zero-padded (zero columns change neither q.k nor the wanted columns of the
+        # output) and the output is cut back: correct, at the price of the padded copies.
+        assert resume is None, "resume needs equal head dims"
+        d_qk, d_v = q.shape[-1], v.shape[-1]
+        assert d_qk <= 128 and d_v <= 128, "FlashAttention only support head dimensions up to 128"
+        wide = max(d_qk, d_v)
+        pad = lambda x: torch.nn.functional.pad(x, (0, wide - x.shape[-1]))
+        o, lse = hyper_attn_func(pad(q), pad(k), pad(v), q_sort_idx, k_sort_idx, block_size, sample_size,
+                                 softmax_scale or 1.0 / math.sqrt(d_qk), smooth_block, sampled_idx=sampled_idx)
+        return o[..., :d_v], lse
     batch, seqlen_q, nheads, d = q.shape
     _, seqlen_k, _, _ = k.shape
     assert k.shape == (batch, seqlen_k, nheads, d)

@@ -258,6 +258,22 @@ def test_block_attention_resumes_partial_result(ha, dtype, shift):
     assert_close(lse, want_lse, "resumed lse")
 
 
+def test_block_attention_value_dim_differs(ha):
+    """unit_tests/test_hyper_attention.py:120-133: V narrower than Q and K gives the matching columns
+    of the full-width result; the other way round (wider V) follows from the same definition."""
+    b, h, n, d = 1, 2, 1024, 128
+    q, k, v, qi, ki = _sorted_inputs(b, h, n, d, torch.bfloat16, 80)
+    full, lse_full = _run_hyper(ha, q, k, v, qi, ki, 256, 128, None, False)
+    small, lse_small = _run_hyper(ha, q, k, v[..., :d // 2].clone(), qi, ki, 256, 128, None, False)
+    assert small.shape == (b, h, n, d // 2)
+    assert torch.equal(small, full[..., :d // 2]) and torch.equal(lse_small, lse_full)
+    wide, lse_wide = _run_hyper(ha, q[..., :64].clone(), k[..., :64].clone(), v, qi, ki, 256, 128, None, False)
+    ro, rl = O.block_sampled_attention(q[..., :64], k[..., :64], v, qi, ki, 256, 128, None, False)
+    assert wide.shape == (b, h, n, d)
+    assert_close(wide, ro, "wide-v out", torch.bfloat16)
+    assert_close(lse_wide, rl, "wide-v lse")
+
+
 def test_block_attention_argument_errors(ha):
     z = torch.zeros((1, 256, 1, 64), dtype=torch.float16, device="cuda")
     idx = torch.arange(256, device="cuda").view(1, 256, 1)
