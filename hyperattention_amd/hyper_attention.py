@@ -55,6 +55,22 @@ class HyperAttention(torch.nn.Module):
         scale = scale or dim ** (-0.5)
         assert n_query == n_key
 
+        dim_v = value.shape[-1]
+        if dim not in ops.KERNEL_HEAD_DIMS or dim_v != dim:
+            # head dims the kernels are not built for (and a value dim different from the q/k dim) run
+            # zero-padded: zero columns change neither the projections, nor q.k, nor the wanted outputs
+            assert dim <= 128 and dim_v <= 128, "FlashAttention only support head dimensions up to 128"
+            wide = ops.padded_head_dim(max(dim, dim_v))
+            pad = lambda x: torch.nn.functional.pad(x, (0, wide - x.shape[-1]))
+            proj = self.lsh.proj_dir
+            self.lsh.proj_dir = torch.nn.functional.pad(proj, (0, 0, 0, wide - dim))
+            try:
+                res = self.forward(pad(query), pad(key), pad(value), scale, causal, True)
+            finally:
+                self.lsh.proj_dir = proj
+            attn, lse = res[0][..., :dim_v], res[1]
+            return (attn, lse) if return_lse else attn
+
         if ops.forward_plan_supported(n_key, self.min_seq_len, causal is not False, self.lsh_num_projs):
             attn, lse = ops.hyper_forward(
                 query, key, value, self.lsh.proj_dir, scale=scale, causal=causal is not False,

@@ -128,6 +128,14 @@ def _operands(q, k, v, out, lse, scale, *, layout_bnhd: bool, lse_row_stride: in
     return t
 
 
+KERNEL_HEAD_DIMS = (64, 128)  # head dims the attention kernels are built for
+
+
+def padded_head_dim(d):
+    """The built head dim that a head dim d <= 128 is zero-padded to."""
+    return 64 if d <= 64 else 128
+
+
 def hyper_attn_func(q, k, v, q_sort_idx, k_sort_idx, block_size, sample_size=0, softmax_scale=None,
                     smooth_block=False, *, sampled_idx=None, resume=None):
     """q, k: (batch, seqlen, nheads, headdim); v: (batch, seqlen, nheads, v_headdim);
@@ -139,15 +147,15 @@ def hyper_attn_func(q, k, v, q_sort_idx, k_sort_idx, block_size, sample_size=0, 
     which equals add_self_attentions(previous, this call) in fp32."""
     q, k, v = [x if x.stride(-1) == 1 else x.contiguous() for x in [q, k, v]]
     assert sample_size % 128 == 0
-    if v.shape[-1] != q.shape[-1]:
+    if v.shape[-1] != q.shape[-1] or q.shape[-1] not in KERNEL_HEAD_DIMS:
         # A value head dim different from the q/k head dim (src/hyper_attn_triton.py:679,692-693;
-        # unit_tests/test_hyper_attention.py:120-133).  The kernels are built for equal dims, so the
-        # narrower side is zero-padded (zero columns change neither q.k nor the wanted columns of the
-        # output) and the output is cut back: correct, at the price of the padded copies.
-        assert resume is None, "resume needs equal head dims"
+        # unit_tests/test_hyper_attention.py:120-133), or a head dim the kernels are not built for.
+        # Zero columns change neither q.k nor the wanted columns of the output, so both sides are
+        # zero-padded to a built width and the output is cut back: exact, at the price of the copies.
+        assert resume is None, "resume needs a head dim the kernels are built for"
         d_qk, d_v = q.shape[-1], v.shape[-1]
         assert d_qk <= 128 and d_v <= 128, "FlashAttention only support head dimensions up to 128"
-        wide = max(d_qk, d_v)
+        wide = padded_head_dim(max(d_qk, d_v))
         pad = lambda x: torch.nn.functional.pad(x, (0, wide - x.shape[-1]))
         o, lse = hyper_attn_func(pad(q), pad(k), pad(v), q_sort_idx, k_sort_idx, block_size, sample_size,
                                  softmax_scale or 1.0 / math.sqrt(d_qk), smooth_block, sampled_idx=sampled_idx)
@@ -204,6 +212,11 @@ def flash_attn_func(q, k, v, bias=None, causal=False, softmax_scale=None):
     assert k.shape == (batch, seqlen_k, nheads, d)
     assert v.shape == (batch, seqlen_k, nheads, d)
     assert d <= 128, "FlashAttention only support head dimensions up to 128"
+    if d not in KERNEL_HEAD_DIMS:
+        # other head dims run zero-padded to a built width (exact; costs the padded copies)
+        pad = lambda x: torch.nn.functional.pad(x, (0, padded_head_dim(d) - d))
+        o, lse = flash_attn_func(pad(q), pad(k), pad(v), None, causal, softmax_scale or 1.0 / math.sqrt(d))
+        return o[..., :d], lse
     assert q.dtype == k.dtype == v.dtype, "All tensors must have the same type"
     assert q.dtype in [torch.float16, torch.bfloat16], "Only support fp16 and bf16"
     assert q.is_cuda and k.is_cuda and v.is_cuda

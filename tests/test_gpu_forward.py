@@ -130,6 +130,18 @@ def test_permuted_views_are_read_in_place(ha, causal):
     assert got.is_contiguous() and torch.equal(got, want) and torch.equal(lse, wlse)
 
 
+@pytest.mark.parametrize("causal", [False, True])
+def test_module_other_head_dim(ha, causal):
+    """input_dim 96: hashed with the module's own (96, r) projection, attention zero-padded to 128."""
+    q, k, v = (_randn((1, 2, 2048, 96), s, torch.float16) for s in (180, 181, 182))
+    m, proj = _module(ha, 96, torch.float16, 183, min_seq_len=512)
+    attn, lse = m(q.cuda(), k.cuda(), v.cuda(), causal=causal, return_lse=True)
+    assert attn.shape == (1, 2, 2048, 96) and m.lsh.proj_dir.shape[-2] == 96
+    ro, rl = _oracle(q, k, v, proj, m, causal)
+    assert_close(attn, ro, "attn", torch.float16)
+    assert_close(lse, rl, "lse")
+
+
 def test_module_argument_errors(ha):
     m, _ = _module(ha, 64, torch.float16, 160)
     q = torch.zeros((1, 1, 256, 64), dtype=torch.float16, device="cuda")

@@ -157,6 +157,19 @@ def test_flash_attention_wide_logit_range(ha, dtype, causal):
     assert_close(lse[:, :, :n], rl, "flash lse")
 
 
+@pytest.mark.parametrize("d", [32, 96, 40])
+def test_flash_attention_other_head_dims(ha, d):
+    """Head dims other than the built 64 / 128 (the reference takes any d <= 128,
+    src/flash_attn_triton.py:801) run zero-padded; the default scale is that of the original d."""
+    b, h, n = 1, 2, 640
+    q, k, v = (_randn((b, n, h, d), s, torch.float16) for s in (66, 67, 68))
+    o, lse = ha.flash_attn_func(q.cuda(), k.cuda(), v.cuda(), None, True, None)
+    assert o.shape == (b, n, h, d)
+    ro, rl = O.exact_attention(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), None, True)
+    assert_close(o.transpose(1, 2), ro, "flash out", torch.float16)
+    assert_close(lse[:, :, :n], rl, "flash lse")
+
+
 def test_flash_rejects_bias_and_bad_types(ha):
     q = torch.zeros((1, 128, 1, 64), dtype=torch.float16, device="cuda")
     with pytest.raises(NotImplementedError):
