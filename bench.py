@@ -4,7 +4,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c4|c5]
 
 A step is one forward pass over one batch of synthetic input already resident in HBM.  The default
-workload is the configuration the headline metric is quoted on (BASELINE config 3): batch 1,
+workload is the configuration the headline metric is quoted on (benchmark configuration c3): batch 1,
 32 heads, seq 131072, head dim 64, fp16, causal, 8 projections, block 256, sample 256,
 min_seq_len 2048.  Prints one JSON line (see the keys below).
 

@@ -31,7 +31,7 @@ def _oracle(q, k, v, proj, m, causal, scale=None, sampled_idx=None):
 
 # --------------------------------------------------------------------------- non-causal
 def test_non_causal_config1(ha):
-    """BASELINE config 1: batch 1, 4 heads, seq 4096, d 64, r 8, block 256, sample 256, min_seq_len 2048
+    """benchmark configuration c1: batch 1, 4 heads, seq 4096, d 64, r 8, block 256, sample 256, min_seq_len 2048
     (inputs cast to fp16 for the GPU; both the default and an explicit seeded sample set)."""
     g = _gen(100)
     q, k, v = (torch.randn((1, 4, 4096, 64), generator=g).half() for _ in range(3))
@@ -49,7 +49,7 @@ def test_non_causal_config1(ha):
 
 
 @pytest.mark.parametrize("dtype,d,block,sample,smooth", [
-    (torch.bfloat16, 128, 512, 512, True),    # BASELINE config 4 at reduced batch/heads/length
+    (torch.bfloat16, 128, 512, 512, True),    # benchmark configuration c4 at reduced batch/heads/length
     (torch.float16, 64, 256, 256, True),
     (torch.bfloat16, 64, 128, 128, False),
 ])
@@ -159,7 +159,7 @@ def test_module_argument_errors(ha):
 
 # ----------------------------------------------- full-size shapes: size-independent properties
 def test_full_size_non_causal_properties(ha):
-    """BASELINE config 2 (batch 1, 32 heads, seq 32768, d 64, fp16): permutations are valid and stable,
+    """benchmark configuration c2 (batch 1, 32 heads, seq 32768, d 64, fp16): permutations are valid and stable,
     the fused forward equals the operator-by-operator composition, and a sampled head slice matches
     the oracle."""
     b, h, n, d = 1, 32, 32768, 64
@@ -184,7 +184,7 @@ def test_full_size_non_causal_properties(ha):
 
 
 def test_full_size_causal_properties(ha):
-    """BASELINE config 3 (batch 1, 32 heads, seq 131072, d 64, fp16, causal): the first leaf is exact
+    """benchmark configuration c3 (batch 1, 32 heads, seq 131072, d 64, fp16, causal): the first leaf is exact
     causal attention, lse is finite, heads are independent, and one head matches the oracle."""
     b, h, n, d = 1, 32, 131072, 64
     g = torch.Generator(device="cuda").manual_seed(180)
@@ -209,7 +209,7 @@ def test_full_size_causal_properties(ha):
 
 
 def test_grouped_query_heads(ha):
-    """BASELINE config 5 shape family (32 query heads on 2 KV heads, d 128, bf16, causal, clustered
+    """benchmark configuration c5 shape family (32 query heads on 2 KV heads, d 128, bf16, causal, clustered
     keys) at reduced length: the expanded-KV module call matches the oracle, and the native grouped
     call (K/V not expanded) gives bit-identical results."""
     from hyperattention_amd import ops
