@@ -58,10 +58,11 @@ struct Mfma<f16_t> {
   static __device__ __forceinline__ f32x16 run(f16x8 a, f16x8 b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
   }
-  // c + a[0] + a[1]
-  static __device__ __forceinline__ float pair_sum(f16x2 a, float c) {
-    const f16x2 ones = {(f16_t)1.0f, (f16_t)1.0f};
-    return __builtin_amdgcn_fdot2(a, ones, c, false);
+  // c[*] + a[0] + a[1] + a[2] + a[3] on the matrix pipe: the 4x4x4 MFMA works on 16 independent
+  // blocks of 4 lanes; with an all-ones A a lane's four results are all the sum of its own four B values
+  static __device__ __forceinline__ f32x4 quad_sum(f16x4 a, f32x4 c) {
+    const f16x4 ones = {(f16_t)1.0f, (f16_t)1.0f, (f16_t)1.0f, (f16_t)1.0f};
+    return __builtin_amdgcn_mfma_f32_4x4x4f16(ones, a, c, 0, 0, 0);
   }
 };
 template <>
@@ -69,9 +70,10 @@ struct Mfma<bf16_t> {
   static __device__ __forceinline__ f32x16 run(bf16x8 a, bf16x8 b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
   }
-  static __device__ __forceinline__ float pair_sum(bf16x2 a, float c) {
-    const bf16x2 ones = {(bf16_t)1.0f, (bf16_t)1.0f};
-    return __builtin_amdgcn_fdot2_f32_bf16(a, ones, c, false);
+  static __device__ __forceinline__ f32x4 quad_sum(bf16x4 a, f32x4 c) {
+    typedef short s16x4 __attribute__((ext_vector_type(4)));
+    const bf16x4 ones = {(bf16_t)1.0f, (bf16_t)1.0f, (bf16_t)1.0f, (bf16_t)1.0f};
+    return __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(__builtin_bit_cast(s16x4, ones), __builtin_bit_cast(s16x4, a), c, 0, 0, 0);
   }
 };
 
@@ -152,21 +154,19 @@ __device__ __forceinline__ void global_to_lds_16(const void* src, unsigned char*
 template <typename T, int H>
 __device__ __forceinline__ void half_step_p(const f32x16 (&s_use)[2], const float (&m)[2], float scale_log2,
                                             typename ElemTraits<T>::vec8 (&pn)[2], float (&sum)[2]) {
-  typedef typename ElemTraits<T>::vec2 vec2;
+  typedef typename ElemTraits<T>::vec4 vec4;
 #pragma unroll
   for (int nb = 0; nb < 2; ++nb) {
-    float acc_sum = 0.f;
 #pragma unroll
-    for (int e = 0; e < 8; e += 2) {
-      const int i = H * 8 + e;
-      vec2 pp;
-      pp[0] = (T)__builtin_amdgcn_exp2f(__builtin_fmaf(s_use[nb][i], scale_log2, -m[nb]));
-      pp[1] = (T)__builtin_amdgcn_exp2f(__builtin_fmaf(s_use[nb][i + 1], scale_log2, -m[nb]));
-      acc_sum = Mfma<T>::pair_sum(pp, acc_sum);
-      pn[nb][e] = pp[0];
-      pn[nb][e + 1] = pp[1];
-    }
-    sum[nb] = acc_sum;
+    for (int e = 0; e < 8; ++e)
+      pn[nb][e] = (T)__builtin_amdgcn_exp2f(__builtin_fmaf(s_use[nb][H * 8 + e], scale_log2, -m[nb]));
+    // the row sums go through the matrix pipe: v_dot2 does not overlap with the big MFMAs at all
+    const vec4 lo = __builtin_shufflevector(pn[nb], pn[nb], 0, 1, 2, 3);
+    const vec4 hi = __builtin_shufflevector(pn[nb], pn[nb], 4, 5, 6, 7);
+    f32x4 acc_sum = {0.f, 0.f, 0.f, 0.f};
+    acc_sum = Mfma<T>::quad_sum(lo, acc_sum);
+    acc_sum = Mfma<T>::quad_sum(hi, acc_sum);
+    sum[nb] = acc_sum[0];
   }
 }
 
