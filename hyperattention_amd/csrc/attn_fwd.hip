@@ -337,7 +337,15 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
       int cnt = last > first ? (last - first) / KC : 0;
       if (t * 128 >= p.n_q) cnt = 0;
       int s = first / KC;
-      if (p.smooth) s = (first + p.n_k + (t - block_id * p.block_tiles) * 128 - ((p.block_tiles - 1) * 128) / 2) / KC;
+      if (p.smooth) {
+        // the window starts (block_tiles - 1) * 64 keys before the tile's own keys, modulo the sequence
+        // (src/hyper_attn_triton.py:101,105-106); reduced to 0..n_k-1 here, also when the block is
+        // longer than the sequence, and kept behind the first tile's window for the second tile
+        int sk = (first + (t - block_id * p.block_tiles) * 128 - ((p.block_tiles - 1) * 128) / 2) % p.n_k;
+        sk += sk < 0 ? p.n_k : 0;
+        s = sk / KC;
+        if (t2 == 1 && s < start[0]) s += nk_chunks;
+      }
       start[t2] = s;
       end[t2] = s + cnt;
     }

@@ -166,6 +166,9 @@ def block_key_positions(n_q: int, n_k: int, block_size: int, smooth_block: bool)
 
     Follows src/hyper_attn_triton.py:99-109 with ``block_size`` already divided by 128 as at
     :726.  Returns (pos, valid): int64 (tiles, T*128) and bool mask of the same shape.
+    When the block is so much longer than the sequence that (T-1)*64 > n_k the reference's offset
+    goes negative before its remainder (outside what it was written for); the mathematical modulo is
+    used here, and by the HIP kernel.
     """
     T = -(-block_size // TILE)
     tiles = -(-n_q // TILE)

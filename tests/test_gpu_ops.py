@@ -231,6 +231,17 @@ def test_block_sampled_explicit_samples_int32_idx_and_ragged_tail(ha):
         assert_close(lse, rl, "hyper lse")
 
 
+@pytest.mark.parametrize("n,block", [(128, 512), (256, 1024), (384, 512)])
+def test_block_attention_smooth_block_longer_than_sequence(ha, n, block):
+    """smooth_block with a block much longer than the sequence: the window offset
+    (src/hyper_attn_triton.py:101,105-106) is negative before the modulo; every key is visited once."""
+    q, k, v, qi, ki = _sorted_inputs(1, 2, n, 64, torch.float16, 90)
+    o, lse = _run_hyper(ha, q, k, v, qi, ki, block, 0, None, True, idx_dtype=torch.int32)
+    ro, rl = O.block_sampled_attention(q, k, v, qi, ki, block, 0, None, True)
+    assert_close(o, ro, "hyper out", torch.float16)
+    assert_close(lse, rl, "hyper lse")
+
+
 def test_block_attention_full_block_is_exact_attention(ha):
     b, h, n, d = 1, 2, 512, 64
     q, k, v, qi, ki = _sorted_inputs(b, h, n, d, torch.float16, 40)
