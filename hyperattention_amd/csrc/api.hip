@@ -126,8 +126,11 @@ int make_plan(const ha_forward_args& a, Plan& pl) {
   if (!a.causal) {
     pl.level_hyper[0] = !(a.min_seq_len > a.n);  // hyper_attention.py:109
     pl.any_hyper = pl.level_hyper[0];
-    if (pl.any_hyper)
+    if (pl.any_hyper) {
       HA_REQUIRE(a.n % 128 == 0, HA_ERR_SHAPE, "ha_forward: keys sequence length must be divisible by 128");
+      HA_REQUIRE(a.sampled_idx || a.sample_size <= a.n, HA_ERR_SHAPE,
+                 "ha_forward: default sampled rows 0..sample_size-1 exceed the key length");
+    }
     return HA_OK;
   }
   while (pl.len[pl.levels] > a.min_seq_len) {  // hyper_attention.py:52
@@ -139,6 +142,9 @@ int make_plan(const ha_forward_args& a, Plan& pl) {
     pl.level_hyper[pl.levels] = !(a.min_seq_len > half);
     if (pl.level_hyper[pl.levels]) {
       HA_REQUIRE(half % 128 == 0, HA_ERR_SHAPE, "ha_forward: keys sequence length must be divisible by 128");
+      HA_REQUIRE(a.sampled_idx || a.sample_size <= half, HA_ERR_SHAPE,
+                 "ha_forward: default sampled rows 0..sample_size-1 exceed the key length %lld of a level",
+                 (long long)half);
       pl.any_hyper = true;
     }
     pl.len[++pl.levels] = half;

@@ -83,6 +83,11 @@ class HyperAttention(torch.nn.Module):
             else:
                 lse = lse.unsqueeze(-1)
         else:
+            if key.shape[1] != query.shape[1]:
+                # grouped-query inputs on the operator-by-operator path: it follows the reference, which
+                # wants as many k/v heads as q heads (hyper_attention.py:43,67-68)
+                group = query.shape[1] // key.shape[1]
+                key, value = key.repeat_interleave(group, dim=1), value.repeat_interleave(group, dim=1)
             attn, lse = self._forward_composed(query.contiguous(), key.contiguous(), value.contiguous(), scale, causal)
 
         if not return_lse:

@@ -137,6 +137,10 @@ def test_forward_plan_and_workspace(lib):
     assert lib.ha_forward_workspace_bytes(ctypes.byref(f)) == -5
     f.n = 131072 + 2  # the first halves (65537) are hashed and must be a multiple of 128
     assert lib.ha_forward_workspace_bytes(ctypes.byref(f)) == -3
+    f.n, f.min_seq_len, f.sample_size = 2048, 128, 256  # the deepest hashed level has 128 keys < 256 default samples
+    assert lib.ha_forward_workspace_bytes(ctypes.byref(f)) == -3
+    assert b"sampled rows" in lib.ha_last_error()
+    f.min_seq_len = 2048
     f.n, f.causal = 4000, 0  # hashed path needs n % 128 == 0
     assert lib.ha_forward_workspace_bytes(ctypes.byref(f)) == -3
     f.n, f.min_seq_len = 1000, 2048  # exact path: no workspace needed beyond the minimum

@@ -142,6 +142,19 @@ def test_module_other_head_dim(ha, causal):
     assert_close(lse, rl, "lse")
 
 
+def test_grouped_query_on_the_composed_path(ha):
+    """An odd length takes the operator-by-operator recursion, which wants equal head counts
+    (hyper_attention.py:43,67-68): grouped-query k/v are expanded there."""
+    n, h, hk = 1001, 4, 2
+    q = _randn((1, h, n, 64), 190, torch.float16)
+    k, v = (_randn((1, hk, n, 64), s, torch.float16) for s in (191, 192))
+    m, proj = _module(ha, 64, torch.float16, 193, block_size=256, sample_size=128, min_seq_len=600)
+    attn, lse = m(q.cuda(), k.cuda(), v.cuda(), causal=True, return_lse=True)
+    ro, rl = _oracle(q, k.repeat_interleave(2, dim=1), v.repeat_interleave(2, dim=1), proj, m, True)
+    assert_close(attn, ro, "attn", torch.float16)
+    assert_close(lse, rl, "lse")
+
+
 def test_module_argument_errors(ha):
     m, _ = _module(ha, 64, torch.float16, 160)
     q = torch.zeros((1, 1, 256, 64), dtype=torch.float16, device="cuda")
