@@ -181,9 +181,11 @@ __device__ __forceinline__ void half_step_rescale(const f32x16 (&s_use)[2], floa
   float m_use[2];
 #pragma unroll
   for (int nb = 0; nb < 2; ++nb) {
-    float v = s_use[nb][0];
+    // only this half-step's values: the other half of the step raises the exponents itself if it has
+    // to, and the two rare paths of a step then share no work the compiler would compute up front
+    float v = s_use[nb][H * 8];
 #pragma unroll
-    for (int i = 1; i < 16; ++i) v = fmaxf(v, s_use[nb][i]);
+    for (int e = 1; e < 8; ++e) v = fmaxf(v, s_use[nb][H * 8 + e]);
     v = fmaxf(v, __shfl_xor(v, 32)) * scale_log2;
     const float m_new = fmaxf(m_run[nb], v);
     // nothing accumulated yet under m_run = -inf; otherwise 2^(old - new) <= 1
@@ -262,9 +264,11 @@ __device__ __forceinline__ void half_step(const f32x16 (&s_use)[2], f32x16 (&s_f
     __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);  // three VALU
     __builtin_amdgcn_sched_group_barrier(0x400, 2, 0);  // two transcendental
   }
-  // not "sum >= limit": a NaN (row that has seen nothing yet) must take the rare path too
-  const bool redo = !(sum[0] < HALF_SUM_LIMIT) || !(sum[1] < HALF_SUM_LIMIT);
-  if (__any(redo)) {
+  // One compare for both query blocks: their sums are >= 0 or NaN, so the total is below the limit
+  // only if both are.  Not "total >= limit": a NaN (row that has seen nothing yet) must take the rare
+  // path too.
+  const bool redo = !(sum[0] + sum[1] < HALF_SUM_LIMIT);
+  if (__builtin_amdgcn_ballot_w64(redo) != 0) {
     half_step_rescale<T, D, H>(s_use, scale_log2, alpha_pend, m_run, l_run, pn, sum);
     rescale_pend = true;
   }
