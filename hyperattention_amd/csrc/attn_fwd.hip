@@ -218,7 +218,7 @@ __device__ __forceinline__ void half_step(const f32x16 (&s_use)[2], f32x16 (&s_f
   constexpr int KH = D / 32;  // k-steps of this half
   constexpr int DB = D / 32;
 
-  if (rescale_pend) {
+  if (__builtin_expect(rescale_pend, false)) {
 #pragma unroll
     for (int db = 0; db < DB; ++db)
 #pragma unroll
@@ -268,7 +268,7 @@ __device__ __forceinline__ void half_step(const f32x16 (&s_use)[2], f32x16 (&s_f
   // only if both are.  Not "total >= limit": a NaN (row that has seen nothing yet) must take the rare
   // path too.
   const bool redo = !(sum[0] + sum[1] < HALF_SUM_LIMIT);
-  if (__builtin_amdgcn_ballot_w64(redo) != 0) {
+  if (__builtin_expect(__builtin_amdgcn_ballot_w64(redo) != 0, false)) {
     half_step_rescale<T, D, H>(s_use, scale_log2, alpha_pend, m_run, l_run, pn, sum);
     rescale_pend = true;
   }
@@ -445,14 +445,36 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
   const int k_chunk_shift = (wave_s >> 1) - 1;
 #define HA_FETCH_ROWS_K(tile_c, rs) fetch_rows((tile_c) + k_chunk_shift, k_kk0, rs);
 #define HA_FETCH_ROWS_V(ci, rs) fetch_rows((ci), v_kk0, rs);
+// Rows listed by an index array cost a lane one multiply-add each.  Consecutive rows cost it nothing
+// per tile: the first row of the load goes into the wave-uniform base, the lane's own row and piece
+// are loop constants.  Only a tile that reaches past the last key (or lies outside the chunk range:
+// row0 < 0, every lane reads row 0) computes and clamps row numbers per lane.  All branches are
+// wave-uniform.
 #define HA_LOAD_TILE(base, stride, rs, kk0, tile, SWZ)                                                   \
-  _Pragma("unroll") for (int j = 0; j < LPW; ++j) {                                                      \
-    const int r = (wave_s * LPW + j) * ROWS_PER_LOAD + my_lr;                                            \
-    int row = rs.first + (kk0) + j * ROWS_PER_LOAD + my_lr; /* consecutive rows */                       \
-    if (!GATHER && row >= p.n_k) row = 0;                                                                \
-    if (GATHER && rs.first == ROWS_LOADED) row = rs.rows[j];                                             \
-    if (rs.first == ROWS_NONE) row = 0;                                                                  \
-    global_to_lds_16(row_address(base, row, stride, (my_pp ^ SWZ(r)) << 4), (tile) + (wave_s * LPW + j) * 1024); \
+  if (GATHER && rs.first == ROWS_LOADED) {                                                               \
+    _Pragma("unroll") for (int j = 0; j < LPW; ++j) {                                                    \
+      const int r = (wave_s * LPW + j) * ROWS_PER_LOAD + my_lr;                                          \
+      global_to_lds_16(row_address(base, rs.rows[j], stride, (my_pp ^ SWZ(r)) << 4),                     \
+                       (tile) + (wave_s * LPW + j) * 1024);                                              \
+    }                                                                                                    \
+  } else {                                                                                               \
+    const int row0 = rs.first == ROWS_NONE ? -1 : rs.first + (kk0);                                      \
+    if (row0 >= 0 && (GATHER || row0 + LPW * ROWS_PER_LOAD <= p.n_k)) {                                  \
+      _Pragma("unroll") for (int j = 0; j < LPW; ++j) {                                                  \
+        const int r = (wave_s * LPW + j) * ROWS_PER_LOAD + my_lr;                                        \
+        const uint32_t first_row = __builtin_amdgcn_readfirstlane((uint32_t)(row0 + j * ROWS_PER_LOAD) * (stride)); \
+        global_to_lds_16(row_address(base + first_row, my_lr, stride, (my_pp ^ SWZ(r)) << 4),            \
+                         (tile) + (wave_s * LPW + j) * 1024);                                            \
+      }                                                                                                  \
+    } else {                                                                                             \
+      _Pragma("unroll") for (int j = 0; j < LPW; ++j) {                                                  \
+        const int r = (wave_s * LPW + j) * ROWS_PER_LOAD + my_lr;                                        \
+        int row = row0 + j * ROWS_PER_LOAD + my_lr;                                                      \
+        if (row0 < 0 || row >= p.n_k) row = 0;                                                           \
+        global_to_lds_16(row_address(base, row, stride, (my_pp ^ SWZ(r)) << 4),                          \
+                         (tile) + (wave_s * LPW + j) * 1024);                                            \
+      }                                                                                                  \
+    }                                                                                                    \
   }
 
   // ---- first loads: row numbers of the queries and of the first key tiles, then the rows ----------
@@ -618,12 +640,12 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
     /* causal: once a chunk lies wholly above this wave's queries, so do all later ones */                  \
     if (!(CAUSAL && (ci) * KC > wave_q_first + 63)) {                                                       \
       const bool masked = chunk_masked(ci);                                                                 \
-      if (masked) { HA_APPLY_MASK(ci, 0, s_a) }                                                             \
+      if (__builtin_expect(masked, false)) { HA_APPLY_MASK(ci, 0, s_a) }                                                             \
       half_step<T, D, 0>(s_a, s_b, K_RD, 0, V_CUR, 0, lo, qf, acc, m_run, l_run, pb, vf,                    \
                          p.scale_log2, alpha_pend, rescale_pend);                                           \
       half_step<T, D, 1>(s_a, s_b, K_RD, 0, V_CUR, 16 * D * 2, lo, qf, acc, m_run, l_run, pb, vf,           \
                          p.scale_log2, alpha_pend, rescale_pend);                                           \
-      if (masked) { HA_APPLY_MASK(ci, 1, s_b) }                                                             \
+      if (__builtin_expect(masked, false)) { HA_APPLY_MASK(ci, 1, s_b) }                                                             \
       half_step<T, D, 0>(s_b, s_a, K_RD, 32 * D * 2, V_CUR, 32 * D * 2, lo, qf, acc, m_run, l_run, pb, vf,  \
                          p.scale_log2, alpha_pend, rescale_pend);                                           \
       half_step<T, D, 1>(s_b, s_a, K_RD, 32 * D * 2, V_CUR, 48 * D * 2, lo, qf, acc, m_run, l_run, pb, vf,  \
