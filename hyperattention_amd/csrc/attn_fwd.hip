@@ -170,13 +170,12 @@ __device__ __forceinline__ void half_step_p(const f32x16 (&s_use)[2], const floa
   }
 }
 
-// The rare path of a half-step: raise the reference exponents to the row maxima of the step, rescale
-// the row sums and redo the half-step's P.  The accumulators hold everything up to the previous
-// half-step (its P.V was issued in this block); they are rescaled by alpha_pend at the start of the
-// next block, before the P.V of this half-step is added.
+// The rare path of a half-step: raise the reference exponents to the row maxima of the half-step,
+// rescale the row sums and redo the half-step's P.  alpha is what everything accumulated under the old
+// exponents has to be multiplied by.
 template <typename T, int D, int H>
 __device__ __forceinline__ void half_step_rescale(const f32x16 (&s_use)[2], float scale_log2,
-                                                  float (&alpha_pend)[2], float (&m_run)[2], float (&l_run)[2],
+                                                  float (&alpha)[2], float (&m_run)[2], float (&l_run)[2],
                                                   typename ElemTraits<T>::vec8 (&pn)[2], float (&sum)[2]) {
   float m_use[2];
 #pragma unroll
@@ -189,10 +188,9 @@ __device__ __forceinline__ void half_step_rescale(const f32x16 (&s_use)[2], floa
     v = fmaxf(v, __shfl_xor(v, 32)) * scale_log2;
     const float m_new = fmaxf(m_run[nb], v);
     // nothing accumulated yet under m_run = -inf; otherwise 2^(old - new) <= 1
-    const float alpha = m_run[nb] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m_run[nb] - m_new);
+    alpha[nb] = m_run[nb] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m_run[nb] - m_new);
     m_run[nb] = m_new;
-    l_run[nb] *= alpha;
-    alpha_pend[nb] = alpha;
+    l_run[nb] *= alpha[nb];
     // rows that have seen no key yet (all masked) keep m_run = -inf; their P is 2^(-inf - 0) = 0
     m_use[nb] = m_new == -INFINITY ? 0.f : m_new;
   }
@@ -204,7 +202,6 @@ __device__ __forceinline__ void half_step_rescale(const f32x16 (&s_use)[2], floa
 //           (k-steps H*KSTEPS/2 ..) of the next step's S^T, K rows k_row_off.. of k_tile
 //   VALU  : P of this half-step from s_use -> pb (for the next block) and the row sums
 //   LDS   : V^T of this half-step's keys (v_key_off.. of v_tile) -> vf (for the next block)
-// rescale_pend (wave-uniform) / alpha_pend: accumulator rescale left over by the previous block
 template <typename T, int D, int H>
 __device__ __forceinline__ void half_step(const f32x16 (&s_use)[2], f32x16 (&s_fill)[2],
                                           const unsigned char* k_tile, int k_row_off,
@@ -212,21 +209,11 @@ __device__ __forceinline__ void half_step(const f32x16 (&s_use)[2], f32x16 (&s_f
                                           const typename ElemTraits<T>::vec8 (&qf)[2][D / 16],
                                           f32x16 (&acc)[D / 32][2], float (&m_run)[2], float (&l_run)[2],
                                           typename ElemTraits<T>::vec8 (&pb)[2],
-                                          typename ElemTraits<T>::vec8 (&vf)[D / 32], float scale_log2,
-                                          float (&alpha_pend)[2], bool& rescale_pend) {
+                                          typename ElemTraits<T>::vec8 (&vf)[D / 32], float scale_log2) {
   typedef typename ElemTraits<T>::vec8 vec8;
   constexpr int KH = D / 32;  // k-steps of this half
   constexpr int DB = D / 32;
 
-  if (__builtin_expect(rescale_pend, false)) {
-#pragma unroll
-    for (int db = 0; db < DB; ++db)
-#pragma unroll
-      for (int nb = 0; nb < 2; ++nb)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) acc[db][nb][i] *= alpha_pend[nb];
-    rescale_pend = false;
-  }
   vec8 kf[KH];
 #pragma unroll
   for (int k2 = 0; k2 < KH; ++k2) kf[k2] = lds_read_k<T>(k_tile, lo.k[H * KH + k2] + k_row_off);
@@ -269,8 +256,16 @@ __device__ __forceinline__ void half_step(const f32x16 (&s_use)[2], f32x16 (&s_f
   // path too.
   const bool redo = !(sum[0] + sum[1] < HALF_SUM_LIMIT);
   if (__builtin_expect(__builtin_amdgcn_ballot_w64(redo) != 0, false)) {
-    half_step_rescale<T, D, H>(s_use, scale_log2, alpha_pend, m_run, l_run, pn, sum);
-    rescale_pend = true;
+    float alpha[2];
+    half_step_rescale<T, D, H>(s_use, scale_log2, alpha, m_run, l_run, pn, sum);
+    // the accumulators hold everything up to the previous half-step (its P.V was issued above; the
+    // P.V of this half-step is added by the next block, under the new exponents)
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[db][nb][i] *= alpha[nb];
   }
 #pragma unroll
   for (int nb = 0; nb < 2; ++nb) {
@@ -459,7 +454,7 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
     }                                                                                                    \
   } else {                                                                                               \
     const int row0 = rs.first == ROWS_NONE ? -1 : rs.first + (kk0);                                      \
-    if (row0 >= 0 && (GATHER || row0 + LPW * ROWS_PER_LOAD <= p.n_k)) {                                  \
+    if (__builtin_expect(row0 >= 0 && (GATHER || row0 + LPW * ROWS_PER_LOAD <= p.n_k), true)) {          \
       _Pragma("unroll") for (int j = 0; j < LPW; ++j) {                                                  \
         const int r = (wave_s * LPW + j) * ROWS_PER_LOAD + my_lr;                                        \
         const uint32_t first_row = __builtin_amdgcn_readfirstlane((uint32_t)(row0 + j * ROWS_PER_LOAD) * (stride)); \
@@ -612,8 +607,6 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
   for (int nb = 0; nb < 2; ++nb) pb[nb] = vec8{};
 #pragma unroll
   for (int db = 0; db < DB; ++db) vf[db] = vec8{};
-  float alpha_pend[2] = {1.f, 1.f};  // accumulator rescale owed by the last half-step, if rescale_pend
-  bool rescale_pend = false;
   bool pending = false;  // pb/vf hold a half-step whose P.V has not been issued
   // all waves hold their operands of K tile 0: its buffer may be overwritten from iteration 0 on
   __syncthreads();
@@ -624,17 +617,16 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
   // tile ci was read from during iteration ci-1, and V tile ci+1 into the buffer of V tile ci-1.
   // The loop is unrolled by two so that every tile access names its LDS object statically.
 #define HA_PV_DRAIN()                                                                                       \
-  if (rescale_pend) {                                                                                       \
-    _Pragma("unroll") for (int db = 0; db < DB; ++db) _Pragma("unroll") for (int nb = 0; nb < 2; ++nb)      \
-        _Pragma("unroll") for (int i = 0; i < 16; ++i) acc[db][nb][i] *= alpha_pend[nb];                    \
-    rescale_pend = false;                                                                                   \
-  }                                                                                                         \
   _Pragma("unroll") for (int db = 0; db < DB; ++db) _Pragma("unroll") for (int nb = 0; nb < 2; ++nb)        \
       acc[db][nb] = Mfma<T>::run(vf[db], pb[nb], acc[db][nb]);
 #define HA_ITERATION(ci, K_RD, K_WR, V_CUR, V_WR)                                                           \
   {                                                                                                         \
-    if ((ci) + 2 <= n_chunks) { HA_LOAD_TILE(kb, k_rb, rows_k, k_kk0, K_WR, k_swizzle) } /* K tile ci+2 */  \
-    if ((ci) + 1 < n_chunks) { HA_LOAD_TILE(vb, v_rb, rows_v, v_kk0, V_WR, v_swizzle) }  /* V tile ci+1 */  \
+    if (__builtin_expect((ci) + 2 <= n_chunks, true)) {                                                     \
+      HA_LOAD_TILE(kb, k_rb, rows_k, k_kk0, K_WR, k_swizzle) /* K tile ci+2 */                              \
+    }                                                                                                       \
+    if (__builtin_expect((ci) + 1 < n_chunks, true)) {                                                      \
+      HA_LOAD_TILE(vb, v_rb, rows_v, v_kk0, V_WR, v_swizzle) /* V tile ci+1 */                              \
+    }                                                                                                       \
     HA_FETCH_ROWS_K((ci) + 3, rows_k)                                                                       \
     HA_FETCH_ROWS_V((ci) + 2, rows_v)                                                                       \
     /* causal: once a chunk lies wholly above this wave's queries, so do all later ones */                  \
@@ -642,14 +634,14 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
       const bool masked = chunk_masked(ci);                                                                 \
       if (__builtin_expect(masked, false)) { HA_APPLY_MASK(ci, 0, s_a) }                                                             \
       half_step<T, D, 0>(s_a, s_b, K_RD, 0, V_CUR, 0, lo, qf, acc, m_run, l_run, pb, vf,                    \
-                         p.scale_log2, alpha_pend, rescale_pend);                                           \
+                         p.scale_log2);                                                                     \
       half_step<T, D, 1>(s_a, s_b, K_RD, 0, V_CUR, 16 * D * 2, lo, qf, acc, m_run, l_run, pb, vf,           \
-                         p.scale_log2, alpha_pend, rescale_pend);                                           \
+                         p.scale_log2);                                                                     \
       if (__builtin_expect(masked, false)) { HA_APPLY_MASK(ci, 1, s_b) }                                                             \
       half_step<T, D, 0>(s_b, s_a, K_RD, 32 * D * 2, V_CUR, 32 * D * 2, lo, qf, acc, m_run, l_run, pb, vf,  \
-                         p.scale_log2, alpha_pend, rescale_pend);                                           \
+                         p.scale_log2);                                                                     \
       half_step<T, D, 1>(s_b, s_a, K_RD, 32 * D * 2, V_CUR, 48 * D * 2, lo, qf, acc, m_run, l_run, pb, vf,  \
-                         p.scale_log2, alpha_pend, rescale_pend);                                           \
+                         p.scale_log2);                                                                     \
       pending = true;                                                                                       \
     } else if (pending) {                                                                                   \
       HA_PV_DRAIN()                                                                                         \
