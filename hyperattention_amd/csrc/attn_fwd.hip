@@ -291,10 +291,12 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
   // knows that a tile being filled from HBM and a tile being read do not alias, and does not
   // serialise them.  The query region (one tile per wave) is reused for the output rows at the end.
   constexpr int TILE_BYTES = KC * D * 2;
-  __shared__ __attribute__((aligned(16))) unsigned char lds_k0[TILE_BYTES];
-  __shared__ __attribute__((aligned(16))) unsigned char lds_k1[TILE_BYTES];
-  __shared__ __attribute__((aligned(16))) unsigned char lds_v0[TILE_BYTES];
-  __shared__ __attribute__((aligned(16))) unsigned char lds_v1[TILE_BYTES];
+  // The key tiles ask for the larger alignment only to be placed first: LDS offsets below 64 KB fit
+  // the immediate field of the LDS reads, which matters at d = 128 where the workgroup uses 130 KB.
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_k0[TILE_BYTES];
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_k1[TILE_BYTES];
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_v0[TILE_BYTES];
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_v1[TILE_BYTES];
   __shared__ __attribute__((aligned(16))) unsigned char lds_q[4 * TILE_BYTES];
   __shared__ int lds_qrow[WG_QUERIES];   // original row of every query position (-1: past the end)
   __shared__ float lds_w[WG_QUERIES];    // weight of the resumed partial result per query position
