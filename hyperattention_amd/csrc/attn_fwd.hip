@@ -389,7 +389,8 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
 
   // Original rows of keys kk0 + j*ROWS_PER_LOAD + my_lr (j < LPW) of chunk ci.  The source of a chunk
   // is wave-uniform: either a run of an index array (sorted keys of the block part, or an explicit
-  // sample list) or consecutive rows (default samples, exact attention).  Index arrays are read as
+  // sample list) or consecutive rows (default samples; exact attention needs none of this and takes
+  // its rows straight from the chunk number when it loads a tile).  Index arrays are read as
   // 4-byte words at a stride of 4 or 8 bytes (row numbers fit the low word of an int64).  Keys past
   // n_k and chunks outside 0..n_chunks-1 alias row 0: row 0 holds finite data and their scores are
   // masked or never used.  Every branch is wave-uniform and nothing touches a loaded value here: the
@@ -440,14 +441,14 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
   const int v_kk0 = wave_s * (LPW * ROWS_PER_LOAD);
   const int k_kk0 = (v_kk0 + 32) & 63;
   const int k_chunk_shift = (wave_s >> 1) - 1;
-#define HA_FETCH_ROWS_K(tile_c, rs) fetch_rows((tile_c) + k_chunk_shift, k_kk0, rs);
-#define HA_FETCH_ROWS_V(ci, rs) fetch_rows((ci), v_kk0, rs);
+#define HA_FETCH_ROWS_K(tile_c, rs) if (GATHER) fetch_rows((tile_c) + k_chunk_shift, k_kk0, rs);
+#define HA_FETCH_ROWS_V(ci, rs) if (GATHER) fetch_rows((ci), v_kk0, rs);
 // Rows listed by an index array cost a lane one multiply-add each.  Consecutive rows cost it nothing
 // per tile: the first row of the load goes into the wave-uniform base, the lane's own row and piece
 // are loop constants.  Only a tile that reaches past the last key (or lies outside the chunk range:
 // row0 < 0, every lane reads row 0) computes and clamps row numbers per lane.  All branches are
 // wave-uniform.
-#define HA_LOAD_TILE(base, stride, rs, kk0, tile, SWZ)                                                   \
+#define HA_LOAD_TILE(base, stride, rs, chunk, kk0, tile, SWZ)                                            \
   if (GATHER && rs.first == ROWS_LOADED) {                                                               \
     _Pragma("unroll") for (int j = 0; j < LPW; ++j) {                                                    \
       const int r = (wave_s * LPW + j) * ROWS_PER_LOAD + my_lr;                                          \
@@ -455,7 +456,9 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
                        (tile) + (wave_s * LPW + j) * 1024);                                              \
     }                                                                                                    \
   } else {                                                                                               \
-    const int row0 = rs.first == ROWS_NONE ? -1 : rs.first + (kk0);                                      \
+    /* exact attention: chunk c is rows 64 c ..; a chunk before the first reads row 0 */                 \
+    const int row0 = GATHER ? (rs.first == ROWS_NONE ? -1 : rs.first + (kk0))                            \
+                            : ((chunk) < 0 ? -1 : (chunk) * KC + (kk0));                                  \
     if (__builtin_expect(row0 >= 0 && (GATHER || row0 + LPW * ROWS_PER_LOAD <= p.n_k), true)) {          \
       _Pragma("unroll") for (int j = 0; j < LPW; ++j) {                                                  \
         const int r = (wave_s * LPW + j) * ROWS_PER_LOAD + my_lr;                                        \
@@ -509,7 +512,7 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
 #pragma unroll
     for (int nb = 0; nb < 2; ++nb)
       if (wave_q_first + nb * 32 + col >= p.n_q) qrow[nb] = -1;
-    HA_LOAD_TILE(kb, k_rb, rows_k, k_kk0, lds_k0, k_swizzle)
+    HA_LOAD_TILE(kb, k_rb, rows_k, k_chunk_shift, k_kk0, lds_k0, k_swizzle)
 #pragma unroll
     for (int j = 0; j < PR; ++j) {
       // positions past the end read row 0 (finite data; their results are never written)
@@ -517,8 +520,8 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
       global_to_lds_16(row_address(qb, q_rows[j] < 0 ? 0 : q_rows[j], q_rb, (my_pp ^ (r & 7)) << 4), my_q + j * 1024);
       if (my_pp == 0) lds_qrow[wave * 64 + r] = q_rows[j];
     }
-    HA_LOAD_TILE(vb, v_rb, rows_v, v_kk0, lds_v0, v_swizzle)
-    HA_LOAD_TILE(kb, k_rb, rows_k1, k_kk0, lds_k1, k_swizzle)
+    HA_LOAD_TILE(vb, v_rb, rows_v, 0, v_kk0, lds_v0, v_swizzle)
+    HA_LOAD_TILE(kb, k_rb, rows_k1, 1 + k_chunk_shift, k_kk0, lds_k1, k_swizzle)
   }
   HA_FETCH_ROWS_K(2, rows_k)
   HA_FETCH_ROWS_V(1, rows_v)
@@ -624,10 +627,10 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
 #define HA_ITERATION(ci, K_RD, K_WR, V_CUR, V_WR)                                                           \
   {                                                                                                         \
     if (__builtin_expect((ci) + 2 <= n_chunks, true)) {                                                     \
-      HA_LOAD_TILE(kb, k_rb, rows_k, k_kk0, K_WR, k_swizzle) /* K tile ci+2 */                              \
+      HA_LOAD_TILE(kb, k_rb, rows_k, (ci) + 2 + k_chunk_shift, k_kk0, K_WR, k_swizzle) /* K tile ci+2 */    \
     }                                                                                                       \
     if (__builtin_expect((ci) + 1 < n_chunks, true)) {                                                      \
-      HA_LOAD_TILE(vb, v_rb, rows_v, v_kk0, V_WR, v_swizzle) /* V tile ci+1 */                              \
+      HA_LOAD_TILE(vb, v_rb, rows_v, (ci) + 1, v_kk0, V_WR, v_swizzle) /* V tile ci+1 */                    \
     }                                                                                                       \
     HA_FETCH_ROWS_K((ci) + 3, rows_k)                                                                       \
     HA_FETCH_ROWS_V((ci) + 2, rows_v)                                                                       \
