@@ -41,16 +41,20 @@ __device__ __forceinline__ BlockRef locate_block(const ha_sort_jobs& jobs, int b
   return r;
 }
 
-// lanes of the wave holding the same digit as this lane, restricted to valid lanes
+// lanes of the wave holding the same digit as this lane, restricted to valid lanes.  Per bit: the
+// lane's own bit spread over a word (0 or ~0), one ballot, and per mask half one three-input bit
+// operation "keep the lanes whose bit equals mine".
 __device__ __forceinline__ uint64_t match_digit(int digit, bool valid) {
-  uint64_t mask = __ballot(valid);
+  const uint64_t all = __ballot(valid);
+  uint32_t lo = (uint32_t)all, hi = (uint32_t)(all >> 32);
 #pragma unroll
   for (int bit = 0; bit < 8; ++bit) {
-    const bool set = (digit >> bit) & 1;
-    const uint64_t b = __ballot(set);
-    mask &= set ? b : ~b;
+    const uint32_t mine = (uint32_t)((int32_t)((uint32_t)digit << (31 - bit)) >> 31);
+    const uint64_t b = __ballot(mine != 0u);
+    lo &= ~((uint32_t)b ^ mine);
+    hi &= ~((uint32_t)(b >> 32) ^ mine);
   }
-  return mask;
+  return ((uint64_t)hi << 32) | lo;
 }
 
 // number of set bits of `mask` below this lane
@@ -58,11 +62,18 @@ __device__ __forceinline__ uint32_t rank_below(uint64_t mask) {
   return __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0u));
 }
 
-__device__ __forceinline__ int load_digit(const ha_sort_job& job, const int32_t* prev, int64_t seg_base, int i,
-                                          int shift, int* src) {
-  const int s = prev ? prev[i] : i;
-  *src = s;
-  return (job.keys[seg_base + s] >> shift) & 255;
+// Digits (and source rows) of positions first + s*stride (s < SORT_STEPS) of a segment.  Positions past the
+// end are clamped to the last one, so every load is unconditional and all of them are in flight
+// together: one memory round trip per pass instead of one per step.
+__device__ __forceinline__ void load_digits(const ha_sort_job& job, const int32_t* prev, int64_t seg_base, int first,
+                                            int stride, int shift, int (&src)[SORT_STEPS], int (&digit)[SORT_STEPS]) {
+#pragma unroll
+  for (int s = 0; s < SORT_STEPS; ++s) {
+    const int i = min(first + s * stride, job.seg_len - 1);
+    src[s] = prev ? prev[i] : i;
+  }
+#pragma unroll
+  for (int s = 0; s < SORT_STEPS; ++s) digit[s] = (job.keys[seg_base + src[s]] >> shift) & 255;
 }
 
 // ---- per-chunk histograms (only for segments longer than one chunk) -------------------------
@@ -77,14 +88,11 @@ __global__ __launch_bounds__(SORT_THREADS) void sort_hist_kernel(ha_sort_jobs jo
   const int64_t seg_base = job.seg_offset + (int64_t)br.seg * job.seg_stride;
   const int32_t* prev = job.prev ? job.prev + (int64_t)br.seg * job.seg_len : nullptr;
   const int chunk_start = br.chunk * HA_SORT_CHUNK;
-#pragma unroll 4
-  for (int s = 0; s < SORT_STEPS; ++s) {
-    const int i = chunk_start + s * SORT_THREADS + tid;
-    if (i < job.seg_len) {
-      int src;
-      atomicAdd(&hist[load_digit(job, prev, seg_base, i, jobs.shift, &src)], 1u);
-    }
-  }
+  int src[SORT_STEPS], digit[SORT_STEPS];
+  load_digits(job, prev, seg_base, chunk_start + tid, SORT_THREADS, jobs.shift, src, digit);
+#pragma unroll
+  for (int s = 0; s < SORT_STEPS; ++s)
+    if (chunk_start + s * SORT_THREADS + tid < job.seg_len) atomicAdd(&hist[digit[s]], 1u);
   __syncthreads();
   job.hist[((int64_t)br.seg * job.chunks_per_seg + br.chunk) * 256 + tid] = hist[tid];
 }
@@ -124,9 +132,9 @@ __global__ __launch_bounds__(SORT_THREADS) void sort_scan_kernel(ha_sort_jobs jo
 }
 
 // ---- stable scatter --------------------------------------------------------------------------
-// A wave owns a contiguous run of the chunk (wave order = key order).  Pass 1 counts digits per wave
-// with LDS atomics; pass 2 re-reads the keys (they are cache resident) and ranks them inside each
-// 64-key step by ballot matching, which is what keeps equal keys in ascending row order.  The chunk is
+// A wave owns a contiguous run of the chunk (wave order = key order) and holds its digits in registers.
+// Pass 1 counts digits per wave with LDS atomics; pass 2 ranks the keys inside each 64-key step by
+// ballot matching, which is what keeps equal keys in ascending row order.  The chunk is
 // put in order in LDS first and then written out by consecutive threads, so that the runs of equal
 // keys leave as whole cache lines instead of scattered 4-byte writes.
 __global__ __launch_bounds__(SORT_THREADS) void sort_scatter_kernel(ha_sort_jobs jobs) {
@@ -147,14 +155,11 @@ __global__ __launch_bounds__(SORT_THREADS) void sort_scatter_kernel(ha_sort_jobs
   const int wave_start = chunk_start + wave * (SORT_STEPS * HA_WAVE);
   const bool stage = job.seg_len <= (1 << 24);  // rows fit 24 bits next to the digit
 
-#pragma unroll 4
-  for (int s = 0; s < SORT_STEPS; ++s) {
-    const int i = wave_start + s * HA_WAVE + lane;
-    if (i < job.seg_len) {
-      int src;
-      atomicAdd(&wave_hist[wave][load_digit(job, prev, seg_base, i, jobs.shift, &src)], 1u);
-    }
-  }
+  int src_all[SORT_STEPS], digit_all[SORT_STEPS];
+  load_digits(job, prev, seg_base, wave_start + lane, HA_WAVE, jobs.shift, src_all, digit_all);
+#pragma unroll
+  for (int s = 0; s < SORT_STEPS; ++s)
+    if (wave_start + s * HA_WAVE + lane < job.seg_len) atomicAdd(&wave_hist[wave][digit_all[s]], 1u);
   __syncthreads();
 
   // chunk-local first slot of key tid, and the global first slot of (this chunk, key tid): from the
@@ -177,12 +182,11 @@ __global__ __launch_bounds__(SORT_THREADS) void sort_scatter_kernel(ha_sort_jobs
   __syncthreads();
 
   const int64_t out_base = (int64_t)br.seg * job.seg_len;
-#pragma unroll 2
+#pragma unroll
   for (int s = 0; s < SORT_STEPS; ++s) {
     const int i = wave_start + s * HA_WAVE + lane;
     const bool valid = i < job.seg_len;
-    int src = 0, digit = 0;
-    if (valid) digit = load_digit(job, prev, seg_base, i, jobs.shift, &src);
+    const int src = src_all[s], digit = digit_all[s];
     const uint64_t m = match_digit(digit, valid);
     const uint32_t below = rank_below(m);
     if (valid) {
