@@ -320,6 +320,33 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
   const int b = fast_div(bh, p.heads, p.heads_shift), h = bh - b * p.heads;
   const int hk = fast_div(h, p.kv_group, p.kv_group_shift);
 
+  // ---- row numbers of the queries: the first thing the workgroup has to wait for, so they are asked
+  // for before the rest of the set-up (sorted query positions of this head: entries of 4 or 8 bytes,
+  // the row number in the low word) ------------------------------------------------------------------
+  constexpr int ROWS_PER_LOAD = 64 / PR;
+  const int my_pp = lane % PR;  // physical piece of this lane's LDS slot in a tile load
+  const int my_lr = lane / PR;  // row inside one tile load
+  const int wave_q_first = qt * WG_QUERIES + wave * 64;
+  const int idx_shift = p.idx64 ? 3 : 2;
+  const int64_t qidx_off = b * p.qi_sb + h * p.qi_sh + (int64_t)seg * p.n_q * p.qi_sn;
+  const unsigned char* const q_idx_base = (const unsigned char*)p.q_idx + (qidx_off << idx_shift);
+  const uint32_t qi_rb = (uint32_t)p.qi_sn << idx_shift;
+  int q_rows[PR];  // rows of this wave's query tile, in the order of its PR loads
+  int qrow[2];     // original row of the query a lane's S^T / O^T columns belong to
+#pragma unroll
+  for (int j = 0; j < PR; ++j) {
+    // positions past the end load the index of position 0 (replaced by -1 once all the index loads
+    // of the prologue are in flight)
+    const int pq = wave_q_first + j * ROWS_PER_LOAD + my_lr;
+    q_rows[j] = GATHER ? *reinterpret_cast<const int*>(row_address(q_idx_base, pq < p.n_q ? pq : 0, qi_rb, 0)) : pq;
+  }
+#pragma unroll
+  for (int nb = 0; nb < 2; ++nb) {
+    const int pq = wave_q_first + nb * 32 + col;
+    qrow[nb] = GATHER ? *reinterpret_cast<const int*>(row_address(q_idx_base, pq < p.n_q ? pq : 0, qi_rb, 0)) : pq;
+  }
+  if (GATHER) __builtin_amdgcn_sched_barrier(0);
+
   // bases of this (virtual) head as byte pointers, row strides in bytes
   const unsigned char* qb = (const unsigned char*)((const T*)p.q + b * p.q_sb + h * p.q_sh + (p.q_seg_off + (int64_t)seg * p.seg_stride) * p.q_sn);
   const unsigned char* kb = (const unsigned char*)((const T*)p.k + b * p.k_sb + hk * p.k_sh + (p.k_seg_off + (int64_t)seg * p.seg_stride) * p.k_sn);
@@ -327,7 +354,6 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
   unsigned char* ob = (unsigned char*)((T*)p.out + b * p.o_sb + h * p.o_sh + (p.q_seg_off + (int64_t)seg * p.seg_stride) * p.o_sn);
   const uint32_t q_rb = (uint32_t)p.q_sn * 2, k_rb = (uint32_t)p.k_sn * 2, v_rb = (uint32_t)p.v_sn * 2, o_rb = (uint32_t)p.o_sn * 2;
   float* lb = p.lse + b * p.lse_sb + h * p.lse_sh + p.q_seg_off + (int64_t)seg * p.seg_stride;
-  const int64_t qidx_off = b * p.qi_sb + h * p.qi_sh + (int64_t)seg * p.n_q * p.qi_sn;
   const int64_t kidx_off = b * p.ki_sb + hk * p.ki_sh + (int64_t)seg * p.n_k * p.ki_sn;
   const int64_t sidx_off = b * p.si_sb + hk * p.si_sh;
 
@@ -374,7 +400,6 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
     }
     n_chunks = (kend + KC - 1) / KC;
   }
-  const int wave_q_first = qt * WG_QUERIES + wave * 64;
 
   // ---- rows: HBM -> LDS without passing through registers -----------------------------------------
   // One global_load_lds moves 16 bytes per lane to 1 KB of consecutive LDS: 64/PR rows of a tile.
@@ -382,10 +407,7 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
   // A lane's LDS slot is (row, physical piece lane % PR); it fetches the logical piece that the
   // swizzle puts there.  Original row numbers are fetched one tile ahead of the rows, so a row load
   // never waits for an index load.
-  constexpr int ROWS_PER_LOAD = 64 / PR;
   constexpr int LPW = PR / 4;  // loads per wave per key tile
-  const int my_pp = lane % PR;  // physical piece of this lane's LDS slot
-  const int my_lr = lane / PR;  // row inside one load
 
   // Original rows of keys kk0 + j*ROWS_PER_LOAD + my_lr (j < LPW) of chunk ci.  The source of a chunk
   // is wave-uniform: either a run of an index array (sorted keys of the block part, or an explicit
@@ -398,7 +420,6 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
   // Loaded row numbers live in registers that only loads write (rows); consecutive rows are kept as
   // their wave-uniform first row and turned into per-lane numbers where they are used, so a register
   // with a load in flight is never overwritten by a vector instruction (which would have to wait).
-  const int idx_shift = p.idx64 ? 3 : 2;
   constexpr int ROWS_LOADED = -1, ROWS_NONE = -2;  // values of RowSource::first
   struct RowSource {
     int rows[LPW];  // valid when first == ROWS_LOADED
@@ -482,24 +503,7 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
   RowSource rows_k, rows_v;
 #pragma unroll
   for (int j = 0; j < LPW; ++j) rows_k.rows[j] = rows_v.rows[j] = 0;
-  int qrow[2];  // original row of the query a lane's S^T / O^T columns belong to
-  // sorted query positions of this head: entries of 4 or 8 bytes, the row number in the low word
-  const unsigned char* const q_idx_base = (const unsigned char*)p.q_idx + (qidx_off << idx_shift);
-  const uint32_t qi_rb = (uint32_t)p.qi_sn << idx_shift;
   {
-    int q_rows[PR];  // rows of this wave's query tile, in the order of its PR loads
-#pragma unroll
-    for (int j = 0; j < PR; ++j) {
-      // positions past the end load the index of position 0 (replaced by -1 below, once all the
-      // index loads of this prologue are in flight)
-      const int pq = wave_q_first + j * ROWS_PER_LOAD + my_lr;
-      q_rows[j] = GATHER ? *reinterpret_cast<const int*>(row_address(q_idx_base, pq < p.n_q ? pq : 0, qi_rb, 0)) : pq;
-    }
-#pragma unroll
-    for (int nb = 0; nb < 2; ++nb) {
-      const int pq = wave_q_first + nb * 32 + col;
-      qrow[nb] = GATHER ? *reinterpret_cast<const int*>(row_address(q_idx_base, pq < p.n_q ? pq : 0, qi_rb, 0)) : pq;
-    }
     RowSource rows_k1;
 #pragma unroll
     for (int j = 0; j < LPW; ++j) rows_k1.rows[j] = 0;
