@@ -141,7 +141,8 @@ def hyper_attn_func(q, k, v, q_sort_idx, k_sort_idx, block_size, sample_size=0, 
     """q, k: (batch, seqlen, nheads, headdim); v: (batch, seqlen, nheads, v_headdim);
     q_sort_idx, k_sort_idx: (batch, seqlen, nheads) permutations; returns o (batch, seqlen, nheads,
     v_headdim) and lse (batch, nheads, seqlen) fp32.  `sampled_idx` (keyword only, not in the
-    reference) lists the sampled key rows, shape (sample_size,); default 0..sample_size-1.
+    reference) lists the sampled key rows: shape (sample_size,) for one list shared by every head, or
+    (nheads, sample_size) / (batch, nheads, sample_size) for a list per head; default 0..sample_size-1.
     `resume` (keyword only, not in the reference) is a pair (o, lse) of a previous partial attention
     over other keys, shaped like the results: the kernel continues from it and updates both in place,
     which equals add_self_attentions(previous, this call) in fp32."""
@@ -189,11 +190,16 @@ def hyper_attn_func(q, k, v, q_sort_idx, k_sort_idx, block_size, sample_size=0, 
     a.q_idx_stride_b, a.q_idx_stride_h, a.q_idx_stride_n = q_sort_idx.stride(0), q_sort_idx.stride(2), q_sort_idx.stride(1)
     a.k_idx_stride_b, a.k_idx_stride_h, a.k_idx_stride_n = k_sort_idx.stride(0), k_sort_idx.stride(2), k_sort_idx.stride(1)
     keep = None
+    a.sampled_stride_b = a.sampled_stride_h = 0
     if sampled_idx is not None:
         keep = sampled_idx.to(device=q.device, dtype=q_sort_idx.dtype).contiguous()
-        assert keep.shape == (sample_size,)
+        assert keep.shape in ((sample_size,), (nheads, sample_size), (batch, nheads, sample_size)), \
+            "sampled_idx must be (sample_size,), (nheads, sample_size) or (batch, nheads, sample_size)"
         a.sampled_idx = keep.data_ptr()
-    a.sampled_stride_b = a.sampled_stride_h = 0
+        if keep.dim() >= 2:
+            a.sampled_stride_h = sample_size
+        if keep.dim() == 3:
+            a.sampled_stride_b = nheads * sample_size
     a.block_size, a.sample_size = block_size, sample_size
     a.smooth_block, a.accumulate = int(bool(smooth_block)), int(resume is not None)
     with torch.cuda.device(q.device):

@@ -231,6 +231,25 @@ def test_block_sampled_explicit_samples_int32_idx_and_ragged_tail(ha):
         assert_close(lse, rl, "hyper lse")
 
 
+@pytest.mark.parametrize("per_batch", [False, True])
+def test_block_sampled_one_sample_list_per_head(ha, per_batch):
+    """A different explicit sample list for every head (and batch entry): checked head by head against the
+    oracle, which takes one list."""
+    b, h, n, d = 2, 3, 1024, 64
+    q, k, v, qi, ki = _sorted_inputs(b, h, n, d, torch.bfloat16, 35)
+    sampled = torch.randint(0, n, (b, h, 128), generator=_gen(36))
+    if not per_batch:
+        sampled = sampled[0]
+    o, lse = _run_hyper(ha, q, k, v, qi, ki, 256, 128, None, False, sampled, torch.int32)
+    for bi in range(b):
+        for hi in range(h):
+            sl = (slice(bi, bi + 1), slice(hi, hi + 1))
+            s_list = sampled[bi, hi] if per_batch else sampled[hi]
+            ro, rl = O.block_sampled_attention(q[sl], k[sl], v[sl], qi[sl], ki[sl], 256, 128, None, False, s_list)
+            assert_close(o[sl], ro, f"hyper out b{bi} h{hi}", torch.bfloat16)
+            assert_close(lse[sl], rl, f"hyper lse b{bi} h{hi}")
+
+
 @pytest.mark.parametrize("n,block", [(128, 512), (256, 1024), (384, 512)])
 def test_block_attention_smooth_block_longer_than_sequence(ha, n, block):
     """smooth_block with a block much longer than the sequence: the window offset
