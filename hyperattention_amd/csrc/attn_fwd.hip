@@ -628,19 +628,35 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
 #define HA_PV_DRAIN()                                                                                       \
   _Pragma("unroll") for (int db = 0; db < DB; ++db) _Pragma("unroll") for (int nb = 0; nb < 2; ++nb)        \
       acc[db][nb] = Mfma<T>::run(vf[db], pb[nb], acc[db][nb]);
-#define HA_ITERATION(ci, K_RD, K_WR, V_CUR, V_WR)                                                           \
+  /* consecutive rows known to lie inside the keys: no row numbers, no bounds */                             \
+#define HA_LOAD_TILE_INSIDE(base, stride, chunk, kk0, tile, SWZ)                                            \
+  _Pragma("unroll") for (int j = 0; j < LPW; ++j) {                                                         \
+    const int r = (wave_s * LPW + j) * ROWS_PER_LOAD + my_lr;                                               \
+    const uint32_t first_row =                                                                              \
+        __builtin_amdgcn_readfirstlane((uint32_t)((chunk) * KC + (kk0) + j * ROWS_PER_LOAD) * (stride));    \
+    global_to_lds_16(row_address(base + first_row, my_lr, stride, (my_pp ^ SWZ(r)) << 4),                   \
+                     (tile) + (wave_s * LPW + j) * 1024);                                                   \
+  }
+  // INTERIOR (exact attention only): every row of the tiles the iteration loads exists and no score of
+  // the chunk it consumes is masked for any wave, so all of that bookkeeping is compiled out
+#define HA_ITERATION(ci, K_RD, K_WR, V_CUR, V_WR, INTERIOR)                                                 \
   {                                                                                                         \
-    if (__builtin_expect((ci) + 2 <= n_chunks, true)) {                                                     \
-      HA_LOAD_TILE(kb, k_rb, rows_k, (ci) + 2 + k_chunk_shift, k_kk0, K_WR, k_swizzle) /* K tile ci+2 */    \
+    if (INTERIOR) {                                                                                         \
+      HA_LOAD_TILE_INSIDE(kb, k_rb, (ci) + 2 + k_chunk_shift, k_kk0, K_WR, k_swizzle)                       \
+      HA_LOAD_TILE_INSIDE(vb, v_rb, (ci) + 1, v_kk0, V_WR, v_swizzle)                                       \
+    } else {                                                                                                \
+      if (__builtin_expect((ci) + 2 <= n_chunks, true)) {                                                   \
+        HA_LOAD_TILE(kb, k_rb, rows_k, (ci) + 2 + k_chunk_shift, k_kk0, K_WR, k_swizzle) /* K tile ci+2 */  \
+      }                                                                                                     \
+      if (__builtin_expect((ci) + 1 < n_chunks, true)) {                                                    \
+        HA_LOAD_TILE(vb, v_rb, rows_v, (ci) + 1, v_kk0, V_WR, v_swizzle) /* V tile ci+1 */                  \
+      }                                                                                                     \
+      HA_FETCH_ROWS_K((ci) + 3, rows_k)                                                                     \
+      HA_FETCH_ROWS_V((ci) + 2, rows_v)                                                                     \
     }                                                                                                       \
-    if (__builtin_expect((ci) + 1 < n_chunks, true)) {                                                      \
-      HA_LOAD_TILE(vb, v_rb, rows_v, (ci) + 1, v_kk0, V_WR, v_swizzle) /* V tile ci+1 */                    \
-    }                                                                                                       \
-    HA_FETCH_ROWS_K((ci) + 3, rows_k)                                                                       \
-    HA_FETCH_ROWS_V((ci) + 2, rows_v)                                                                       \
     /* causal: once a chunk lies wholly above this wave's queries, so do all later ones */                  \
-    if (!(CAUSAL && (ci) * KC > wave_q_first + 63)) {                                                       \
-      const bool masked = chunk_masked(ci);                                                                 \
+    if (INTERIOR || !(CAUSAL && (ci) * KC > wave_q_first + 63)) {                                           \
+      const bool masked = INTERIOR ? false : chunk_masked(ci);                                              \
       if (__builtin_expect(masked, false)) { HA_APPLY_MASK(ci, 0, s_a) }                                                             \
       half_step<T, D, 0>(s_a, s_b, K_RD, 0, V_CUR, 0, lo, qf, acc, m_run, l_run, pb, vf,                    \
                          p.scale_log2);                                                                     \
@@ -659,12 +675,25 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
     __builtin_amdgcn_s_waitcnt(0x0F70); /* this wave's parts of K tile ci+2, V tile ci+1 have landed */     \
     __syncthreads();                                                                                        \
   }
-  for (int ci = 0; ci < n_chunks; ci += 2) {
-    HA_ITERATION(ci, lds_k1, lds_k0, lds_v0, lds_v1)
-    if (ci + 1 < n_chunks) HA_ITERATION(ci + 1, lds_k0, lds_k1, lds_v1, lds_v0)
+  int ci = 0;
+  if (!GATHER) {
+    // chunks 0 .. n_interior-1 (an even number): chunk ci + 2 is not the last one, so all its rows
+    // exist, and causal chunks end at or before the first query of the workgroup
+    int n_interior = n_chunks - 3;
+    if (CAUSAL) n_interior = min(n_interior, qt * (WG_QUERIES / KC));
+    n_interior = max(n_interior, 0) & ~1;
+    for (; ci < n_interior; ci += 2) {
+      HA_ITERATION(ci, lds_k1, lds_k0, lds_v0, lds_v1, true)
+      HA_ITERATION(ci + 1, lds_k0, lds_k1, lds_v1, lds_v0, true)
+    }
+  }
+  for (; ci < n_chunks; ci += 2) {
+    HA_ITERATION(ci, lds_k1, lds_k0, lds_v0, lds_v1, false)
+    if (ci + 1 < n_chunks) HA_ITERATION(ci + 1, lds_k0, lds_k1, lds_v1, lds_v0, false)
   }
   if (pending) { HA_PV_DRAIN() }
 #undef HA_ITERATION
+#undef HA_LOAD_TILE_INSIDE
 #undef HA_PV_DRAIN
 
   // ---- epilogue: normalise, stage O through LDS, write whole rows ---------------------------------
