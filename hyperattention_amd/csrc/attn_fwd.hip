@@ -409,52 +409,46 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
   // never waits for an index load.
   constexpr int LPW = PR / 4;  // loads per wave per key tile
 
-  // Original rows of keys kk0 + j*ROWS_PER_LOAD + my_lr (j < LPW) of chunk ci.  The source of a chunk
-  // is wave-uniform: either a run of an index array (sorted keys of the block part, or an explicit
-  // sample list) or consecutive rows (default samples; exact attention needs none of this and takes
-  // its rows straight from the chunk number when it loads a tile).  Index arrays are read as
-  // 4-byte words at a stride of 4 or 8 bytes (row numbers fit the low word of an int64).  Keys past
-  // n_k and chunks outside 0..n_chunks-1 alias row 0: row 0 holds finite data and their scores are
-  // masked or never used.  Every branch is wave-uniform and nothing touches a loaded value here: the
-  // loads stay in flight until the row numbers are needed for the tile loads of a later iteration.
-  // Loaded row numbers live in registers that only loads write (rows); consecutive rows are kept as
-  // their wave-uniform first row and turned into per-lane numbers where they are used, so a register
-  // with a load in flight is never overwritten by a vector instruction (which would have to wait).
-  constexpr int ROWS_LOADED = -1, ROWS_NONE = -2;  // values of RowSource::first
+  // Gathered kernel: original rows of keys kk0 + j*ROWS_PER_LOAD + my_lr (j < LPW) of chunk ci, one
+  // register per tile load of the wave.  The source of a chunk is wave-uniform: a run of an index array
+  // (sorted keys of the block part, or an explicit sample list), consecutive rows (default samples), or
+  // nothing (chunks outside 0..n_chunks-1 read row 0: finite data whose scores are never used).  Index
+  // arrays are read as 4-byte words at a stride of 4 or 8 bytes (row numbers fit the low word of an
+  // int64).  Row numbers are fetched one iteration before the tile load that uses them and every
+  // iteration ends by waiting for all loads, so the loads stay in flight through the iteration's
+  // arithmetic, and a register is never written (by the next fetch, load or not) with a load pending.
+  // Exact attention needs none of this: its tile loads take their rows from the chunk number.
   struct RowSource {
-    int rows[LPW];  // valid when first == ROWS_LOADED
-    int first;      // >= 0: rows first + key number; ROWS_NONE: chunk out of range (row 0)
+    int rows[LPW];
   };
+  const unsigned char* const blk_idx = (const unsigned char*)p.k_idx + (kidx_off << idx_shift);
+  const uint32_t blk_idx_rb = (uint32_t)p.ki_sn << idx_shift;  // bytes between entries of the key order
+  const unsigned char* const smp_idx =
+      p.sampled_idx ? (const unsigned char*)p.sampled_idx + (sidx_off << idx_shift) : nullptr;
   auto fetch_rows = [&](int ci, int kk0, RowSource& rs) {
-    const unsigned char* src = nullptr;  // index array run, or null for consecutive rows
-    uint32_t stride = 0;                 // bytes between its entries
-    int first = 0;
-    if (GATHER) {
+    // Consecutive rows (or row 0 for every lane) are written first and without a branch; an index run
+    // then overwrites them by loads.  A vector write behind a branch that follows a load of the same
+    // register would make the compiler wait for every load in flight, the tile loads included.
+    const bool in_range = ci >= 0 && ci < n_chunks;
+    const int first = in_range ? (ci - n_blk_chunks) * KC + kk0 : 0;
+    const uint32_t per_lane = in_range ? 1u : 0u;
+#pragma unroll
+    for (int j = 0; j < LPW; ++j) rs.rows[j] = (int)__umul24((uint32_t)(j * ROWS_PER_LOAD + my_lr), per_lane) + first;
+    if (in_range) {
       if (ci < n_blk_chunks) {
         int u = uni_start + ci;  // smooth windows wrap around the key sequence
         u -= u >= nk_chunks ? nk_chunks : 0;
         u -= u >= nk_chunks ? nk_chunks : 0;
-        src = (const unsigned char*)p.k_idx + ((kidx_off + (int64_t)u * KC * p.ki_sn) << idx_shift);
-        stride = (uint32_t)p.ki_sn << idx_shift;
-      } else {
-        first = (ci - n_blk_chunks) * KC;
-        if (p.sampled_idx) {
-          src = (const unsigned char*)p.sampled_idx + ((sidx_off + first) << idx_shift);
-          stride = 1u << idx_shift;
-        }
-      }
-    } else {
-      first = ci * KC;
-    }
-    if (ci < 0 || ci >= n_chunks) {
-      rs.first = ROWS_NONE;
-    } else if (src) {
-      rs.first = ROWS_LOADED;
+        const unsigned char* const src = blk_idx + (uint32_t)(u * KC) * blk_idx_rb;
 #pragma unroll
-      for (int j = 0; j < LPW; ++j)
-        rs.rows[j] = *reinterpret_cast<const int*>(row_address(src, kk0 + j * ROWS_PER_LOAD + my_lr, stride, 0));
-    } else {
-      rs.first = first;
+        for (int j = 0; j < LPW; ++j)
+          rs.rows[j] = *reinterpret_cast<const int*>(row_address(src, kk0 + j * ROWS_PER_LOAD + my_lr, blk_idx_rb, 0));
+      } else if (smp_idx) {
+        const unsigned char* const src = smp_idx + ((uint32_t)(ci - n_blk_chunks) * KC << idx_shift);
+#pragma unroll
+        for (int j = 0; j < LPW; ++j)
+          rs.rows[j] = *reinterpret_cast<const int*>(row_address(src, kk0 + j * ROWS_PER_LOAD + my_lr, 1u << idx_shift, 0));
+      }
     }
   };
   // V tile c holds keys 0..63 of chunk c.  K tile c holds keys 32..63 of chunk c-1 in its rows 0..31
@@ -464,23 +458,22 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
   const int k_chunk_shift = (wave_s >> 1) - 1;
 #define HA_FETCH_ROWS_K(tile_c, rs) if (GATHER) fetch_rows((tile_c) + k_chunk_shift, k_kk0, rs);
 #define HA_FETCH_ROWS_V(ci, rs) if (GATHER) fetch_rows((ci), v_kk0, rs);
-// Rows listed by an index array cost a lane one multiply-add each.  Consecutive rows cost it nothing
-// per tile: the first row of the load goes into the wave-uniform base, the lane's own row and piece
-// are loop constants.  Only a tile that reaches past the last key (or lies outside the chunk range:
+// Gathered kernel: one multiply-add per lane and load turns a row number into an address.  Exact
+// attention: the first row of the load goes into the wave-uniform base, the lane's own row and piece
+// are loop constants; only a tile that reaches past the last key (or lies before the first chunk:
 // row0 < 0, every lane reads row 0) computes and clamps row numbers per lane.  All branches are
 // wave-uniform.
 #define HA_LOAD_TILE(base, stride, rs, chunk, kk0, tile, SWZ)                                            \
-  if (GATHER && rs.first == ROWS_LOADED) {                                                               \
+  if (GATHER) {                                                                                          \
     _Pragma("unroll") for (int j = 0; j < LPW; ++j) {                                                    \
       const int r = (wave_s * LPW + j) * ROWS_PER_LOAD + my_lr;                                          \
       global_to_lds_16(row_address(base, rs.rows[j], stride, (my_pp ^ SWZ(r)) << 4),                     \
                        (tile) + (wave_s * LPW + j) * 1024);                                              \
     }                                                                                                    \
   } else {                                                                                               \
-    /* exact attention: chunk c is rows 64 c ..; a chunk before the first reads row 0 */                 \
-    const int row0 = GATHER ? (rs.first == ROWS_NONE ? -1 : rs.first + (kk0))                            \
-                            : ((chunk) < 0 ? -1 : (chunk) * KC + (kk0));                                  \
-    if (__builtin_expect(row0 >= 0 && (GATHER || row0 + LPW * ROWS_PER_LOAD <= p.n_k), true)) {          \
+    /* chunk c is rows 64 c ..; a chunk before the first reads row 0 */                                  \
+    const int row0 = (chunk) < 0 ? -1 : (chunk) * KC + (kk0);                                            \
+    if (__builtin_expect(row0 >= 0 && row0 + LPW * ROWS_PER_LOAD <= p.n_k, true)) {                      \
       _Pragma("unroll") for (int j = 0; j < LPW; ++j) {                                                  \
         const int r = (wave_s * LPW + j) * ROWS_PER_LOAD + my_lr;                                        \
         const uint32_t first_row = __builtin_amdgcn_readfirstlane((uint32_t)(row0 + j * ROWS_PER_LOAD) * (stride)); \
