@@ -58,6 +58,17 @@ struct Mfma<f16_t> {
   static __device__ __forceinline__ f32x16 run(f16x8 a, f16x8 b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
   }
+  // The same MFMA with its accumulator pinned to VGPRs and its B operand to AGPRs.  A kernel that
+  // needs more than 256 registers gets the AGPR form for every MFMA the compiler selects, and a vector
+  // instruction cannot read an AGPR: accumulators that the soft-max reads (S^T) would cost a copy per
+  // value.  Written as assembly the instruction keeps them where the FMAs can use them, while the
+  // query fragments (B) sit in AGPRs for the whole kernel.  first: accumulate onto zero.
+  static __device__ __forceinline__ void run_vgpr_acc(f16x8 a, f16x8 b, f32x16& c, bool first) {
+    if (first)
+      asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "a"(b));
+    else
+      asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "a"(b));
+  }
   // c[*] + a[0] + a[1] + a[2] + a[3] on the matrix pipe: the 4x4x4 MFMA works on 16 independent
   // blocks of 4 lanes; with an all-ones A a lane's four results are all the sum of its own four B values
   static __device__ __forceinline__ f32x4 quad_sum(f16x4 a, f32x4 c) {
@@ -70,11 +81,23 @@ struct Mfma<bf16_t> {
   static __device__ __forceinline__ f32x16 run(bf16x8 a, bf16x8 b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
   }
+  static __device__ __forceinline__ void run_vgpr_acc(bf16x8 a, bf16x8 b, f32x16& c, bool first) {
+    if (first)
+      asm("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "a"(b));
+    else
+      asm("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "a"(b));
+  }
   static __device__ __forceinline__ f32x4 quad_sum(bf16x4 a, f32x4 c) {
     typedef short s16x4 __attribute__((ext_vector_type(4)));
     const bf16x4 ones = {(bf16_t)1.0f, (bf16_t)1.0f, (bf16_t)1.0f, (bf16_t)1.0f};
     return __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(__builtin_bit_cast(s16x4, ones), __builtin_bit_cast(s16x4, a), c, 0, 0, 0);
   }
+};
+
+// Head dims whose kernel needs more than 256 registers keep the S^T accumulators in VGPRs by hand.
+template <int D>
+struct S_IN_VGPR {
+  static constexpr bool value = D > 64;
 };
 
 // Workgroups are handed to the 8 XCDs round-robin by their linear id, and each XCD has its own L2.
@@ -151,16 +174,13 @@ __device__ __forceinline__ void global_to_lds_16(const void* src, unsigned char*
 
 // P of the 8 values of half-step H a lane holds per query block (elements 8H..8H+7 of its S^T
 // registers), rounded to T, and their sums.  m is the reference exponent (log2 units).
-template <typename T, int H>
-__device__ __forceinline__ void half_step_p(const f32x16 (&s_use)[2], const float (&m)[2], float scale_log2,
-                                            typename ElemTraits<T>::vec8 (&pn)[2], float (&sum)[2]) {
+// sums of the 8 values per query block of a half-step's P.  They go through the matrix pipe: v_dot2
+// does not overlap with the big MFMAs at all.
+template <typename T>
+__device__ __forceinline__ void half_step_sums(const typename ElemTraits<T>::vec8 (&pn)[2], float (&sum)[2]) {
   typedef typename ElemTraits<T>::vec4 vec4;
 #pragma unroll
   for (int nb = 0; nb < 2; ++nb) {
-#pragma unroll
-    for (int e = 0; e < 8; ++e)
-      pn[nb][e] = (T)__builtin_amdgcn_exp2f(__builtin_fmaf(s_use[nb][H * 8 + e], scale_log2, -m[nb]));
-    // the row sums go through the matrix pipe: v_dot2 does not overlap with the big MFMAs at all
     const vec4 lo = __builtin_shufflevector(pn[nb], pn[nb], 0, 1, 2, 3);
     const vec4 hi = __builtin_shufflevector(pn[nb], pn[nb], 4, 5, 6, 7);
     f32x4 acc_sum = {0.f, 0.f, 0.f, 0.f};
@@ -168,6 +188,16 @@ __device__ __forceinline__ void half_step_p(const f32x16 (&s_use)[2], const floa
     acc_sum = Mfma<T>::quad_sum(hi, acc_sum);
     sum[nb] = acc_sum[0];
   }
+}
+template <typename T, int H, bool SUMS = true>
+__device__ __forceinline__ void half_step_p(const f32x16 (&s_use)[2], const float (&m)[2], float scale_log2,
+                                            typename ElemTraits<T>::vec8 (&pn)[2], float (&sum)[2]) {
+#pragma unroll
+  for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+    for (int e = 0; e < 8; ++e)
+      pn[nb][e] = (T)__builtin_amdgcn_exp2f(__builtin_fmaf(s_use[nb][H * 8 + e], scale_log2, -m[nb]));
+  if (SUMS) half_step_sums<T>(pn, sum);
 }
 
 // The rare path of a half-step: raise the reference exponents to the row maxima of the half-step,
@@ -228,20 +258,27 @@ __device__ __forceinline__ void half_step(const f32x16 (&s_use)[2], f32x16 (&s_f
   for (int db = 0; db < DB; ++db)
 #pragma unroll
     for (int nb = 0; nb < 2; ++nb) acc[db][nb] = Mfma<T>::run(vf[db], pb[nb], acc[db][nb]);
-  if (H == 0) {
+  if (S_IN_VGPR<D>::value) {
 #pragma unroll
-    for (int nb = 0; nb < 2; ++nb)
+    for (int k2 = 0; k2 < KH; ++k2)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) s_fill[nb][i] = 0.f;
+      for (int nb = 0; nb < 2; ++nb) Mfma<T>::run_vgpr_acc(kf[k2], qf[nb][H * KH + k2], s_fill[nb], H == 0 && k2 == 0);
+  } else {
+    if (H == 0) {
+#pragma unroll
+      for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) s_fill[nb][i] = 0.f;
+    }
+#pragma unroll
+    for (int k2 = 0; k2 < KH; ++k2)
+#pragma unroll
+      for (int nb = 0; nb < 2; ++nb) s_fill[nb] = Mfma<T>::run(kf[k2], qf[nb][H * KH + k2], s_fill[nb]);
   }
-#pragma unroll
-  for (int k2 = 0; k2 < KH; ++k2)
-#pragma unroll
-    for (int nb = 0; nb < 2; ++nb) s_fill[nb] = Mfma<T>::run(kf[k2], qf[nb][H * KH + k2], s_fill[nb]);
 
   vec8 pn[2];
   float sum[2];
-  half_step_p<T, H>(s_use, m_run, scale_log2, pn, sum);
+  half_step_p<T, H, !S_IN_VGPR<D>::value>(s_use, m_run, scale_log2, pn, sum);
   // Issue order of the block: each of its 2*D/16 large MFMAs is followed by a share of the P
   // arithmetic (3 plain VALU, 2 exp), so the softmax fills the issue slots behind every MFMA instead
   // of running as one burst after the last of them.  Measured 3 % faster than the scheduler's own order.
@@ -250,6 +287,14 @@ __device__ __forceinline__ void half_step(const f32x16 (&s_use)[2], f32x16 (&s_f
     __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
     __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);  // three VALU
     __builtin_amdgcn_sched_group_barrier(0x400, 2, 0);  // two transcendental
+  }
+  if (S_IN_VGPR<D>::value) {
+    // The S^T MFMAs written as assembly get none of the compiler's wait states between an MFMA and a
+    // vector instruction that reads its result.  They are all issued before this point, the MFMAs of
+    // the sums after it, the matrix pipe completes in order, and the branch below waits for the sums:
+    // so when the next block reads S^T, those MFMAs have completed.
+    __builtin_amdgcn_sched_barrier(0);
+    half_step_sums<T>(pn, sum);
   }
   // One compare for both query blocks: their sums are >= 0 or NaN, so the total is below the limit
   // only if both are.  Not "total >= limit": a NaN (row that has seen nothing yet) must take the rare
@@ -594,14 +639,21 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
     vec8 kf[KSTEPS];
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ++ks) kf[ks] = lds_read_k<T>(lds_k0, lo.k[ks] + 32 * D * 2);
+    if (S_IN_VGPR<D>::value) {
 #pragma unroll
-    for (int nb = 0; nb < 2; ++nb)
+      for (int ks = 0; ks < KSTEPS; ++ks)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) s_a[nb][i] = 0.f;
+        for (int nb = 0; nb < 2; ++nb) Mfma<T>::run_vgpr_acc(kf[ks], qf[nb][ks], s_a[nb], ks == 0);
+    } else {
 #pragma unroll
-    for (int ks = 0; ks < KSTEPS; ++ks)
+      for (int nb = 0; nb < 2; ++nb)
 #pragma unroll
-      for (int nb = 0; nb < 2; ++nb) s_a[nb] = Mfma<T>::run(kf[ks], qf[nb][ks], s_a[nb]);
+        for (int i = 0; i < 16; ++i) s_a[nb][i] = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ++ks)
+#pragma unroll
+        for (int nb = 0; nb < 2; ++nb) s_a[nb] = Mfma<T>::run(kf[ks], qf[nb][ks], s_a[nb]);
+    }
   }
   // the P.V of "the half-step before the first" adds nothing
   vec8 pb[2], vf[DB];
