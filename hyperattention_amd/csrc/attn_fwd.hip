@@ -323,7 +323,10 @@ __device__ __forceinline__ void half_step(const f32x16 (&s_use)[2], f32x16 (&s_f
 
 }  // namespace
 
-template <typename T, int D, bool GATHER, bool CAUSAL>
+// PLAIN (gathered kernel only): the common configuration, for which the per-iteration bookkeeping of the
+// general one is compiled out: no smoothing, default samples (rows 0 .. sample_size-1), and both
+// 128-query tiles of the workgroup inside one key block, so no chunk is ever masked for half of it.
+template <typename T, int D, bool GATHER, bool CAUSAL, bool PLAIN = false>
 __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_kernel(const ha_attn_kernel_params p) {
   typedef typename ElemTraits<T>::vec8 vec8;
   typedef typename ElemTraits<T>::vec4 vec4;
@@ -418,7 +421,7 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
       int cnt = last > first ? (last - first) / KC : 0;
       if (t * 128 >= p.n_q) cnt = 0;
       int s = first / KC;
-      if (p.smooth) {
+      if (!PLAIN && p.smooth) {
         // the window starts (block_tiles - 1) * 64 keys before the tile's own keys, modulo the sequence
         // (src/hyper_attn_triton.py:101,105-106); reduced to 0..n_k-1 here, also when the block is
         // longer than the sequence, and kept behind the first tile's window for the second tile
@@ -469,7 +472,7 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
   const unsigned char* const blk_idx = (const unsigned char*)p.k_idx + (kidx_off << idx_shift);
   const uint32_t blk_idx_rb = (uint32_t)p.ki_sn << idx_shift;  // bytes between entries of the key order
   const unsigned char* const smp_idx =
-      p.sampled_idx ? (const unsigned char*)p.sampled_idx + (sidx_off << idx_shift) : nullptr;
+      !PLAIN && p.sampled_idx ? (const unsigned char*)p.sampled_idx + (sidx_off << idx_shift) : nullptr;
   auto fetch_rows = [&](int ci, int kk0, RowSource& rs) {
     // Consecutive rows (or row 0 for every lane) are written first and without a branch; an index run
     // then overwrites them by loads.  A vector write behind a branch that follows a load of the same
@@ -481,9 +484,11 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
     for (int j = 0; j < LPW; ++j) rs.rows[j] = (int)__umul24((uint32_t)(j * ROWS_PER_LOAD + my_lr), per_lane) + first;
     if (in_range) {
       if (ci < n_blk_chunks) {
-        int u = uni_start + ci;  // smooth windows wrap around the key sequence
-        u -= u >= nk_chunks ? nk_chunks : 0;
-        u -= u >= nk_chunks ? nk_chunks : 0;
+        int u = uni_start + ci;
+        if (!PLAIN) {  // smooth windows wrap around the key sequence
+          u -= u >= nk_chunks ? nk_chunks : 0;
+          u -= u >= nk_chunks ? nk_chunks : 0;
+        }
         const unsigned char* const src = blk_idx + (uint32_t)(u * KC) * blk_idx_rb;
 #pragma unroll
         for (int j = 0; j < LPW; ++j)
@@ -609,6 +614,7 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
 
   // ---- masks (wave-uniform decision per chunk) -------------------------------------------------
   auto chunk_masked = [&](int ci) -> bool {
+    if (PLAIN) return false;
     if (GATHER) return ci < n_blk_chunks && !(uni_start + ci >= my_lo && uni_start + ci < my_hi);
     const int k_first = ci * KC;
     return (CAUSAL && k_first + KC - 1 > wave_q_first) || (k_first + KC > p.n_k);
@@ -802,15 +808,19 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
 
 namespace {
 
-template <typename T, int D, bool GATHER, bool CAUSAL>
+template <typename T, int D, bool GATHER, bool CAUSAL, bool PLAIN = false>
 int launch_one(const ha_attn_kernel_params& p, int grid, hipStream_t stream, const char* what) {
-  hipLaunchKernelGGL((ha_attn_fwd_kernel<T, D, GATHER, CAUSAL>), dim3(grid), dim3(WG_THREADS), 0, stream, p);
+  hipLaunchKernelGGL((ha_attn_fwd_kernel<T, D, GATHER, CAUSAL, PLAIN>), dim3(grid), dim3(WG_THREADS), 0, stream, p);
   return ha_launch_status(what);
 }
 
 template <typename T, int D>
 int launch_variant(const ha_attn_kernel_params& p, int grid, bool gather, bool causal, hipStream_t stream) {
-  if (gather) return launch_one<T, D, true, false>(p, grid, stream, "ha_block_attn_fwd");
+  if (gather) {
+    const bool plain = !p.smooth && !p.sampled_idx && p.block_tiles % 2 == 0 && p.n_q % WG_QUERIES == 0;
+    if (plain) return launch_one<T, D, true, false, true>(p, grid, stream, "ha_block_attn_fwd");
+    return launch_one<T, D, true, false>(p, grid, stream, "ha_block_attn_fwd");
+  }
   if (causal) return launch_one<T, D, false, true>(p, grid, stream, "ha_flash_attn_fwd");
   return launch_one<T, D, false, false>(p, grid, stream, "ha_flash_attn_fwd");
 }
