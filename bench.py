@@ -31,7 +31,7 @@ MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense fp16/bf16
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the gathered attention kernel, measured with rocprofv3 --pmc (see the
 # summary of that run under profiles/); only the workload that was measured has a figure
-MEASURED_TRAFFIC_BYTES = {"c3": 1.3926e9}
+MEASURED_TRAFFIC_BYTES = {"c3": 1.3903e9}
 
 WORKLOADS = {
     # name: batch, q heads, kv heads, n, d, dtype, causal, block, sample, min_seq_len, smooth
