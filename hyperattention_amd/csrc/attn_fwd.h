@@ -3,6 +3,13 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+// x / y for 0 <= x < 2^31 as (x * magic) >> shift, with shift = 31 + ceil(log2 y) and
+// magic = floor(2^shift / y) + 1 < 2^32 (exact for every such x)
+struct ha_divisor {
+  uint32_t magic;
+  int shift;
+};
+
 struct ha_attn_kernel_params {
   const void* q;
   const void* k;
@@ -27,9 +34,9 @@ struct ha_attn_kernel_params {
   int sample_chunks;  // sample_size / 64
   int smooth, accumulate, idx64;
   float scale_log2;   // softmax scale * log2(e)
-  // log2 of the divisors of the workgroup -> (head, segment, tile) decomposition when they are powers
-  // of two, else -1 (filled by ha_attn_launch): the kernel then shifts instead of dividing
-  int qtiles_shift, segs_shift, heads_shift, kv_group_shift, block_tiles_shift;
+  // the divisors of the workgroup -> (head, segment, tile) decomposition as multiply-and-shift
+  // constants (filled by ha_attn_launch): the kernel never divides
+  ha_divisor div_qtiles, div_segs, div_heads, div_kv_group, div_block_tiles;
 };
 
 int ha_attn_launch(const ha_attn_kernel_params& p, int d, int dtype, bool gather, bool causal, hipStream_t stream);

@@ -104,13 +104,13 @@ struct S_IN_VGPR {
 // Re-number them so that every XCD works through one contiguous range of (head, query tile): the
 // query tiles that share a head's K/V then meet in the same L2.
 __device__ __forceinline__ int xcd_contiguous_id(int linear, int total) {
-  const int xcd = linear % NUM_XCD, k = linear / NUM_XCD;
-  const int q = total / NUM_XCD, r = total % NUM_XCD;
+  const int xcd = (unsigned)linear % NUM_XCD, k = (unsigned)linear / NUM_XCD;
+  const int q = (unsigned)total / NUM_XCD, r = (unsigned)total % NUM_XCD;
   return xcd * q + (xcd < r ? xcd : r) + k;
 }
 
-// x / y for non-negative x; shift = log2(y) when y is a power of two, else -1
-__device__ __forceinline__ int fast_div(int x, int y, int shift) { return shift >= 0 ? x >> shift : x / y; }
+// x / y for 0 <= x < 2^31 by the divisor's multiply-and-shift constants
+__device__ __forceinline__ int fast_div(int x, ha_divisor y) { return (int)(((uint64_t)(uint32_t)x * y.magic) >> y.shift); }
 
 // Address of 16-byte piece `piece_bytes` of row `row`: a wave-uniform base plus a 32-bit byte offset,
 // so that a lane spends one 24-bit multiply-add on it instead of a 64-bit multiplication.  The entry
@@ -359,14 +359,14 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
   // ---- which (virtual) head and query tile -----------------------------------------------------
   const int wg = xcd_contiguous_id(blockIdx.x, gridDim.x);
   const int qtiles = (p.n_q + WG_QUERIES - 1) / WG_QUERIES;
-  const int vhead = fast_div(wg, qtiles, p.qtiles_shift);
+  const int vhead = fast_div(wg, p.div_qtiles);
   // causal: the tiles with the most keys go first, so that the last workgroups of the grid are short
   const int qt_fwd = wg - vhead * qtiles;
   const int qt = CAUSAL ? qtiles - 1 - qt_fwd : qt_fwd;
-  const int bh = fast_div(vhead, p.segs, p.segs_shift);
+  const int bh = fast_div(vhead, p.div_segs);
   const int seg = vhead - bh * p.segs;
-  const int b = fast_div(bh, p.heads, p.heads_shift), h = bh - b * p.heads;
-  const int hk = fast_div(h, p.kv_group, p.kv_group_shift);
+  const int b = fast_div(bh, p.div_heads), h = bh - b * p.heads;
+  const int hk = fast_div(h, p.div_kv_group);
 
   // ---- row numbers of the queries: the first thing the workgroup has to wait for, so they are asked
   // for before the rest of the set-up (sorted query positions of this head: entries of 4 or 8 bytes,
@@ -414,7 +414,7 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
 #pragma unroll
     for (int t2 = 0; t2 < 2; ++t2) {
       const int t = qt * 2 + t2;  // reference query tile of 128
-      const int block_id = fast_div(t, p.block_tiles, p.block_tiles_shift);
+      const int block_id = fast_div(t, p.div_block_tiles);
       const int first = block_id * p.block_tiles * 128;
       int last = (block_id + 1) * p.block_tiles * 128;
       last = last < p.n_k ? last : p.n_k;
@@ -827,21 +827,24 @@ int launch_variant(const ha_attn_kernel_params& p, int grid, bool gather, bool c
 
 }  // namespace
 
-static int log2_if_pow2(int64_t v) {
-  if (v <= 0 || (v & (v - 1))) return -1;
+static ha_divisor make_divisor(int64_t y) {
+  if (y < 1) y = 1;
   int s = 0;
-  while ((int64_t(1) << s) < v) ++s;
-  return s;
+  while ((int64_t(1) << s) < y) ++s;
+  ha_divisor d;
+  d.shift = 31 + s;
+  d.magic = (uint32_t)((uint64_t(1) << d.shift) / (uint64_t)y + 1);
+  return d;
 }
 
 int ha_attn_launch(const ha_attn_kernel_params& params, int d, int dtype, bool gather, bool causal, hipStream_t stream) {
   ha_attn_kernel_params p = params;
   const int64_t qtiles = (p.n_q + WG_QUERIES - 1) / WG_QUERIES;
-  p.qtiles_shift = log2_if_pow2(qtiles);
-  p.segs_shift = log2_if_pow2(p.segs);
-  p.heads_shift = log2_if_pow2(p.heads);
-  p.kv_group_shift = log2_if_pow2(p.kv_group);
-  p.block_tiles_shift = log2_if_pow2(p.block_tiles);
+  p.div_qtiles = make_divisor(qtiles);
+  p.div_segs = make_divisor(p.segs);
+  p.div_heads = make_divisor(p.heads);
+  p.div_kv_group = make_divisor(p.kv_group);
+  p.div_block_tiles = make_divisor(p.block_tiles);
   const int64_t grid = qtiles * p.batch * p.heads * p.segs;
   if (grid <= 0 || grid >= (1ll << 31)) return ha_fail(HA_ERR_SHAPE, "attention: grid of %lld workgroups", (long long)grid);
   if (dtype == HA_F16) {
