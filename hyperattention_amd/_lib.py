@@ -16,7 +16,8 @@ _CSRC = os.path.join(_PKG, "csrc")
 _BUILD = os.path.join(_PKG, "build")
 LIB_PATH = os.path.join(_PKG, "libhyperattn.so")
 
-SOURCES = ["api.hip", "lsh_hash.hip", "bucket_sort.hip", "gather_rows.hip", "lse_merge.hip", "attn_fwd.hip"]
+SOURCES = ["api.hip", "lsh_hash.hip", "bucket_sort.hip", "gather_rows.hip", "lse_merge.hip", "attn_fwd.hip",
+           "attn_bwd.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
@@ -27,7 +28,8 @@ HIPCC_FLAGS = [
 # exported symbols, in the order of include/hyperattn.h
 SYMBOLS = [
     "ha_abi_version", "ha_last_error", "ha_lsh_hash", "ha_bucket_argsort_workspace_bytes",
-    "ha_bucket_argsort", "ha_gather_rows", "ha_block_attn_fwd", "ha_flash_attn_fwd", "ha_lse_merge",
+    "ha_bucket_argsort", "ha_gather_rows", "ha_block_attn_fwd", "ha_flash_attn_fwd",
+    "ha_attn_bwd_workspace_bytes", "ha_block_attn_bwd", "ha_flash_attn_bwd", "ha_lse_merge",
     "ha_forward_workspace_bytes", "ha_forward",
 ]
 
@@ -94,6 +96,17 @@ class BlockAttnArgs(ctypes.Structure):
     ]
 
 
+class AttnGrads(ctypes.Structure):
+    _fields_ = [
+        ("dout", ctypes.c_void_p), ("dq", ctypes.c_void_p), ("dk", ctypes.c_void_p), ("dv", ctypes.c_void_p),
+        ("do_stride_b", ctypes.c_int64), ("do_stride_h", ctypes.c_int64), ("do_stride_n", ctypes.c_int64),
+        ("dq_stride_b", ctypes.c_int64), ("dq_stride_h", ctypes.c_int64), ("dq_stride_n", ctypes.c_int64),
+        ("dk_stride_b", ctypes.c_int64), ("dk_stride_h", ctypes.c_int64), ("dk_stride_n", ctypes.c_int64),
+        ("dv_stride_b", ctypes.c_int64), ("dv_stride_h", ctypes.c_int64), ("dv_stride_n", ctypes.c_int64),
+        ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_int64),
+    ]
+
+
 class ForwardArgs(ctypes.Structure):
     _fields_ = [
         ("q", ctypes.c_void_p), ("k", ctypes.c_void_p), ("v", ctypes.c_void_p),
@@ -133,6 +146,12 @@ def _declare(lib):
     lib.ha_block_attn_fwd.argtypes = [ctypes.POINTER(BlockAttnArgs), vp]
     lib.ha_flash_attn_fwd.restype = ci
     lib.ha_flash_attn_fwd.argtypes = [ctypes.POINTER(AttnOperands), ci, vp]
+    lib.ha_attn_bwd_workspace_bytes.restype = i64
+    lib.ha_attn_bwd_workspace_bytes.argtypes = [ctypes.POINTER(AttnOperands)]
+    lib.ha_block_attn_bwd.restype = ci
+    lib.ha_block_attn_bwd.argtypes = [ctypes.POINTER(BlockAttnArgs), ctypes.POINTER(AttnGrads), vp]
+    lib.ha_flash_attn_bwd.restype = ci
+    lib.ha_flash_attn_bwd.argtypes = [ctypes.POINTER(AttnOperands), ci, ctypes.POINTER(AttnGrads), vp]
     lib.ha_lse_merge.restype = ci
     lib.ha_lse_merge.argtypes = [vp] * 6 + [i64] * 8 + [ci, vp]
     lib.ha_forward_workspace_bytes.restype = i64
@@ -151,7 +170,7 @@ def lib():
                 "(hipcc, gfx950). There is no fallback path.")
         loaded = ctypes.CDLL(LIB_PATH)
         _declare(loaded)
-        if loaded.ha_abi_version() != 2:
+        if loaded.ha_abi_version() != 3:
             raise RuntimeError("libhyperattn.so: ABI version mismatch")
         _lib = loaded
     return _lib

@@ -19,7 +19,9 @@ namespace {
 
 constexpr float LOG2E_F = 1.4426950408889634f;
 
-int check_operands(const ha_attn_operands& t, const char* who) {
+}  // namespace
+
+int ha_check_operands(const ha_attn_operands& t, const char* who) {
   HA_REQUIRE(t.q && t.k && t.v && t.out && t.lse, HA_ERR_NULL, "%s: null tensor pointer", who);
   HA_REQUIRE(t.dtype == HA_F16 || t.dtype == HA_BF16, HA_ERR_DTYPE, "%s: Only support fp16 and bf16", who);
   HA_REQUIRE(t.batch > 0 && t.heads > 0 && t.n_q > 0 && t.n_k > 0, HA_ERR_SHAPE, "%s: sizes must be positive", who);
@@ -49,6 +51,30 @@ int check_operands(const ha_attn_operands& t, const char* who) {
   return HA_OK;
 }
 
+int ha_check_block_attn_args(const ha_block_attn_args& a, const char* who) {
+  int st = ha_check_operands(a.t, who);
+  if (st != HA_OK) return st;
+  HA_REQUIRE(a.q_idx && a.k_idx, HA_ERR_NULL, "%s: null index pointer", who);
+  HA_REQUIRE(a.idx_type == HA_IDX_I32 || a.idx_type == HA_IDX_I64, HA_ERR_DTYPE, "%s: bad idx_type", who);
+  HA_REQUIRE(a.t.n_k % 128 == 0, HA_ERR_SHAPE, "%s: keys sequence length must be divisible by 128", who);
+  HA_REQUIRE(a.t.n_q % 128 == 0, HA_ERR_SHAPE, "%s: query sequence length must be divisible by 128", who);
+  HA_REQUIRE(a.sample_size >= 0 && a.sample_size % 128 == 0, HA_ERR_SHAPE,
+             "%s: sample_size must be a non-negative multiple of 128", who);
+  HA_REQUIRE(a.block_size > 0, HA_ERR_SHAPE, "%s: block_size must be positive", who);
+  HA_REQUIRE(a.sampled_idx || a.sample_size <= a.t.n_k, HA_ERR_SHAPE,
+             "%s: default sampled rows 0..sample_size-1 exceed the key length", who);
+  {
+    const int64_t esz = a.idx_type == HA_IDX_I64 ? 8 : 4;
+    HA_REQUIRE(a.q_idx_stride_n > 0 && a.k_idx_stride_n > 0 && a.q_idx_stride_n * esz < (1ll << 24) &&
+                   a.k_idx_stride_n * esz < (1ll << 24) && (a.t.n_q - 1) * a.q_idx_stride_n * esz < (1ll << 32) &&
+                   (a.t.n_k - 1) * a.k_idx_stride_n * esz < (1ll << 32),
+               HA_ERR_UNSUPPORTED, "%s: index strides must be positive, below 16 MiB, and span 4 GiB at most", who);
+  }
+  return HA_OK;
+}
+
+namespace {
+
 void fill_params(const ha_attn_operands& t, ha_attn_kernel_params& p) {
   p.q = t.q; p.k = t.k; p.v = t.v; p.out = t.out; p.lse = t.lse;
   p.q_idx = nullptr; p.k_idx = nullptr; p.sampled_idx = nullptr;
@@ -68,24 +94,8 @@ void fill_params(const ha_attn_operands& t, ha_attn_kernel_params& p) {
 }
 
 int block_attn(const ha_block_attn_args& a, hipStream_t stream) {
-  int st = check_operands(a.t, "ha_block_attn_fwd");
+  int st = ha_check_block_attn_args(a, "ha_block_attn_fwd");
   if (st != HA_OK) return st;
-  HA_REQUIRE(a.q_idx && a.k_idx, HA_ERR_NULL, "ha_block_attn_fwd: null index pointer");
-  HA_REQUIRE(a.idx_type == HA_IDX_I32 || a.idx_type == HA_IDX_I64, HA_ERR_DTYPE, "ha_block_attn_fwd: bad idx_type");
-  HA_REQUIRE(a.t.n_k % 128 == 0, HA_ERR_SHAPE, "ha_block_attn_fwd: keys sequence length must be divisible by 128");
-  HA_REQUIRE(a.t.n_q % 128 == 0, HA_ERR_SHAPE, "ha_block_attn_fwd: query sequence length must be divisible by 128");
-  HA_REQUIRE(a.sample_size >= 0 && a.sample_size % 128 == 0, HA_ERR_SHAPE,
-             "ha_block_attn_fwd: sample_size must be a non-negative multiple of 128");
-  HA_REQUIRE(a.block_size > 0, HA_ERR_SHAPE, "ha_block_attn_fwd: block_size must be positive");
-  HA_REQUIRE(a.sampled_idx || a.sample_size <= a.t.n_k, HA_ERR_SHAPE,
-             "ha_block_attn_fwd: default sampled rows 0..sample_size-1 exceed the key length");
-  {
-    const int64_t esz = a.idx_type == HA_IDX_I64 ? 8 : 4;
-    HA_REQUIRE(a.q_idx_stride_n > 0 && a.k_idx_stride_n > 0 && a.q_idx_stride_n * esz < (1ll << 24) &&
-                   a.k_idx_stride_n * esz < (1ll << 24) && (a.t.n_q - 1) * a.q_idx_stride_n * esz < (1ll << 32) &&
-                   (a.t.n_k - 1) * a.k_idx_stride_n * esz < (1ll << 32),
-               HA_ERR_UNSUPPORTED, "ha_block_attn_fwd: index strides must be positive, below 16 MiB, and span 4 GiB at most");
-  }
   ha_attn_kernel_params p;
   fill_params(a.t, p);
   p.q_idx = a.q_idx; p.k_idx = a.k_idx; p.sampled_idx = a.sampled_idx;
@@ -101,7 +111,7 @@ int block_attn(const ha_block_attn_args& a, hipStream_t stream) {
 }
 
 int flash_attn(const ha_attn_operands& t, int causal, int accumulate, hipStream_t stream) {
-  int st = check_operands(t, "ha_flash_attn_fwd");
+  int st = ha_check_operands(t, "ha_flash_attn_fwd");
   if (st != HA_OK) return st;
   ha_attn_kernel_params p;
   fill_params(t, p);

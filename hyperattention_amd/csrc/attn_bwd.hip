@@ -1,0 +1,673 @@
+// MFMA attention backward kernels for gfx950: gradients of the sorted block-diagonal + sampled-column
+// attention and of exact (flash) attention with respect to q, k and v.
+//
+// Reference semantics: _hyper_attn_backward with _bwd_preprocess_do_o_dot,
+// _bwd_permuted_block_diagonal_kernel and _bwd_sampled_col_kernel (src/hyper_attn_triton.py:195-665,
+// :745-893) and _flash_attn_backward (src/flash_attn_triton.py:270-792, :875-992): given dO, the
+// forward's O and its log-sum-exp L (a gradient arriving for L itself is ignored, as in
+// HyperAttnFunc.backward, src/hyper_attn_triton.py:922-945),
+//   D_i  = sum_c dO_ic O_ic,            P_ij = exp(scale q_i.k_j - L_i),
+//   dV_j = sum_i P_ij dO_i,             dS_ij = P_ij (dO_i.v_j - D_i) scale,
+//   dQ_i = sum_j dS_ij k_j,             dK_j = sum_i dS_ij q_i,
+// over exactly the (query, key) pairs the forward visits: a key that is both in a query's block and in
+// the sample list counts twice.  P and dS are rounded to the input type before the products, as the
+// reference does.
+//
+// One kernel body serves five passes.  A workgroup of 4 waves keeps 128 "stationary" rows (32 per
+// wave, as B operands in registers) and streams tiles of 64 rows of the other side through LDS:
+//   dQ passes    stationary = queries (Q, dO), streamed = keys (K, V):      dQ^T += K^T dS^T
+//   dK/dV passes stationary = keys (K, V),     streamed = queries (Q, dO):  dK^T += Q^T dS, dV^T += dO^T P
+// Both compute S' = Y1 X1^T and dP' = Y2 X2^T (streamed rows as MFMA rows, stationary rows as MFMA
+// columns), so a lane holds 16 streamed rows of ONE stationary row and P', dS' are the B operands of
+// the products that follow, whose A operands (Y^T) come from the transposing LDS reads.  The dQ passes
+// see all keys of a query in one workgroup and store dQ; the dK/dV passes add into fp32 accumulators
+// in HBM with atomics (a key receives contributions from its block, from the sample list, and from
+// every query head of its group), which a last kernel rounds to the output type.
+#include "ha_common.h"
+#include "attn_tiles.h"
+#include "attn_fwd.h"
+#include "attn_bwd.h"
+
+namespace {
+
+constexpr int WG_THREADS = 256;
+constexpr int ST_ROWS = 128;       // stationary rows per workgroup
+constexpr int YC = 64;             // streamed rows per LDS tile
+constexpr int MAX_SMOOTH_TILES = 1024;  // query tiles that can attend one 128-key tile (smoothed blocks)
+
+template <typename T, int D, int PASS, bool CAUSAL>
+__global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_bwd_kernel(const ha_attn_bwd_params p) {
+  typedef typename ElemTraits<T>::vec8 vec8;
+  typedef typename ElemTraits<T>::vec4 vec4;
+  constexpr bool KEY_ST = PASS == HA_BWD_DKV_EXACT || PASS == HA_BWD_DKV_BLOCK || PASS == HA_BWD_DKV_SAMPLED;
+  constexpr int KSTEPS = D / 16;  // MFMA k-steps over the head dim
+  constexpr int DB = D / 32;      // 32-row blocks of the transposed gradients
+  constexpr int PR = D / 8;       // 16-byte pieces per row
+  constexpr int RPL = 64 / PR;    // rows per tile load (one load = 64 lanes x 16 bytes)
+  constexpr int LPW = PR / 4;     // tile loads per wave per tile
+  constexpr int TILE_BYTES = YC * D * 2;
+
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_y1[2][TILE_BYTES];
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_y2[2][TILE_BYTES];
+  __shared__ __attribute__((aligned(16))) float lds_lse[2][YC];    // dK/dV passes: L (log2 units) of the streamed queries
+  __shared__ __attribute__((aligned(16))) float lds_delta[2][YC];  // and their D
+  __shared__ int lds_tiles[PASS == HA_BWD_DKV_BLOCK ? MAX_SMOOTH_TILES : 1];
+  __shared__ int lds_ntiles;
+
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6, lane = tid & 63;
+  const int wave_s = __builtin_amdgcn_readfirstlane(wave);
+  const int hi = lane >> 5, col = lane & 31;
+
+  // ---- which head, which stationary tile ------------------------------------------------------
+  const int st_total = PASS == HA_BWD_DKV_SAMPLED ? p.sample_size : (KEY_ST ? p.n_k : p.n_q);
+  const int st_tiles = (st_total + ST_ROWS - 1) / ST_ROWS;
+  const int splits = PASS == HA_BWD_DKV_SAMPLED ? (p.n_q + p.q_split - 1) / p.q_split : 1;
+  int rest = blockIdx.x;
+  const int tile = rest % st_tiles;
+  rest /= st_tiles;
+  const int split = rest % splits;
+  const int bh = rest / splits;
+  const int b = bh / p.heads, h = bh - b * p.heads;
+  const int hk = h / p.kv_group;
+  const int kv_heads = p.heads / p.kv_group;
+
+  const unsigned char* const qb = (const unsigned char*)((const T*)p.q + b * p.q_sb + h * p.q_sh);
+  const unsigned char* const kb = (const unsigned char*)((const T*)p.k + b * p.k_sb + hk * p.k_sh);
+  const unsigned char* const vb = (const unsigned char*)((const T*)p.v + b * p.v_sb + hk * p.v_sh);
+  const unsigned char* const dob = (const unsigned char*)((const T*)p.dout + b * p.do_sb + h * p.do_sh);
+  const uint32_t q_rb = (uint32_t)p.q_sn * 2, k_rb = (uint32_t)p.k_sn * 2, v_rb = (uint32_t)p.v_sn * 2,
+                 do_rb = (uint32_t)p.do_sn * 2;
+  const float* const lse_b = p.lse + b * p.lse_sb + h * p.lse_sh;
+  const float* const delta_b = p.delta + (int64_t)bh * p.n_q;
+  const int idx_shift = p.idx64 ? 3 : 2;
+  const unsigned char* const q_idx = (const unsigned char*)p.q_idx + ((b * p.qi_sb + h * p.qi_sh) << idx_shift);
+  const unsigned char* const k_idx = (const unsigned char*)p.k_idx + ((b * p.ki_sb + hk * p.ki_sh) << idx_shift);
+  const unsigned char* const s_idx =
+      p.sampled_idx ? (const unsigned char*)p.sampled_idx + ((b * p.si_sb + hk * p.si_sh) << idx_shift) : nullptr;
+  const uint32_t qi_rb = (uint32_t)p.qi_sn << idx_shift, ki_rb = (uint32_t)p.ki_sn << idx_shift;
+  const uint32_t si_rb = 1u << idx_shift;
+
+  // stationary (X) and streamed (Y) operands of this pass
+  const unsigned char* const x1b = KEY_ST ? kb : qb;
+  const unsigned char* const x2b = KEY_ST ? vb : dob;
+  const uint32_t x1_rb = KEY_ST ? k_rb : q_rb, x2_rb = KEY_ST ? v_rb : do_rb;
+  const unsigned char* const y1b = KEY_ST ? qb : kb;
+  const unsigned char* const y2b = KEY_ST ? dob : vb;
+  const uint32_t y1_rb = KEY_ST ? q_rb : k_rb, y2_rb = KEY_ST ? do_rb : v_rb;
+  const int n_y = KEY_ST ? p.n_q : p.n_k;  // rows on the streamed side
+
+  // ---- the stationary row of this lane's MFMA column ------------------------------------------
+  const int st_pos = tile * ST_ROWS + wave * 32 + col;  // position in the stationary order
+  const bool st_valid = st_pos < st_total;
+  int st_row;  // original row
+  {
+    const int pos = st_valid ? st_pos : 0;
+    if (PASS == HA_BWD_DQ_BLOCK)
+      st_row = *reinterpret_cast<const int*>(row_address(q_idx, pos, qi_rb, 0));
+    else if (PASS == HA_BWD_DKV_BLOCK)
+      st_row = *reinterpret_cast<const int*>(row_address(k_idx, pos, ki_rb, 0));
+    else if (PASS == HA_BWD_DKV_SAMPLED)
+      st_row = s_idx ? *reinterpret_cast<const int*>(row_address(s_idx, pos, si_rb, 0)) : pos;
+    else
+      st_row = pos;
+  }
+  vec8 x1f[KSTEPS], x2f[KSTEPS];
+#pragma unroll
+  for (int ks = 0; ks < KSTEPS; ++ks) {
+    x1f[ks] = *reinterpret_cast<const vec8*>(row_address(x1b, st_row, x1_rb, (ks * 16 + hi * 8) * 2));
+    x2f[ks] = *reinterpret_cast<const vec8*>(row_address(x2b, st_row, x2_rb, (ks * 16 + hi * 8) * 2));
+  }
+  float st_lse2 = 0.f, st_delta = 0.f;  // dQ passes: the lane's query
+  if (!KEY_ST) {
+    st_lse2 = lse_b[st_row] * LOG2E;
+    st_delta = delta_b[st_row];
+  }
+
+  // ---- the streamed chunks of this workgroup ---------------------------------------------------
+  const int T_blk = p.block_tiles;
+  const int nkc = p.n_k / YC;  // gathered passes: n_k % 128 == 0
+  int nc = 0;                  // number of streamed chunks
+  int y_first = 0;             // exact / sampled passes: first streamed row
+  int y_end = n_y;             // exact / sampled passes: end of the valid streamed rows
+  int blk_start = 0, n_blk = 0;  // dQ of the gathered kernel: first chunk (sorted keys) and count of the block part
+  int t_first = 0;               // dK/dV of the block part, plain blocks: first attending query tile
+  if (PASS == HA_BWD_DQ_EXACT) {
+    if (CAUSAL) {
+      const int qend = (tile + 1) * ST_ROWS;
+      y_end = y_end < qend ? y_end : qend;
+    }
+    nc = (y_end + YC - 1) / YC;
+  } else if (PASS == HA_BWD_DKV_EXACT) {
+    y_first = CAUSAL ? tile * ST_ROWS : 0;
+    nc = y_end > y_first ? (y_end - y_first + YC - 1) / YC : 0;
+  } else if (PASS == HA_BWD_DKV_SAMPLED) {
+    y_first = split * p.q_split;
+    const int e = y_first + p.q_split;
+    y_end = e < p.n_q ? e : p.n_q;
+    nc = (y_end - y_first + YC - 1) / YC;
+  } else if (PASS == HA_BWD_DQ_BLOCK) {
+    // the key window of reference query tile `tile` (src/hyper_attn_triton.py:99-107)
+    const int block_id = tile / T_blk;
+    const int first = block_id * T_blk * 128;
+    int last = first + T_blk * 128;
+    last = last < p.n_k ? last : p.n_k;
+    n_blk = last > first ? (last - first) / YC : 0;
+    blk_start = first / YC;
+    if (p.smooth) {
+      int sk = (tile * 128 - (T_blk - 1) * 64) % p.n_k;
+      sk += sk < 0 ? p.n_k : 0;
+      blk_start = sk / YC;
+    }
+    nc = n_blk + p.sample_size / YC;
+  } else {  // HA_BWD_DKV_BLOCK: the query tiles whose window holds this key tile
+    const int n_qt = p.n_q / 128;
+    if (!p.smooth) {
+      const int block_id = tile / T_blk;
+      t_first = block_id * T_blk;
+      int t_last = t_first + T_blk;
+      t_last = t_last < n_qt ? t_last : n_qt;
+      nc = t_last > t_first ? 2 * (t_last - t_first) : 0;
+    } else {
+      // list them (ascending), with one flag per 64-key half of this tile: bit 30 lower, bit 31 upper
+      if (wave_s == 0) {
+        int count = 0;
+        for (int t0 = 0; t0 < n_qt; t0 += 64) {
+          const int t = t0 + lane;
+          bool m0 = false, m1 = false;
+          if (t < n_qt) {
+            const int block_id = t / T_blk;
+            const int first = block_id * T_blk * 128;
+            int last = first + T_blk * 128;
+            last = last < p.n_k ? last : p.n_k;
+            const int cnt = last > first ? (last - first) / YC : 0;
+            int sk = (t * 128 - (T_blk - 1) * 64) % p.n_k;
+            sk += sk < 0 ? p.n_k : 0;
+            int o0 = 2 * tile - sk / YC;
+            o0 += o0 < 0 ? nkc : 0;
+            int o1 = 2 * tile + 1 - sk / YC;
+            o1 += o1 < 0 ? nkc : 0;
+            m0 = o0 < cnt;
+            m1 = o1 < cnt;
+          }
+          const bool any = m0 || m1;
+          const uint64_t mask = __ballot(any);
+          if (any) {
+            const int pos = count + __popcll(mask & ((1ull << lane) - 1));
+            if (pos < MAX_SMOOTH_TILES) lds_tiles[pos] = t | (m0 ? 1 << 30 : 0) | (m1 ? (int)(1u << 31) : 0);
+          }
+          count += __popcll(mask);
+        }
+        if (lane == 0) lds_ntiles = count < MAX_SMOOTH_TILES ? count : MAX_SMOOTH_TILES;
+      }
+      __syncthreads();
+      nc = 2 * lds_ntiles;
+    }
+  }
+  nc = __builtin_amdgcn_readfirstlane(nc);
+
+  // Original row of streamed row r (0..63) of chunk c, clamped to rows that exist; chunks past the
+  // end repeat the last one.  Gathered passes read an index array here.
+  auto attending_tile = [&](int k) -> int {  // dK/dV of the block part: k-th attending query tile with its flags
+    if (PASS != HA_BWD_DKV_BLOCK) return 0;
+    return p.smooth ? lds_tiles[k] : ((t_first + k) | (int)(3u << 30));
+  };
+  auto stream_row = [&](int c, int r) -> int {
+    c = c < nc ? c : nc - 1;
+    if (PASS == HA_BWD_DQ_BLOCK) {
+      if (c < n_blk) {
+        int u = blk_start + c;
+        u -= u >= nkc ? nkc : 0;
+        return *reinterpret_cast<const int*>(row_address(k_idx, u * YC + r, ki_rb, 0));
+      }
+      const int s = (c - n_blk) * YC + r;
+      return s_idx ? *reinterpret_cast<const int*>(row_address(s_idx, s, si_rb, 0)) : s;
+    } else if (PASS == HA_BWD_DKV_BLOCK) {
+      const int t = attending_tile(c >> 1) & 0x3fffffff;
+      return *reinterpret_cast<const int*>(row_address(q_idx, t * 128 + (c & 1) * YC + r, qi_rb, 0));
+    } else {
+      const int row = y_first + c * YC + r;
+      return row < n_y ? row : n_y - 1;
+    }
+  };
+
+  if (nc <= 0) {
+    // nothing attends (or is attended by) this tile: its gradient is zero
+    if (!KEY_ST && st_valid) {
+      unsigned char* const dqb = (unsigned char*)((T*)p.dq + b * p.dq_sb + h * p.dq_sh) + (int64_t)st_row * p.dq_sn * 2;
+      const vec4 zero = {(T)0.f, (T)0.f, (T)0.f, (T)0.f};
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) *reinterpret_cast<vec4*>(dqb + (32 * db + 8 * g + 4 * hi) * 2) = zero;
+    }
+    return;
+  }
+
+  // ---- tile loads: HBM -> LDS, 16 bytes per lane, whole rows, swizzle applied on the source side ----
+  const int my_pp = lane % PR;  // physical piece of this lane's LDS slot
+  const int my_lr = lane / PR;  // row inside one tile load
+  int rows_next[LPW];           // source rows of this wave's loads of the next tile
+  int stat_row_next = 0;        // wave 0, dK/dV passes: source row of streamed row `lane` of the next tile
+  float stat_lse = 0.f, stat_delta = 0.f;
+  auto fetch_rows = [&](int c) {
+#pragma unroll
+    for (int j = 0; j < LPW; ++j) rows_next[j] = stream_row(c, (wave_s * LPW + j) * RPL + my_lr);
+    if (KEY_ST && wave_s == 0) stat_row_next = stream_row(c, lane);
+  };
+  auto load_tile = [&](int buf) {  // the tile whose rows are in rows_next
+#pragma unroll
+    for (int j = 0; j < LPW; ++j) {
+      const int r = (wave_s * LPW + j) * RPL + my_lr;
+      const uint32_t piece = (uint32_t)((my_pp ^ v_swizzle(r)) << 4);
+      unsigned char* const dst1 = lds_y1[buf] + (wave_s * LPW + j) * 1024;
+      unsigned char* const dst2 = lds_y2[buf] + (wave_s * LPW + j) * 1024;
+      global_to_lds_16(row_address(y1b, rows_next[j], y1_rb, piece), dst1);
+      global_to_lds_16(row_address(y2b, rows_next[j], y2_rb, piece), dst2);
+    }
+    if (KEY_ST && wave_s == 0) {
+      stat_lse = lse_b[stat_row_next] * LOG2E;
+      stat_delta = delta_b[stat_row_next];
+    }
+  };
+
+  fetch_rows(0);
+  load_tile(0);
+  fetch_rows(1);
+
+  // per-lane LDS offsets of the operand reads
+  int off_rows[KSTEPS];  // piece of k-step ks of tile row lane%32, 16-byte read
+#pragma unroll
+  for (int ks = 0; ks < KSTEPS; ++ks) off_rows[ks] = v_tile_offset<D>(col, ks * 2 + hi);
+  int off_tr[DB];  // transposing read: streamed rows 0..3 (+4 for the upper lane half), column word of block db
+  {
+    const int g = lane >> 4, sl = lane & 15;
+    const int key = (g >> 1) * 4 + (sl >> 2);
+    const int w = sl & 3;
+#pragma unroll
+    for (int db = 0; db < DB; ++db) off_tr[db] = v_tile_offset<D>(key, db * 4 + (g & 1) * 2 + (w >> 1)) + (w & 1) * 8;
+  }
+
+  f32x16 acc1[DB], acc2[DB];  // dQ^T, or dK^T and dV^T: rows = head dim, column = the lane's stationary row
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      acc1[db][i] = 0.f;
+      acc2[db][i] = 0.f;
+    }
+
+  for (int c = 0; c < nc; ++c) {
+    const int buf = c & 1;
+    if (KEY_ST && wave_s == 0) {
+      lds_lse[buf][lane] = stat_lse;
+      lds_delta[buf][lane] = stat_delta;
+    }
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's part of tile c has landed
+    __syncthreads();
+    if (c + 1 < nc) {
+      load_tile(buf ^ 1);
+      fetch_rows(c + 2);
+    }
+
+    // does this wave take part in the chunk at all (smoothed blocks: the window of a query tile can end
+    // between the two 64-key halves of the stationary tile)
+    bool wave_in = true;
+    if (PASS == HA_BWD_DKV_BLOCK) wave_in = (attending_tile(c >> 1) >> (30 + (wave_s >> 1))) & 1;
+
+    if (wave_in) {
+      const unsigned char* const y1 = lds_y1[buf];
+      const unsigned char* const y2 = lds_y2[buf];
+      f32x16 s[2], dp[2];
+#pragma unroll
+      for (int rb = 0; rb < 2; ++rb) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          s[rb][i] = 0.f;
+          dp[rb][i] = 0.f;
+        }
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ++ks) {
+          const vec8 a1 = lds_read_k<T>(y1, off_rows[ks] + rb * 32 * D * 2);
+          const vec8 a2 = lds_read_k<T>(y2, off_rows[ks] + rb * 32 * D * 2);
+          s[rb] = Mfma<T>::run(a1, x1f[ks], s[rb]);
+          dp[rb] = Mfma<T>::run(a2, x2f[ks], dp[rb]);
+        }
+      }
+
+      // P' and dS' of the lane's 32 (streamed row, stationary row) pairs, rounded to the input type
+      vec8 pb[2][2], dsb[2][2];
+#pragma unroll
+      for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const int r0 = rb * 32 + g * 8 + hi * 4;  // streamed rows r0..r0+3 of the chunk
+          f32x4 l4 = {st_lse2, st_lse2, st_lse2, st_lse2}, d4 = {st_delta, st_delta, st_delta, st_delta};
+          if (KEY_ST) {
+            l4 = *reinterpret_cast<const f32x4*>(&lds_lse[buf][r0]);
+            d4 = *reinterpret_cast<const f32x4*>(&lds_delta[buf][r0]);
+          }
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const int i = g * 4 + e;
+            bool ok = true;
+            if (PASS == HA_BWD_DQ_EXACT) {
+              const int key = c * YC + r0 + e;
+              ok = key < p.n_k && (!CAUSAL || key <= st_pos);
+            } else if (PASS == HA_BWD_DKV_EXACT) {
+              const int query = y_first + c * YC + r0 + e;
+              ok = query < p.n_q && (!CAUSAL || st_pos <= query);
+            } else if (PASS == HA_BWD_DKV_SAMPLED) {
+              ok = y_first + c * YC + r0 + e < y_end;
+            }
+            float pv = __builtin_amdgcn_exp2f(__builtin_fmaf(s[rb][i], p.scale_log2, -l4[e]));
+            pv = ok ? pv : 0.f;
+            const float dsv = pv * (dp[rb][i] - d4[e]) * p.scale;
+            pb[rb][i >> 3][i & 7] = (T)pv;
+            dsb[rb][i >> 3][i & 7] = (T)dsv;
+          }
+        }
+
+      // the products that contract over the streamed rows
+#pragma unroll
+      for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+        for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+          for (int db = 0; db < DB; ++db) {
+            const int row_off = (rb * 32 + kk * 16) * D * 2;
+            const vec8 t1 = lds_read_vt<T>(y1, off_tr[db] + row_off, D * 2);
+            acc1[db] = Mfma<T>::run(t1, dsb[rb][kk], acc1[db]);
+            if (KEY_ST) {
+              const vec8 t2 = lds_read_vt<T>(y2, off_tr[db] + row_off, D * 2);
+              acc2[db] = Mfma<T>::run(t2, pb[rb][kk], acc2[db]);
+            }
+          }
+    }
+  }
+
+  // ---- results -------------------------------------------------------------------------------
+  if (!st_valid) return;
+  if (!KEY_ST) {
+    unsigned char* const dqb = (unsigned char*)((T*)p.dq + b * p.dq_sb + h * p.dq_sh) + (int64_t)st_row * p.dq_sn * 2;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        vec4 o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o[e] = (T)acc1[db][g * 4 + e];
+        *reinterpret_cast<vec4*>(dqb + (32 * db + 8 * g + 4 * hi) * 2) = o;
+      }
+  } else {
+    const int64_t head_off = ((int64_t)(b * kv_heads + hk) * p.n_k + st_row) * D;
+    float* const dk_row = p.dk32 + head_off;
+    float* const dv_row = p.dv32 + head_off;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int dd = 32 * db + 8 * (i >> 2) + 4 * hi + (i & 3);
+        unsafeAtomicAdd(dk_row + dd, acc1[db][i]);
+        unsafeAtomicAdd(dv_row + dd, acc2[db][i]);
+      }
+  }
+}
+
+// D_i = sum_c dO_ic O_ic (src/hyper_attn_triton.py:195-226): one 16-byte piece per lane, a row per
+// group of D/8 lanes
+template <typename T, int D>
+__global__ __launch_bounds__(256) void ha_bwd_delta_kernel(const T* __restrict__ out, const T* __restrict__ dout,
+                                                           float* __restrict__ delta, int heads, int n_q, int64_t o_sb,
+                                                           int64_t o_sh, int64_t o_sn, int64_t do_sb, int64_t do_sh,
+                                                           int64_t do_sn, int64_t total_rows) {
+  typedef typename ElemTraits<T>::vec8 vec8;
+  constexpr int PR = D / 8;
+  const int64_t item = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t grow = item / PR;
+  const int piece = (int)(item % PR);
+  float acc = 0.f;
+  if (grow < total_rows) {
+    const int64_t bh = grow / n_q;
+    const int row = (int)(grow - bh * n_q);
+    const int64_t b = bh / heads, h = bh - b * heads;
+    const vec8 o = *reinterpret_cast<const vec8*>(out + b * o_sb + h * o_sh + row * o_sn + piece * 8);
+    const vec8 g = *reinterpret_cast<const vec8*>(dout + b * do_sb + h * do_sh + row * do_sn + piece * 8);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc += (float)o[e] * (float)g[e];
+  }
+#pragma unroll
+  for (int m = 1; m < PR; m <<= 1) acc += __shfl_xor(acc, m);
+  if (grow < total_rows && piece == 0) delta[grow] = acc;
+}
+
+__global__ __launch_bounds__(256) void ha_bwd_zero_kernel(f32x4* __restrict__ buf, int64_t n4) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n4) buf[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+}
+
+// fp32 accumulators (batch, kv_heads, n_k, D) -> dk, dv in the output type, 8 elements per lane
+template <typename T, int D>
+__global__ __launch_bounds__(256) void ha_bwd_round_kernel(const float* __restrict__ dk32, const float* __restrict__ dv32,
+                                                           T* __restrict__ dk, T* __restrict__ dv, int kv_heads, int n_k,
+                                                           int64_t dk_sb, int64_t dk_sh, int64_t dk_sn, int64_t dv_sb,
+                                                           int64_t dv_sh, int64_t dv_sn, int64_t total_rows) {
+  typedef typename ElemTraits<T>::vec8 vec8;
+  constexpr int PR = D / 8;
+  const int64_t item = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t grow = item / PR;
+  const int piece = (int)(item % PR);
+  if (grow >= total_rows) return;
+  const int64_t bh = grow / n_k;
+  const int row = (int)(grow - bh * n_k);
+  const int64_t b = bh / kv_heads, h = bh - b * kv_heads;
+  const f32x4* const sk = reinterpret_cast<const f32x4*>(dk32 + grow * D + piece * 8);
+  const f32x4* const sv = reinterpret_cast<const f32x4*>(dv32 + grow * D + piece * 8);
+  const f32x4 k0 = sk[0], k1 = sk[1], v0 = sv[0], v1 = sv[1];
+  vec8 ok, ov;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    ok[e] = (T)k0[e];
+    ok[4 + e] = (T)k1[e];
+    ov[e] = (T)v0[e];
+    ov[4 + e] = (T)v1[e];
+  }
+  *reinterpret_cast<vec8*>(dk + b * dk_sb + h * dk_sh + row * dk_sn + piece * 8) = ok;
+  *reinterpret_cast<vec8*>(dv + b * dv_sb + h * dv_sh + row * dv_sn + piece * 8) = ov;
+}
+
+template <typename T, int D, int PASS, bool CAUSAL>
+int launch_pass(const ha_attn_bwd_params& p, int64_t grid, hipStream_t stream, const char* what) {
+  if (grid <= 0) return HA_OK;
+  if (grid >= (1ll << 31)) return ha_fail(HA_ERR_SHAPE, "%s: grid of %lld workgroups", what, (long long)grid);
+  hipLaunchKernelGGL((ha_attn_bwd_kernel<T, D, PASS, CAUSAL>), dim3((unsigned)grid), dim3(WG_THREADS), 0, stream, p);
+  return ha_launch_status(what);
+}
+
+inline int64_t align256(int64_t v) { return (v + 255) & ~(int64_t)255; }
+
+struct Workspace {
+  float* delta;
+  float* dk32;
+  float* dv32;
+  int64_t acc_floats;  // per accumulator
+  int64_t bytes;
+};
+
+Workspace carve(const ha_attn_operands& t, void* base) {
+  Workspace w;
+  const int64_t delta_bytes = align256(t.batch * t.heads * t.n_q * 4);
+  w.acc_floats = t.batch * (t.heads / t.kv_group) * t.n_k * t.d;
+  const int64_t acc_bytes = align256(w.acc_floats * 4);
+  w.delta = (float*)base;
+  w.dk32 = (float*)((char*)base + delta_bytes);
+  w.dv32 = (float*)((char*)base + delta_bytes + acc_bytes);
+  w.bytes = delta_bytes + 2 * acc_bytes;
+  return w;
+}
+
+int check_grads(const ha_attn_operands& t, const ha_attn_grads& g, const char* who) {
+  HA_REQUIRE(g.dout && g.dq && g.dk && g.dv, HA_ERR_NULL, "%s: null gradient pointer", who);
+  HA_REQUIRE(t.segs == 1 && t.q_seg_offset == 0 && t.k_seg_offset == 0, HA_ERR_UNSUPPORTED,
+             "%s: the backward takes whole heads (segs == 1, no segment offsets)", who);
+  const int64_t strides[] = {g.do_stride_b, g.do_stride_h, g.do_stride_n, g.dq_stride_b, g.dq_stride_h, g.dq_stride_n,
+                             g.dk_stride_b, g.dk_stride_h, g.dk_stride_n, g.dv_stride_b, g.dv_stride_h, g.dv_stride_n};
+  for (int64_t s : strides) HA_REQUIRE(s % 8 == 0, HA_ERR_SHAPE, "%s: gradient rows must be 16-byte aligned", who);
+  HA_REQUIRE(((uintptr_t)g.dout % 16) == 0 && ((uintptr_t)g.dq % 16) == 0 && ((uintptr_t)g.dk % 16) == 0 &&
+                 ((uintptr_t)g.dv % 16) == 0,
+             HA_ERR_SHAPE, "%s: gradient tensors must be 16-byte aligned", who);
+  const int64_t row_strides[] = {g.do_stride_n, g.dq_stride_n, g.dk_stride_n, g.dv_stride_n};
+  const int64_t row_counts[] = {t.n_q, t.n_q, t.n_k, t.n_k};
+  for (int i = 0; i < 4; ++i) {
+    HA_REQUIRE(row_strides[i] > 0 && row_strides[i] * 2 < (1ll << 24), HA_ERR_UNSUPPORTED,
+               "%s: gradient row strides must be positive and below 16 MiB", who);
+    HA_REQUIRE((row_counts[i] - 1) * row_strides[i] * 2 + t.d * 2 <= (1ll << 32), HA_ERR_UNSUPPORTED,
+               "%s: one head of a gradient tensor may span 4 GiB at most", who);
+  }
+  const Workspace w = carve(t, nullptr);
+  HA_REQUIRE(g.workspace && g.workspace_bytes >= w.bytes && ((uintptr_t)g.workspace % 256) == 0, HA_ERR_WORKSPACE,
+             "%s: workspace of %lld bytes (256-byte aligned) required", who, (long long)w.bytes);
+  return HA_OK;
+}
+
+void fill_bwd_params(const ha_attn_operands& t, const ha_attn_grads& g, const Workspace& w, ha_attn_bwd_params& p) {
+  p.q = t.q; p.k = t.k; p.v = t.v; p.dout = g.dout;
+  p.lse = t.lse; p.delta = w.delta;
+  p.dq = g.dq; p.dk32 = w.dk32; p.dv32 = w.dv32;
+  p.q_sb = t.q_stride_b; p.q_sh = t.q_stride_h; p.q_sn = t.q_stride_n;
+  p.k_sb = t.k_stride_b; p.k_sh = t.k_stride_h; p.k_sn = t.k_stride_n;
+  p.v_sb = t.v_stride_b; p.v_sh = t.v_stride_h; p.v_sn = t.v_stride_n;
+  p.do_sb = g.do_stride_b; p.do_sh = g.do_stride_h; p.do_sn = g.do_stride_n;
+  p.dq_sb = g.dq_stride_b; p.dq_sh = g.dq_stride_h; p.dq_sn = g.dq_stride_n;
+  p.lse_sb = t.lse_stride_b; p.lse_sh = t.lse_stride_h;
+  p.q_idx = p.k_idx = p.sampled_idx = nullptr;
+  p.qi_sb = p.qi_sh = p.qi_sn = 0;
+  p.ki_sb = p.ki_sh = p.ki_sn = 0;
+  p.si_sb = p.si_sh = 0;
+  p.batch = (int)t.batch; p.heads = (int)t.heads; p.kv_group = (int)t.kv_group;
+  p.n_q = (int)t.n_q; p.n_k = (int)t.n_k;
+  p.block_tiles = 1; p.sample_size = 0; p.smooth = 0; p.idx64 = 0;
+  p.q_split = (int)t.n_q;
+  p.scale = t.scale;
+  p.scale_log2 = t.scale * LOG2E;
+}
+
+// delta, and zeroed accumulators
+template <typename T, int D>
+int launch_prepare(const ha_attn_operands& t, const ha_attn_grads& g, const Workspace& w, hipStream_t stream) {
+  const int64_t rows = t.batch * t.heads * t.n_q;
+  const int64_t items = rows * (D / 8);
+  hipLaunchKernelGGL((ha_bwd_delta_kernel<T, D>), dim3((unsigned)((items + 255) / 256)), dim3(256), 0, stream,
+                     (const T*)t.out, (const T*)g.dout, w.delta, (int)t.heads, (int)t.n_q, t.o_stride_b, t.o_stride_h,
+                     t.o_stride_n, g.do_stride_b, g.do_stride_h, g.do_stride_n, rows);
+  int st = ha_launch_status("attention backward: delta");
+  if (st != HA_OK) return st;
+  // the two accumulators are adjacent up to alignment padding: clear them with one launch each
+  const int64_t n4 = (w.acc_floats + 3) / 4;
+  hipLaunchKernelGGL(ha_bwd_zero_kernel, dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, stream, (f32x4*)w.dk32, n4);
+  hipLaunchKernelGGL(ha_bwd_zero_kernel, dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, stream, (f32x4*)w.dv32, n4);
+  return ha_launch_status("attention backward: clear");
+}
+
+template <typename T, int D>
+int launch_round(const ha_attn_operands& t, const ha_attn_grads& g, const Workspace& w, hipStream_t stream) {
+  const int64_t kv_heads = t.heads / t.kv_group;
+  const int64_t rows = t.batch * kv_heads * t.n_k;
+  const int64_t items = rows * (D / 8);
+  hipLaunchKernelGGL((ha_bwd_round_kernel<T, D>), dim3((unsigned)((items + 255) / 256)), dim3(256), 0, stream, w.dk32,
+                     w.dv32, (T*)g.dk, (T*)g.dv, (int)kv_heads, (int)t.n_k, g.dk_stride_b, g.dk_stride_h, g.dk_stride_n,
+                     g.dv_stride_b, g.dv_stride_h, g.dv_stride_n, rows);
+  return ha_launch_status("attention backward: round");
+}
+
+template <typename T, int D>
+int run_block_bwd(const ha_block_attn_args& a, const ha_attn_grads& g, hipStream_t stream) {
+  const ha_attn_operands& t = a.t;
+  const Workspace w = carve(t, g.workspace);
+  int st = launch_prepare<T, D>(t, g, w, stream);
+  if (st != HA_OK) return st;
+  ha_attn_bwd_params p;
+  fill_bwd_params(t, g, w, p);
+  p.q_idx = a.q_idx; p.k_idx = a.k_idx; p.sampled_idx = a.sampled_idx;
+  p.qi_sb = a.q_idx_stride_b; p.qi_sh = a.q_idx_stride_h; p.qi_sn = a.q_idx_stride_n;
+  p.ki_sb = a.k_idx_stride_b; p.ki_sh = a.k_idx_stride_h; p.ki_sn = a.k_idx_stride_n;
+  p.si_sb = a.sampled_stride_b; p.si_sh = a.sampled_stride_h;
+  p.block_tiles = (int)((a.block_size + 127) / 128);
+  p.sample_size = (int)a.sample_size;
+  p.smooth = a.smooth_block != 0;
+  p.idx64 = a.idx_type == HA_IDX_I64;
+  const int64_t bh = t.batch * t.heads;
+  st = launch_pass<T, D, HA_BWD_DQ_BLOCK, false>(p, bh * (t.n_q / ST_ROWS), stream, "ha_block_attn_bwd: dq");
+  if (st != HA_OK) return st;
+  st = launch_pass<T, D, HA_BWD_DKV_BLOCK, false>(p, bh * (t.n_k / ST_ROWS), stream, "ha_block_attn_bwd: dk, dv of the blocks");
+  if (st != HA_OK) return st;
+  if (a.sample_size > 0) {
+    // every query attends every sampled key: cut the queries into ranges so that the grid fills the chip
+    int64_t q_split = 2048;
+    while (q_split > 256 && bh * (a.sample_size / ST_ROWS) * ((t.n_q + q_split - 1) / q_split) < 2048) q_split /= 2;
+    p.q_split = (int)q_split;
+    const int64_t splits = (t.n_q + q_split - 1) / q_split;
+    st = launch_pass<T, D, HA_BWD_DKV_SAMPLED, false>(p, bh * (a.sample_size / ST_ROWS) * splits, stream,
+                                                      "ha_block_attn_bwd: dk, dv of the sampled keys");
+    if (st != HA_OK) return st;
+  }
+  return launch_round<T, D>(t, g, w, stream);
+}
+
+template <typename T, int D>
+int run_flash_bwd(const ha_attn_operands& t, bool causal, const ha_attn_grads& g, hipStream_t stream) {
+  const Workspace w = carve(t, g.workspace);
+  int st = launch_prepare<T, D>(t, g, w, stream);
+  if (st != HA_OK) return st;
+  ha_attn_bwd_params p;
+  fill_bwd_params(t, g, w, p);
+  const int64_t bh = t.batch * t.heads;
+  const int64_t q_tiles = (t.n_q + ST_ROWS - 1) / ST_ROWS, k_tiles = (t.n_k + ST_ROWS - 1) / ST_ROWS;
+  if (causal) {
+    st = launch_pass<T, D, HA_BWD_DQ_EXACT, true>(p, bh * q_tiles, stream, "ha_flash_attn_bwd: dq");
+    if (st != HA_OK) return st;
+    st = launch_pass<T, D, HA_BWD_DKV_EXACT, true>(p, bh * k_tiles, stream, "ha_flash_attn_bwd: dk, dv");
+  } else {
+    st = launch_pass<T, D, HA_BWD_DQ_EXACT, false>(p, bh * q_tiles, stream, "ha_flash_attn_bwd: dq");
+    if (st != HA_OK) return st;
+    st = launch_pass<T, D, HA_BWD_DKV_EXACT, false>(p, bh * k_tiles, stream, "ha_flash_attn_bwd: dk, dv");
+  }
+  if (st != HA_OK) return st;
+  return launch_round<T, D>(t, g, w, stream);
+}
+
+}  // namespace
+
+extern "C" int64_t ha_attn_bwd_workspace_bytes(const ha_attn_operands* t) {
+  if (!t || t->batch <= 0 || t->heads <= 0 || t->n_q <= 0 || t->n_k <= 0 || t->d <= 0 || t->kv_group <= 0 ||
+      t->heads % t->kv_group != 0)
+    return ha_fail(HA_ERR_SHAPE, "ha_attn_bwd_workspace_bytes: sizes must be positive, kv_group dividing heads");
+  return carve(*t, nullptr).bytes;
+}
+
+extern "C" int ha_block_attn_bwd(const ha_block_attn_args* args, const ha_attn_grads* grads, void* stream) {
+  HA_REQUIRE(args && grads, HA_ERR_NULL, "ha_block_attn_bwd: null argument");
+  const ha_block_attn_args& a = *args;
+  int st = ha_check_block_attn_args(a, "ha_block_attn_bwd");
+  if (st != HA_OK) return st;
+  st = check_grads(a.t, *grads, "ha_block_attn_bwd");
+  if (st != HA_OK) return st;
+  HA_REQUIRE(!a.accumulate, HA_ERR_UNSUPPORTED, "ha_block_attn_bwd: no backward of the fused merge (accumulate)");
+  HA_REQUIRE(!a.smooth_block || a.block_size <= 128 * (MAX_SMOOTH_TILES - 1), HA_ERR_UNSUPPORTED,
+             "ha_block_attn_bwd: smoothed blocks longer than %d rows are not built", 128 * (MAX_SMOOTH_TILES - 1));
+  hipStream_t s = (hipStream_t)stream;
+  if (a.t.dtype == HA_F16) return a.t.d == 64 ? run_block_bwd<f16_t, 64>(a, *grads, s) : run_block_bwd<f16_t, 128>(a, *grads, s);
+  return a.t.d == 64 ? run_block_bwd<bf16_t, 64>(a, *grads, s) : run_block_bwd<bf16_t, 128>(a, *grads, s);
+}
+
+extern "C" int ha_flash_attn_bwd(const ha_attn_operands* t, int causal, const ha_attn_grads* grads, void* stream) {
+  HA_REQUIRE(t && grads, HA_ERR_NULL, "ha_flash_attn_bwd: null argument");
+  int st = ha_check_operands(*t, "ha_flash_attn_bwd");
+  if (st != HA_OK) return st;
+  st = check_grads(*t, *grads, "ha_flash_attn_bwd");
+  if (st != HA_OK) return st;
+  hipStream_t s = (hipStream_t)stream;
+  if (t->dtype == HA_F16)
+    return t->d == 64 ? run_flash_bwd<f16_t, 64>(*t, causal != 0, *grads, s) : run_flash_bwd<f16_t, 128>(*t, causal != 0, *grads, s);
+  return t->d == 64 ? run_flash_bwd<bf16_t, 64>(*t, causal != 0, *grads, s) : run_flash_bwd<bf16_t, 128>(*t, causal != 0, *grads, s);
+}

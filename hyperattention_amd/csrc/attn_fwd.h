@@ -40,3 +40,8 @@ struct ha_attn_kernel_params {
 };
 
 int ha_attn_launch(const ha_attn_kernel_params& p, int d, int dtype, bool gather, bool causal, hipStream_t stream);
+
+// argument checks shared by the forward and backward entry points (defined in api.hip); `who` names
+// the entry point in the error message
+int ha_check_operands(const ha_attn_operands& t, const char* who);
+int ha_check_block_attn_args(const ha_block_attn_args& a, const char* who);

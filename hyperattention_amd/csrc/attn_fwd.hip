@@ -39,6 +39,7 @@
 // does not depend on m beyond rounding.  m only ever grows, and starts from the true maximum of the
 // first keys or from the log-sum-exp of the partial result that is being resumed.
 #include "ha_common.h"
+#include "attn_tiles.h"
 #include "attn_fwd.h"
 
 namespace {
@@ -46,53 +47,8 @@ namespace {
 constexpr int WG_THREADS = 256;
 constexpr int WG_QUERIES = 256;  // sorted query positions per workgroup
 constexpr int KC = 64;           // keys per LDS tile
-constexpr float LOG2E = 1.4426950408889634f;
-constexpr float LN2 = 0.6931471805599453f;
 constexpr float HALF_SUM_LIMIT = 16384.f;  // 2^14: a lane's half-step sum below this has no fp16 overflow
 constexpr int NUM_XCD = 8;
-
-template <typename T>
-struct Mfma;
-template <>
-struct Mfma<f16_t> {
-  static __device__ __forceinline__ f32x16 run(f16x8 a, f16x8 b, f32x16 c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
-  }
-  // The same MFMA with its accumulator pinned to VGPRs and its B operand to AGPRs.  A kernel that
-  // needs more than 256 registers gets the AGPR form for every MFMA the compiler selects, and a vector
-  // instruction cannot read an AGPR: accumulators that the soft-max reads (S^T) would cost a copy per
-  // value.  Written as assembly the instruction keeps them where the FMAs can use them, while the
-  // query fragments (B) sit in AGPRs for the whole kernel.  first: accumulate onto zero.
-  static __device__ __forceinline__ void run_vgpr_acc(f16x8 a, f16x8 b, f32x16& c, bool first) {
-    if (first)
-      asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "a"(b));
-    else
-      asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "a"(b));
-  }
-  // c[*] + a[0] + a[1] + a[2] + a[3] on the matrix pipe: the 4x4x4 MFMA works on 16 independent
-  // blocks of 4 lanes; with an all-ones A a lane's four results are all the sum of its own four B values
-  static __device__ __forceinline__ f32x4 quad_sum(f16x4 a, f32x4 c) {
-    const f16x4 ones = {(f16_t)1.0f, (f16_t)1.0f, (f16_t)1.0f, (f16_t)1.0f};
-    return __builtin_amdgcn_mfma_f32_4x4x4f16(ones, a, c, 0, 0, 0);
-  }
-};
-template <>
-struct Mfma<bf16_t> {
-  static __device__ __forceinline__ f32x16 run(bf16x8 a, bf16x8 b, f32x16 c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
-  }
-  static __device__ __forceinline__ void run_vgpr_acc(bf16x8 a, bf16x8 b, f32x16& c, bool first) {
-    if (first)
-      asm("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "a"(b));
-    else
-      asm("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "a"(b));
-  }
-  static __device__ __forceinline__ f32x4 quad_sum(bf16x4 a, f32x4 c) {
-    typedef short s16x4 __attribute__((ext_vector_type(4)));
-    const bf16x4 ones = {(bf16_t)1.0f, (bf16_t)1.0f, (bf16_t)1.0f, (bf16_t)1.0f};
-    return __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(__builtin_bit_cast(s16x4, ones), __builtin_bit_cast(s16x4, a), c, 0, 0, 0);
-  }
-};
 
 // Head dims whose kernel needs more than 256 registers keep the S^T accumulators in VGPRs by hand.
 template <int D>
@@ -112,65 +68,12 @@ __device__ __forceinline__ int xcd_contiguous_id(int linear, int total) {
 // x / y for 0 <= x < 2^31 by the divisor's multiply-and-shift constants
 __device__ __forceinline__ int fast_div(int x, ha_divisor y) { return (int)(((uint64_t)(uint32_t)x * y.magic) >> y.shift); }
 
-// Address of 16-byte piece `piece_bytes` of row `row`: a wave-uniform base plus a 32-bit byte offset,
-// so that a lane spends one 24-bit multiply-add on it instead of a 64-bit multiplication.  The entry
-// points check that row numbers and row strides in bytes stay below 2^24 and their products below 2^32.
-__device__ __forceinline__ const unsigned char* row_address(const unsigned char* base, int row, uint32_t stride_bytes,
-                                                            uint32_t piece_bytes) {
-  return base + (uint32_t)(__umul24((uint32_t)row, stride_bytes) + piece_bytes);
-}
-
 // LDS byte offsets of one lane's operand reads, relative to a tile base (fixed for the whole kernel).
 template <int D>
 struct LaneOffsets {
   int k[D / 16];  // Q / K operand piece of k-step ks for tile row lane%32 (add 32 rows for the upper half)
   int v[D / 32];  // V^T operand word for dv block db, keys 0..3 (+4 for the upper lane half) of a 16-key half-step
 };
-
-// 16-byte piece `piece` of row `row` of a row-major [rows][D] 2-byte tile, XOR-swizzled; byte offset.
-// Q and K tiles (read 16 bytes per lane, 8 consecutive rows at a time) move a piece by the row number
-// mod 8.  V tiles are read by the transposing loads, 16 lanes at a time: 4 consecutive rows x 32
-// bytes; they move a PAIR of pieces by the row number mod 4, so that the four rows fall into four
-// different 32-byte bank groups.
-__device__ __forceinline__ int k_swizzle(int row) { return row & 7; }
-__device__ __forceinline__ int v_swizzle(int row) { return (row & 3) << 1; }
-template <int D>
-__device__ __forceinline__ int tile_offset(int row, int piece) {
-  return row * D * 2 + ((piece ^ k_swizzle(row)) << 4);
-}
-template <int D>
-__device__ __forceinline__ int v_tile_offset(int row, int piece) {
-  return row * D * 2 + ((piece ^ v_swizzle(row)) << 4);
-}
-
-template <typename T>
-__device__ __forceinline__ typename ElemTraits<T>::vec8 lds_read_k(const unsigned char* tile, int off) {
-  return *reinterpret_cast<const typename ElemTraits<T>::vec8*>(tile + off);
-}
-
-// 8 keys x 1 dv column of V, transposed by the LDS unit: two 4-key reads
-template <typename T>
-__device__ __forceinline__ typename ElemTraits<T>::vec8 lds_read_vt(const unsigned char* tile, int off, int row_bytes) {
-#if defined(__HIP_DEVICE_COMPILE__)  // the builtin only exists in the device pass
-  typedef short s16x4 __attribute__((ext_vector_type(4)));
-  typedef short s16x8 __attribute__((ext_vector_type(8)));
-  typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
-  const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(tile + off));
-  const s16x4 hi8 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(tile + off + 8 * row_bytes));
-  const s16x8 both = __builtin_shufflevector(lo, hi8, 0, 1, 2, 3, 4, 5, 6, 7);
-  return __builtin_bit_cast(typename ElemTraits<T>::vec8, both);
-#else
-  return typename ElemTraits<T>::vec8{};
-#endif
-}
-
-// 16 bytes per lane from global memory straight into LDS at lds_dst + lane*16 (lds_dst wave-uniform)
-__device__ __forceinline__ void global_to_lds_16(const void* src, unsigned char* lds_dst) {
-#if defined(__HIP_DEVICE_COMPILE__)
-  typedef __attribute__((address_space(3))) unsigned char lds_byte;
-  __builtin_amdgcn_global_load_lds(src, (lds_byte*)lds_dst, 16, 0, 0);
-#endif
-}
 
 // P of the 8 values of half-step H a lane holds per query block (elements 8H..8H+7 of its S^T
 // registers), rounded to T, and their sums.  m is the reference exponent (log2 units).

@@ -71,7 +71,10 @@ class HyperAttention(torch.nn.Module):
             attn, lse = res[0][..., :dim_v], res[1]
             return (attn, lse) if return_lse else attn
 
-        if ops.forward_plan_supported(n_key, self.min_seq_len, causal is not False, self.lsh_num_projs):
+        # gradients are taken operator by operator, as in the reference (each attention operator has its own
+        # backward and the merges are differentiable tensor arithmetic); the one-call forward has none
+        if (ops.forward_plan_supported(n_key, self.min_seq_len, causal is not False, self.lsh_num_projs)
+                and not ops._wants_grad(query, key, value)):
             attn, lse = ops.hyper_forward(
                 query, key, value, self.lsh.proj_dir, scale=scale, causal=causal is not False,
                 lsh_num_projs=self.lsh_num_projs, block_size=self.block_size, sample_size=self.sample_size,

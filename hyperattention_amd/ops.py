@@ -17,7 +17,7 @@ import math
 import torch
 
 from . import _lib
-from ._lib import HA_BF16, HA_F16, HA_IDX_I32, HA_IDX_I64, AttnOperands, BlockAttnArgs, ForwardArgs
+from ._lib import AttnGrads, HA_BF16, HA_F16, HA_IDX_I32, HA_IDX_I64, AttnOperands, BlockAttnArgs, ForwardArgs
 
 
 def _dtype_code(t: torch.Tensor) -> int:
@@ -136,6 +136,32 @@ def padded_head_dim(d):
     return 64 if d <= 64 else 128
 
 
+def _block_attn_args(q, k, v, o, lse, q_sort_idx, k_sort_idx, block_size, sample_size, softmax_scale,
+                     smooth_block, sampled_idx, accumulate=False):
+    """BlockAttnArgs for (b,n,h,d) tensors; the second result keeps the device copy of sampled_idx alive."""
+    batch, seqlen_q, nheads, _ = q.shape
+    a = BlockAttnArgs()
+    a.t = _operands(q, k, v, o, lse, softmax_scale, layout_bnhd=True, lse_row_stride=seqlen_q)
+    a.q_idx, a.k_idx = q_sort_idx.data_ptr(), k_sort_idx.data_ptr()
+    a.idx_type = _idx_code(q_sort_idx)
+    a.q_idx_stride_b, a.q_idx_stride_h, a.q_idx_stride_n = q_sort_idx.stride(0), q_sort_idx.stride(2), q_sort_idx.stride(1)
+    a.k_idx_stride_b, a.k_idx_stride_h, a.k_idx_stride_n = k_sort_idx.stride(0), k_sort_idx.stride(2), k_sort_idx.stride(1)
+    keep = None
+    a.sampled_stride_b = a.sampled_stride_h = 0
+    if sampled_idx is not None:
+        keep = sampled_idx.to(device=q.device, dtype=q_sort_idx.dtype).contiguous()
+        assert keep.shape in ((sample_size,), (nheads, sample_size), (batch, nheads, sample_size)), \
+            "sampled_idx must be (sample_size,), (nheads, sample_size) or (batch, nheads, sample_size)"
+        a.sampled_idx = keep.data_ptr()
+        if keep.dim() >= 2:
+            a.sampled_stride_h = sample_size
+        if keep.dim() == 3:
+            a.sampled_stride_b = nheads * sample_size
+    a.block_size, a.sample_size = block_size, sample_size
+    a.smooth_block, a.accumulate = int(bool(smooth_block)), int(bool(accumulate))
+    return a, keep
+
+
 def hyper_attn_func(q, k, v, q_sort_idx, k_sort_idx, block_size, sample_size=0, softmax_scale=None,
                     smooth_block=False, *, sampled_idx=None, resume=None):
     """q, k: (batch, seqlen, nheads, headdim); v: (batch, seqlen, nheads, v_headdim);
@@ -148,6 +174,10 @@ def hyper_attn_func(q, k, v, q_sort_idx, k_sort_idx, block_size, sample_size=0, 
     which equals add_self_attentions(previous, this call) in fp32."""
     q, k, v = [x if x.stride(-1) == 1 else x.contiguous() for x in [q, k, v]]
     assert sample_size % 128 == 0
+    if _wants_grad(q, k, v) and v.shape[-1] == q.shape[-1] and q.shape[-1] in KERNEL_HEAD_DIMS:
+        assert resume is None, "resume has no backward"
+        return HyperAttnFunc.apply(q, k, v, q_sort_idx, k_sort_idx, block_size, sample_size, softmax_scale,
+                                   smooth_block, sampled_idx)
     if v.shape[-1] != q.shape[-1] or q.shape[-1] not in KERNEL_HEAD_DIMS:
         # A value head dim different from the q/k head dim (src/hyper_attn_triton.py:679,692-693;
         # unit_tests/test_hyper_attention.py:120-133), or a head dim the kernels are not built for.
@@ -183,25 +213,8 @@ def hyper_attn_func(q, k, v, q_sort_idx, k_sort_idx, block_size, sample_size=0, 
         assert o.stride(-1) == 1
     assert seqlen_k % 128 == 0, "keys sequence length must be divisible by 128"
 
-    a = BlockAttnArgs()
-    a.t = _operands(q, k, v, o, lse, softmax_scale, layout_bnhd=True, lse_row_stride=seqlen_q)
-    a.q_idx, a.k_idx = q_sort_idx.data_ptr(), k_sort_idx.data_ptr()
-    a.idx_type = _idx_code(q_sort_idx)
-    a.q_idx_stride_b, a.q_idx_stride_h, a.q_idx_stride_n = q_sort_idx.stride(0), q_sort_idx.stride(2), q_sort_idx.stride(1)
-    a.k_idx_stride_b, a.k_idx_stride_h, a.k_idx_stride_n = k_sort_idx.stride(0), k_sort_idx.stride(2), k_sort_idx.stride(1)
-    keep = None
-    a.sampled_stride_b = a.sampled_stride_h = 0
-    if sampled_idx is not None:
-        keep = sampled_idx.to(device=q.device, dtype=q_sort_idx.dtype).contiguous()
-        assert keep.shape in ((sample_size,), (nheads, sample_size), (batch, nheads, sample_size)), \
-            "sampled_idx must be (sample_size,), (nheads, sample_size) or (batch, nheads, sample_size)"
-        a.sampled_idx = keep.data_ptr()
-        if keep.dim() >= 2:
-            a.sampled_stride_h = sample_size
-        if keep.dim() == 3:
-            a.sampled_stride_b = nheads * sample_size
-    a.block_size, a.sample_size = block_size, sample_size
-    a.smooth_block, a.accumulate = int(bool(smooth_block)), int(resume is not None)
+    a, keep = _block_attn_args(q, k, v, o, lse, q_sort_idx, k_sort_idx, block_size, sample_size, softmax_scale,
+                               smooth_block, sampled_idx, accumulate=resume is not None)
     with torch.cuda.device(q.device):
         _lib.check(_lib.lib().ha_block_attn_fwd(ctypes.byref(a), _stream(q)))
     return o, lse
@@ -218,6 +231,8 @@ def flash_attn_func(q, k, v, bias=None, causal=False, softmax_scale=None):
     assert k.shape == (batch, seqlen_k, nheads, d)
     assert v.shape == (batch, seqlen_k, nheads, d)
     assert d <= 128, "FlashAttention only support head dimensions up to 128"
+    if _wants_grad(q, k, v) and d in KERNEL_HEAD_DIMS:
+        return FlashAttnFunc.apply(q, k, v, bias, causal, softmax_scale)
     if d not in KERNEL_HEAD_DIMS:
         # other head dims run zero-padded to a built width (exact; costs the padded copies)
         pad = lambda x: torch.nn.functional.pad(x, (0, padded_head_dim(d) - d))
@@ -239,6 +254,11 @@ def flash_attn_func(q, k, v, bias=None, causal=False, softmax_scale=None):
 def add_self_attentions(attn1, lse1, attn2, lse2):
     """attn1, attn2: [b, h, n, d]; lse1, lse2: [b, h, n, 1] fp32.  Returns (attn, lse)."""
     assert attn1.is_cuda and attn1.shape == attn2.shape and attn1.dtype == attn2.dtype
+    if _wants_grad(attn1, attn2, lse1, lse2):
+        # differentiable form, in the reference's own arithmetic (src/attn_utils.py:21-23): the weight is
+        # rounded to the attention's type before it is used
+        c = torch.sigmoid(lse1 - lse2).to(attn1.dtype)
+        return c * attn1 + (1 - c) * attn2, lse1 - (c + torch.finfo(lse1.dtype).eps).log()
     b, h, n, d = attn1.shape
     a1 = attn1.contiguous()
     a2 = attn2.contiguous()
@@ -251,6 +271,78 @@ def add_self_attentions(attn1, lse1, attn2, lse2):
         _lib.check(_lib.lib().ha_lse_merge(_ptr(a1), _ptr(l1), _ptr(a2), _ptr(l2), _ptr(out), _ptr(lse),
                                            b * h * n, d, d, d, d, 1, 1, 1, _dtype_code(a1), _stream(a1)))
     return out, lse
+
+
+# ------------------------------------------------------------------------------- backward
+def _wants_grad(*tensors):
+    return torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in tensors)
+
+
+def _attn_grads(t, dout, dq, dk, dv):
+    """AttnGrads for (b,n,h,d) gradient tensors plus the workspace the C side asks for."""
+    g = AttnGrads()
+    g.dout, g.dq, g.dk, g.dv = dout.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr()
+    g.do_stride_b, g.do_stride_h, g.do_stride_n = dout.stride(0), dout.stride(2), dout.stride(1)
+    g.dq_stride_b, g.dq_stride_h, g.dq_stride_n = dq.stride(0), dq.stride(2), dq.stride(1)
+    g.dk_stride_b, g.dk_stride_h, g.dk_stride_n = dk.stride(0), dk.stride(2), dk.stride(1)
+    g.dv_stride_b, g.dv_stride_h, g.dv_stride_n = dv.stride(0), dv.stride(2), dv.stride(1)
+    nbytes = _lib.lib().ha_attn_bwd_workspace_bytes(ctypes.byref(t))
+    if nbytes <= 0:
+        _lib.check(int(nbytes) if nbytes < 0 else -3)
+    ws = torch.empty((nbytes,), device=dout.device, dtype=torch.uint8)
+    g.workspace, g.workspace_bytes = ws.data_ptr(), nbytes
+    return g, ws
+
+
+class HyperAttnFunc(torch.autograd.Function):
+    """hyper_attn_func with its backward (HyperAttnFunc, src/hyper_attn_triton.py:895-945): gradients for
+    q, k, v; a gradient arriving for lse is ignored, as there."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, q_sort_idx, k_sort_idx, block_size, sample_size, softmax_scale, smooth_block,
+                sampled_idx):
+        o, lse = hyper_attn_func(q, k, v, q_sort_idx, k_sort_idx, block_size, sample_size, softmax_scale,
+                                 smooth_block, sampled_idx=sampled_idx)
+        ctx.save_for_backward(q, k, v, q_sort_idx, k_sort_idx, o, lse)
+        ctx.sampled_idx = sampled_idx
+        ctx.conf = (block_size, sample_size, softmax_scale or 1.0 / math.sqrt(q.shape[-1]), smooth_block)
+        return o, lse
+
+    @staticmethod
+    def backward(ctx, do, dlse=None):
+        q, k, v, q_sort_idx, k_sort_idx, o, lse = ctx.saved_tensors
+        block_size, sample_size, softmax_scale, smooth_block = ctx.conf
+        do = do.contiguous()
+        dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+        a, keep = _block_attn_args(q, k, v, o, lse, q_sort_idx, k_sort_idx, block_size, sample_size, softmax_scale,
+                                   smooth_block, ctx.sampled_idx)
+        g, ws = _attn_grads(a.t, do, dq, dk, dv)
+        with torch.cuda.device(q.device):
+            _lib.check(_lib.lib().ha_block_attn_bwd(ctypes.byref(a), ctypes.byref(g), _stream(q)))
+        return dq, dk, dv, None, None, None, None, None, None, None
+
+
+class FlashAttnFunc(torch.autograd.Function):
+    """flash_attn_func with its backward (FlashAttnFunc, src/flash_attn_triton.py:995-1040)."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, bias, causal, softmax_scale):
+        o, lse = flash_attn_func(q, k, v, bias, causal, softmax_scale)
+        ctx.save_for_backward(q, k, v, o, lse)
+        ctx.conf = (bool(causal), softmax_scale or 1.0 / math.sqrt(q.shape[-1]))
+        return o, lse
+
+    @staticmethod
+    def backward(ctx, do, dlse=None):
+        q, k, v, o, lse = ctx.saved_tensors
+        causal, softmax_scale = ctx.conf
+        do = do.contiguous()
+        dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+        t = _operands(q, k, v, o, lse, softmax_scale, layout_bnhd=True, lse_row_stride=lse.shape[-1])
+        g, ws = _attn_grads(t, do, dq, dk, dv)
+        with torch.cuda.device(q.device):
+            _lib.check(_lib.lib().ha_flash_attn_bwd(ctypes.byref(t), int(causal), ctypes.byref(g), _stream(q)))
+        return dq, dk, dv, None, None, None
 
 
 # ------------------------------------------------------------------------- whole forward pass

@@ -1,5 +1,6 @@
 /*
- * hyperattn.h — C ABI of libhyperattn.so, the MI355X (gfx950) HyperAttention forward path.
+ * hyperattn.h — C ABI of libhyperattn.so, the MI355X (gfx950) HyperAttention forward path
+ * (and the backward of its two attention operators).
  *
  * Every entry point takes raw DEVICE pointers, sizes and strides (in ELEMENTS of the tensor's
  * type unless stated otherwise) and a HIP stream passed as void* (hipStream_t; NULL = the
@@ -21,7 +22,7 @@
 extern "C" {
 #endif
 
-#define HA_ABI_VERSION 2
+#define HA_ABI_VERSION 3
 
 typedef enum {
   HA_OK = 0,
@@ -145,6 +146,45 @@ int ha_block_attn_fwd(const ha_block_attn_args* args, void* stream);
  * Any n_q, n_k >= 1; causal mask row >= col (:177); d == dv in {64, 128}.
  */
 int ha_flash_attn_fwd(const ha_attn_operands* t, int causal, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Backward of the two attention operators: gradients with respect to q, k and v given dout, the
+ * gradient of the operator's `out`.  The operands struct is the forward's, with `out` and `lse`
+ * holding the forward's results (read only here); a gradient for `lse` is not taken, as in the
+ * reference (HyperAttnFunc.backward / FlashAttnFunc.backward ignore it).
+ * dq: like q; dk, dv: like k, v, i.e. (batch, heads / kv_group, n_k, d): with grouped queries every
+ * query head of a group adds into its key head.  All in dtype, last dim contiguous, written in full.
+ * Only whole heads: segs == 1 and zero segment offsets.
+ * workspace: ha_attn_bwd_workspace_bytes(t) bytes, 256-byte aligned (row statistics and fp32
+ * accumulators of dk, dv; cleared by the call).
+ */
+typedef struct {
+  const void* dout;  /* (.., n_q, dv)                          */
+  void* dq;
+  void* dk;
+  void* dv;
+  int64_t do_stride_b, do_stride_h, do_stride_n;
+  int64_t dq_stride_b, dq_stride_h, dq_stride_n;
+  int64_t dk_stride_b, dk_stride_h, dk_stride_n;
+  int64_t dv_stride_b, dv_stride_h, dv_stride_n;
+  void* workspace;
+  int64_t workspace_bytes;
+} ha_attn_grads;
+
+int64_t ha_attn_bwd_workspace_bytes(const ha_attn_operands* t);
+
+/* replaces: HyperAttnFunc.backward -> _hyper_attn_backward with _bwd_preprocess_do_o_dot,
+ *           _bwd_permuted_block_diagonal_kernel, _bwd_sampled_col_kernel
+ *           (src/hyper_attn_triton.py:922-945, :745-893, :195-665)
+ * Same arguments as ha_block_attn_fwd (accumulate must be 0).  A key that is in a query's block and in
+ * the sample list receives both contributions, as it is counted twice in the forward.
+ */
+int ha_block_attn_bwd(const ha_block_attn_args* args, const ha_attn_grads* grads, void* stream);
+
+/* replaces: FlashAttnFunc.backward -> _flash_attn_backward (src/flash_attn_triton.py:1014-1040,
+ *           :875-992) with bias=None.
+ */
+int ha_flash_attn_bwd(const ha_attn_operands* t, int causal, const ha_attn_grads* grads, void* stream);
 
 /* Merge of two partial attentions.
  * replaces: add_self_attentions (src/attn_utils.py:6-24)

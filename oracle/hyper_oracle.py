@@ -23,6 +23,9 @@ block_sampled_attention     reduces to exact_attention for block_size = n, sampl
 add_self_attentions         merging attention over two disjoint key sets == attention over union
 hyper_forward               min_seq_len >= n -> exact causal; one-level split with block = n/2
                             -> exact causal; brute-force row-by-row definition on tiny sizes
+gradients (torch autograd   central finite differences of the same functions in float64; the
+of the functions above)     closed formulas dV = P^T dO, dS = P (dP - D) scale, dQ = dS K,
+                            dK = dS^T Q written out per (query, key) pair on tiny sizes
 ==========================  =====================================================================
 
 Parity unpinned (no reference test or fixture fixes it, tolerance comes from the stated
@@ -267,7 +270,8 @@ def add_self_attentions(attn1, lse1, attn2, lse2):
 
 
 def forward_no_causal_mask(q, k, v, scale, proj, lsh_num_projs, block_size, sample_size,
-                           min_seq_len, smooth_block, sampled_idx=None, dtype=torch.float64):
+                           min_seq_len, smooth_block, sampled_idx=None, dtype=torch.float64,
+                           detach_lse=False):
     """Follows hyper_attention.py:103-132.  Returns attn (b,h,n,dv), lse (b,h,n,1)."""
     n_query = q.shape[2]
     if min_seq_len > n_query:  # :109
@@ -277,12 +281,14 @@ def forward_no_causal_mask(q, k, v, scale, proj, lsh_num_projs, block_size, samp
         k_idx = stable_bucket_argsort(lsh_hash(k, proj))  # :117
         attn, lse = block_sampled_attention(q, k, v, q_idx, k_idx, block_size, sample_size,
                                             scale, smooth_block, sampled_idx, dtype)
+    if detach_lse:
+        lse = lse.detach()
     return attn, lse.unsqueeze(-1)
 
 
 def hyper_forward(q, k, v, proj, scale=None, causal=False, lsh_num_projs=8, block_size=256,
                   sample_size=256, min_seq_len=2048, smooth_block=False, sampled_idx=None,
-                  dtype=torch.float64):
+                  dtype=torch.float64, detach_lse=False):
     """HyperAttention.forward with return_lse=True, (b,h,n,d) layout.
 
     Follows hyper_attention.py:25-101: non-causal dispatch (:48-49), causal leaf (:52-57),
@@ -291,6 +297,11 @@ def hyper_forward(q, k, v, proj, scale=None, causal=False, lsh_num_projs=8, bloc
     (:86-89), concatenation and un-padding (:91-96).  ``proj`` is the (d, r) projection
     matrix (already rounded to the input precision); ``sampled_idx`` indexes rows *within the
     key tensor handed to each un-masked call*.  lse is always returned as (b,h,n,1).
+
+    Gradients (torch autograd differentiates this function as it stands).  ``detach_lse=True``
+    gives the gradient the reference's autograd computes: its attention operators return no
+    gradient for their log-sum-exp output (src/hyper_attn_triton.py:922-945,
+    src/flash_attn_triton.py:1014-1040), so every log-sum-exp entering a merge is a constant there.
     """
     q = torch.as_tensor(q).to(dtype)
     k = torch.as_tensor(k).to(dtype)
@@ -301,11 +312,13 @@ def hyper_forward(q, k, v, proj, scale=None, causal=False, lsh_num_projs=8, bloc
     assert n_query == n_key  # :45
     kw = dict(proj=proj, lsh_num_projs=lsh_num_projs, block_size=block_size,
               sample_size=sample_size, min_seq_len=min_seq_len, smooth_block=smooth_block,
-              sampled_idx=sampled_idx, dtype=dtype)
+              sampled_idx=sampled_idx, dtype=dtype, detach_lse=detach_lse)
     if causal is False:
         return forward_no_causal_mask(q, k, v, scale, **kw)
     if n_key <= min_seq_len:  # :52
         attn, lse = exact_attention(q, k, v, scale, True, dtype)
+        if detach_lse:
+            lse = lse.detach()
         return attn, lse.unsqueeze(-1)
     if n_query % 2:  # :61-64
         q = torch.nn.functional.pad(q, (0, 0, 0, 1))

@@ -32,7 +32,7 @@ def test_every_declared_symbol_is_exported(lib):
     assert declared == sorted(_lib.SYMBOLS)
     for name in declared:
         assert hasattr(lib, name), f"{name} declared in hyperattn.h but not exported"
-    assert lib.ha_abi_version() == 2
+    assert lib.ha_abi_version() == 3
 
 
 def test_struct_layouts_match_the_header(tmp_path):

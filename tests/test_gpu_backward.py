@@ -1,0 +1,192 @@
+"""GPU parity tests of the attention backward (through the C ABI, driven by torch autograd) against
+gradients of the CPU oracle.
+
+The oracle's forward functions are plain torch arithmetic in float64, so torch autograd differentiates
+them as they stand; tests/test_oracle.py checks those gradients against finite differences and against
+the closed formulas.  A gradient arriving for the log-sum-exp output is ignored by the operators, as
+in the reference (src/hyper_attn_triton.py:922-945, src/flash_attn_triton.py:1014-1040): the loss used
+here depends on the attention output only.
+
+Tolerances: norm-wise ||g - ref|| <= tol ||ref|| per gradient tensor, tol = 3e-3 for fp16 and 1e-2 for
+bf16.  They are wider than the forward's because P and dS are rounded to the input type before the
+products, as the reference does (src/hyper_attn_triton.py:345,367), and dS has twice the relative
+error of P.
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import hyper_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+from _util import _gen, _randn
+
+TOL = {torch.float16: 3e-3, torch.bfloat16: 1e-2}
+
+
+@pytest.fixture(scope="module")
+def ha():
+    import hyperattention_amd
+    from hyperattention_amd import _lib
+    _lib.lib()  # fails loudly when the HIP library is missing
+    return hyperattention_amd
+
+
+def _check(got, ref, what, dtype):
+    got = got.detach().double().cpu()
+    ref = ref.detach().double().cpu()
+    assert got.shape == ref.shape, f"{what}: shape {tuple(got.shape)} vs {tuple(ref.shape)}"
+    assert torch.isfinite(got).all(), f"{what}: non-finite values"
+    # a gradient that is exactly zero (a single key: the soft-max is constant) is compared absolutely
+    rel = ((got - ref).norm() / ref.norm().clamp(min=1e-3)).item()
+    assert rel <= TOL[dtype], f"{what}: norm-wise relative error {rel:.3e} > {TOL[dtype]}"
+    # no element far off: a wrong row or a dropped tile shows here even when the norm hides it
+    worst = ((got - ref).abs().max() / ref.abs().max().clamp(min=1e-3)).item()
+    assert worst <= 10 * TOL[dtype], f"{what}: worst element error {worst:.3e} of the largest gradient"
+
+
+def _oracle_grads(fn, q, k, v, do):
+    q64, k64, v64 = (x.double().requires_grad_() for x in (q, k, v))
+    out, _ = fn(q64, k64, v64)
+    out.backward(do.double())
+    return q64.grad, k64.grad, v64.grad
+
+
+def _gpu_grads(fn, q, k, v, do):
+    """fn takes (b,n,h,d) CUDA tensors and returns (o (b,n,h,d), lse); inputs here are (b,h,n,d) CPU."""
+    qg, kg, vg = (x.cuda().transpose(1, 2).contiguous().requires_grad_() for x in (q, k, v))
+    o, lse = fn(qg, kg, vg)
+    o.backward(do.cuda().transpose(1, 2).contiguous())
+    torch.cuda.synchronize()
+    return o, lse, qg.grad.transpose(1, 2), kg.grad.transpose(1, 2), vg.grad.transpose(1, 2)
+
+
+# ------------------------------------------------------------------------------- exact attention
+@pytest.mark.parametrize("dtype,b,h,nq,nk,d,causal", [
+    (torch.float16, 1, 2, 256, 256, 64, False),
+    (torch.float16, 1, 2, 256, 256, 64, True),
+    (torch.float16, 2, 3, 300, 300, 64, True),       # ragged: last tiles are partial
+    (torch.bfloat16, 1, 2, 333, 333, 128, True),
+    (torch.bfloat16, 1, 2, 200, 517, 128, False),    # more keys than queries
+    (torch.float16, 1, 1, 640, 130, 64, False),      # more queries than keys
+    (torch.float16, 1, 2, 1, 1, 64, True),           # a single row
+])
+def test_flash_backward(ha, dtype, b, h, nq, nk, d, causal):
+    q = _randn((b, h, nq, d), 11, dtype)
+    k = _randn((b, h, nk, d), 12, dtype)
+    v = _randn((b, h, nk, d), 13, dtype)
+    do = _randn((b, h, nq, d), 14, dtype)
+    ref = _oracle_grads(lambda a, b_, c: O.exact_attention(a, b_, c, None, causal), q, k, v, do)
+    o, lse, dq, dk, dv = _gpu_grads(lambda a, b_, c: ha.flash_attn_func(a, b_, c, None, causal), q, k, v, do)
+    with torch.no_grad():
+        o_plain, _ = ha.flash_attn_func(q.cuda().transpose(1, 2), k.cuda().transpose(1, 2), v.cuda().transpose(1, 2),
+                                        None, causal)
+    assert torch.equal(o.detach(), o_plain), "the forward under autograd differs from the plain forward"
+    for got, want, name in zip((dq, dk, dv), ref, ("dq", "dk", "dv")):
+        _check(got, want, f"flash {name}", dtype)
+
+
+# ------------------------------------------------------------------- sorted blocks + sampled keys
+def _perms(b, h, n, seed):
+    g = _gen(seed)
+    return torch.stack([torch.stack([torch.randperm(n, generator=g) for _ in range(h)]) for _ in range(b)])
+
+
+@pytest.mark.parametrize("dtype,b,h,n,d,block,sample,smooth", [
+    (torch.float16, 1, 2, 1024, 64, 256, 256, False),
+    (torch.float16, 1, 2, 1024, 64, 256, 256, True),
+    (torch.float16, 2, 2, 768, 64, 256, 0, False),      # no samples; the last block is shorter
+    (torch.float16, 1, 1, 768, 64, 512, 128, True),     # smoothed, block does not divide the length
+    (torch.bfloat16, 1, 2, 2048, 128, 512, 512, True),
+    (torch.bfloat16, 1, 3, 1024, 128, 256, 128, False),
+    (torch.float16, 1, 2, 512, 64, 512, 128, False),    # one block = exact attention plus the samples
+    (torch.float16, 1, 1, 384, 64, 128, 128, False),
+])
+def test_block_backward(ha, dtype, b, h, n, d, block, sample, smooth):
+    q = _randn((b, h, n, d), 21, dtype)
+    k = _randn((b, h, n, d), 22, dtype)
+    v = _randn((b, h, n, d), 23, dtype)
+    do = _randn((b, h, n, d), 24, dtype)
+    qi, ki = _perms(b, h, n, 25), _perms(b, h, n, 26)
+    ref = _oracle_grads(lambda a, b_, c: O.block_sampled_attention(a, b_, c, qi, ki, block, sample, None, smooth),
+                        q, k, v, do)
+    qi_g, ki_g = qi.cuda().transpose(1, 2), ki.cuda().transpose(1, 2)
+    o, lse, dq, dk, dv = _gpu_grads(lambda a, b_, c: ha.hyper_attn_func(a, b_, c, qi_g, ki_g, block, sample, None, smooth),
+                                    q, k, v, do)
+    for got, want, name in zip((dq, dk, dv), ref, ("dq", "dk", "dv")):
+        _check(got, want, f"block {name}", dtype)
+
+
+@pytest.mark.parametrize("per_head", [False, True])
+def test_block_backward_explicit_samples_with_repeats(ha, per_head):
+    # sampled rows given explicitly, some of them twice: each occurrence is one more column of the
+    # soft-max, and the key's gradient adds them up
+    dtype, b, h, n, d, block, sample = torch.float16, 1, 2, 1024, 64, 256, 128
+    q = _randn((b, h, n, d), 31, dtype)
+    k = _randn((b, h, n, d), 32, dtype)
+    v = _randn((b, h, n, d), 33, dtype)
+    do = _randn((b, h, n, d), 34, dtype)
+    qi, ki = _perms(b, h, n, 35), _perms(b, h, n, 36)
+    g = _gen(37)
+    if per_head:
+        si = torch.randint(0, n, (b, h, sample), generator=g)
+        si[:, :, 5] = si[:, :, 4]
+        si_gpu = si[0]
+    else:
+        si = torch.randint(0, n, (sample,), generator=g)
+        si[5] = si[4]
+        si[100] = si[4]
+        si_gpu = si
+    ref = _oracle_grads(lambda a, b_, c: O.block_sampled_attention(a, b_, c, qi, ki, block, sample, None, False,
+                                                                   sampled_idx=si), q, k, v, do)
+    qi_g, ki_g = qi.cuda().transpose(1, 2), ki.cuda().transpose(1, 2)
+    o, lse, dq, dk, dv = _gpu_grads(
+        lambda a, b_, c: ha.hyper_attn_func(a, b_, c, qi_g, ki_g, block, sample, None, False, sampled_idx=si_gpu),
+        q, k, v, do)
+    for got, want, name in zip((dq, dk, dv), ref, ("dq", "dk", "dv")):
+        _check(got, want, f"block {name}", dtype)
+
+
+def test_block_backward_int32_indices_and_sorted_buckets(ha):
+    # permutations as the module makes them: stable argsort of LSH buckets, int32
+    dtype, b, h, n, d = torch.float16, 1, 2, 2048, 64
+    q = _randn((b, h, n, d), 41, dtype)
+    k = _randn((b, h, n, d), 42, dtype)
+    v = _randn((b, h, n, d), 43, dtype)
+    do = _randn((b, h, n, d), 44, dtype)
+    proj = _randn((d, 8), 45, dtype)
+    qi = torch.from_numpy(O.stable_bucket_argsort(O.lsh_hash(q, proj)))
+    ki = torch.from_numpy(O.stable_bucket_argsort(O.lsh_hash(k, proj)))
+    ref = _oracle_grads(lambda a, b_, c: O.block_sampled_attention(a, b_, c, qi, ki, 256, 256), q, k, v, do)
+    qi_g, ki_g = qi.int().cuda().transpose(1, 2), ki.int().cuda().transpose(1, 2)
+    o, lse, dq, dk, dv = _gpu_grads(lambda a, b_, c: ha.hyper_attn_func(a, b_, c, qi_g, ki_g, 256, 256), q, k, v, do)
+    for got, want, name in zip((dq, dk, dv), ref, ("dq", "dk", "dv")):
+        _check(got, want, f"block {name}", dtype)
+
+
+# ------------------------------------------------------------------------------- the module
+@pytest.mark.parametrize("causal,n,min_seq_len", [(False, 1024, 256), (True, 1024, 256), (True, 1025, 600)])
+def test_module_backward(ha, causal, n, min_seq_len):
+    # the module under autograd: operators with their own backward, merges as tensor arithmetic;
+    # log-sum-exps carry no gradient (detach_lse), as the reference's operators return none for them
+    dtype, b, h, d = torch.float16, 1, 2, 64
+    q = _randn((b, h, n, d), 51, dtype)
+    k = _randn((b, h, n, d), 52, dtype)
+    v = _randn((b, h, n, d), 53, dtype)
+    do = _randn((b, h, n, d), 54, dtype)
+    m = ha.HyperAttention(input_dim=d, block_size=128, sample_size=128, min_seq_len=min_seq_len, rng=_gen(55))
+    m = m.to(device="cuda", dtype=dtype)
+    proj = m.lsh.proj_dir[0, 0].cpu()
+    ref = _oracle_grads(lambda a, b_, c: O.hyper_forward(a, b_, c, proj, causal=causal, block_size=128, sample_size=128,
+                                                         min_seq_len=min_seq_len, detach_lse=True), q, k, v, do)
+    qg, kg, vg = (x.cuda().requires_grad_() for x in (q, k, v))
+    out = m(qg, kg, vg, causal=causal)
+    with torch.no_grad():
+        out_plain = m(q.cuda(), k.cuda(), v.cuda(), causal=causal)
+    rel = ((out.detach().double() - out_plain.double()).norm() / out_plain.double().norm()).item()
+    assert rel < 2e-3, f"forward under autograd vs one-call forward: {rel:.3e}"
+    out.backward(do.cuda())
+    torch.cuda.synchronize()
+    for got, want, name in zip((qg.grad, kg.grad, vg.grad), ref, ("dq", "dk", "dv")):
+        _check(got, want, f"module {name}", dtype)

@@ -316,3 +316,102 @@ def test_forward_causal_bruteforce_definition():
         want = (torch.softmax(s, 0)[:, None] * V[cols]).sum(0)
         assert torch.allclose(attn[0, 0, i], want, atol=1e-9)
         assert abs(lse[0, 0, i, 0] - want_lse) < 1e-5
+
+
+# ------------------------------------------------------------------------------- gradients
+# The GPU backward is compared with torch autograd applied to the oracle's forward functions.  These
+# tests pin those gradients independently: by central finite differences of the same functions in
+# float64, and by the closed formulas written out pair by pair.
+def _directional(fn, xs, us, eps=1e-6):
+    plus = fn(*[x + eps * u for x, u in zip(xs, us)])
+    minus = fn(*[x - eps * u for x, u in zip(xs, us)])
+    return ((plus - minus) / (2 * eps)).item()
+
+
+def _autograd_directional(fn, xs, us):
+    leaves = [x.clone().requires_grad_() for x in xs]
+    fn(*leaves).backward()
+    return sum((l.grad * u).sum() for l, u in zip(leaves, us)).item()
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_gradient_exact_attention_closed_form_and_finite_differences(causal):
+    g = torch.Generator().manual_seed(70)
+    nq, nk, d = 6, 6, 4
+    q, k, v, do = (torch.randn((1, 1, n, d), generator=g, dtype=torch.float64) for n in (nq, nk, nk, nq))
+    scale = 0.37
+    loss = lambda a, b, c: (O.exact_attention(a, b, c, scale, causal)[0] * do).sum()
+    leaves = [x.clone().requires_grad_() for x in (q, k, v)]
+    loss(*leaves).backward()
+    # closed formulas, one (query, key) pair at a time
+    out, lse = O.exact_attention(q, k, v, scale, causal)
+    dq, dk, dv = torch.zeros_like(q), torch.zeros_like(k), torch.zeros_like(v)
+    for i in range(nq):
+        delta = (do[0, 0, i] * out[0, 0, i]).sum()
+        for j in range(nk):
+            if causal and j > i:
+                continue
+            p = math.exp(scale * (q[0, 0, i] @ k[0, 0, j]).item() - lse[0, 0, i].item())
+            ds = p * ((do[0, 0, i] @ v[0, 0, j]).item() - delta.item()) * scale
+            dv[0, 0, j] += p * do[0, 0, i]
+            dq[0, 0, i] += ds * k[0, 0, j]
+            dk[0, 0, j] += ds * q[0, 0, i]
+    for got, want in zip(leaves, (dq, dk, dv)):
+        assert torch.allclose(got.grad, want, rtol=1e-10, atol=1e-12)
+    for _ in range(3):
+        us = [torch.randn(x.shape, generator=g, dtype=torch.float64) for x in (q, k, v)]
+        fd = _directional(loss, (q, k, v), us)
+        ad = sum((l.grad * u).sum() for l, u in zip(leaves, us)).item()
+        assert abs(fd - ad) <= 1e-7 * max(1.0, abs(ad))
+
+
+@pytest.mark.parametrize("smooth", [False, True])
+def test_gradient_block_sampled_finite_differences(smooth):
+    g = torch.Generator().manual_seed(71)
+    n, d = 256, 4
+    q, k, v, do = (torch.randn((1, 2, n, d), generator=g, dtype=torch.float64) for _ in range(4))
+    qi = torch.stack([torch.randperm(n, generator=g) for _ in range(2)])[None]
+    ki = torch.stack([torch.randperm(n, generator=g) for _ in range(2)])[None]
+    si = torch.randint(0, n, (128,), generator=g)
+    si[3] = si[2]  # a key sampled twice is two columns
+    loss = lambda a, b, c: (O.block_sampled_attention(a, b, c, qi, ki, 128, 128, 0.41, smooth, sampled_idx=si)[0] * do).sum()
+    for _ in range(3):
+        us = [torch.randn(x.shape, generator=g, dtype=torch.float64) for x in (q, k, v)]
+        fd = _directional(loss, (q, k, v), us)
+        ad = _autograd_directional(loss, (q, k, v), us)
+        assert abs(fd - ad) <= 1e-6 * max(1.0, abs(ad))
+
+
+def test_gradient_hyper_forward_true_and_with_constant_log_sum_exps():
+    # one recursion level (n = 2 * min_seq_len): first half exact causal, second half the merge of its
+    # own exact causal part with the un-masked call on (second-half queries, first-half keys)
+    g = torch.Generator().manual_seed(72)
+    n, d, half = 256, 8, 128
+    q, k, v, do = (torch.randn((1, 1, n, d), generator=g, dtype=torch.float64) for _ in range(4))
+    proj = torch.randn((d, 8), generator=g, dtype=torch.float64)
+    kw = dict(causal=True, block_size=128, sample_size=128, min_seq_len=128)
+    us = [torch.randn(x.shape, generator=g, dtype=torch.float64) for x in (q, k, v)]
+    # perturbations small enough that no bucket changes: the loss is smooth around the point
+    true_loss = lambda a, b, c: (O.hyper_forward(a, b, c, proj, **kw)[0] * do).sum()
+    fd = _directional(true_loss, (q, k, v), us, eps=1e-7)
+    ad = _autograd_directional(true_loss, (q, k, v), us)
+    assert abs(fd - ad) <= 1e-5 * max(1.0, abs(ad))
+
+    # detach_lse: the merge weight is a constant taken at the point itself
+    _, lse_a = O.exact_attention(q[:, :, half:], k[:, :, half:], v[:, :, half:], None, True)
+    _, lse_b = O.forward_no_causal_mask(q[:, :, half:], k[:, :, :half], v[:, :, :half], d ** -0.5, proj, 8, 128, 128,
+                                        128, False)
+    c = torch.sigmoid(lse_a.unsqueeze(-1) - lse_b)
+
+    def frozen_loss(a, b, cc):
+        top, _ = O.exact_attention(a[:, :, :half], b[:, :, :half], cc[:, :, :half], None, True)
+        own, _ = O.exact_attention(a[:, :, half:], b[:, :, half:], cc[:, :, half:], None, True)
+        off, _ = O.forward_no_causal_mask(a[:, :, half:], b[:, :, :half], cc[:, :, :half], d ** -0.5, proj, 8, 128,
+                                          128, 128, False)
+        return (torch.cat((top, c * own + (1 - c) * off), dim=2) * do).sum()
+
+    fd = _directional(frozen_loss, (q, k, v), us, eps=1e-7)
+    detached = lambda a, b, cc: (O.hyper_forward(a, b, cc, proj, detach_lse=True, **kw)[0] * do).sum()
+    ad = _autograd_directional(detached, (q, k, v), us)
+    assert abs(fd - ad) <= 1e-5 * max(1.0, abs(ad))
+    assert abs(ad - _autograd_directional(true_loss, (q, k, v), us)) > 1e-6  # the two gradients do differ
