@@ -1,14 +1,16 @@
-"""Sequence-length sweep of one attention layer, forward only, on the MI355X.
+"""Sequence-length sweep of one attention layer on the MI355X: forward, backward, or both.
 
 Same command line, shapes and output lines as the reference's sweep (benchmark_single_attention.py:14-22,
 92-111: batch 1, 24 heads, head dim 64, bf16, seq 2^10 .. 2^17, block 256, sample 256):
 
     python -m hyperattention_amd.benchmark_single_attention --mode fwd --attn_method hyper [--no_causal] [--smooth_block]
-    python -m hyperattention_amd.benchmark_single_attention --mode fwd --attn_method flash [--no_causal]
+    python -m hyperattention_amd.benchmark_single_attention --mode fwd+bwd --attn_method flash [--no_causal]
 
-`flash` is this library's exact MFMA attention.  Only the forward pass exists here, so `--mode` must be
-`fwd`; `bwd` and `fwd+bwd` (the reference's default) stop with a message.  Times are the 20 % / 50 % /
-80 % quantiles in ms over `rep` calls, each bracketed by events on the launch stream.
+`flash` is this library's exact MFMA attention.  `--mode fwd` times the forward without autograd (for
+`hyper` that is the one-call forward); `bwd` times `o.backward(do, retain_graph=True)` and `fwd+bwd` adds
+to it the forward as autograd runs it (operator by operator), quantile by quantile, as the reference's
+script does (benchmark_single_attention.py:42-52, 70-80).  Times are the 20 % / 50 % / 80 % quantiles in
+ms over `rep` calls, each bracketed by events on the launch stream.
 """
 import argparse
 import sys
@@ -24,6 +26,8 @@ def get_arguments(argv=None):
     parser.add_argument("--smooth_block", action="store_true")
     parser.add_argument("--mode", type=str, default="fwd", choices=["fwd", "bwd", "fwd+bwd"])
     parser.add_argument("--attn_method", type=str, default="flash", choices=["flash", "flash-cuda", "hyper"])
+    parser.add_argument("--max_log2_seq", type=int, default=17, help="last sequence length of the sweep (2^k)")
+    parser.add_argument("--rep", type=int, default=100)
     return parser.parse_args(argv)
 
 
@@ -42,36 +46,47 @@ def time_quantiles(fn, warmup=20, rep=100, quantiles=(0.2, 0.5, 0.8)):
     return [float(x) for x in torch.quantile(times, torch.tensor(quantiles, dtype=torch.float64))]
 
 
-def run_flash_attn(batch_size, head_size, seq_len, dim, causal, warmup=20, rep=100):
-    q, k, v = (torch.randn((batch_size, seq_len, head_size, dim), dtype=torch.bfloat16, device="cuda") for _ in range(3))
-    return time_quantiles(lambda: flash_attn_func(q, k, v, None, causal, None)[0], warmup, rep)
+def time_mode(fn, mode, warmup, rep):
+    """fn: the forward, returning the attention output.  Quantiles of the forward, the backward, or their sum."""
+    if mode == "fwd":
+        return time_quantiles(fn, warmup, rep)
+    fwd = time_quantiles(fn, warmup, rep) if mode == "fwd+bwd" else [0.0, 0.0, 0.0]
+    o = fn()
+    do = torch.randn_like(o)
+    bwd = time_quantiles(lambda: o.backward(do, retain_graph=True), warmup, rep)
+    return [a + b for a, b in zip(fwd, bwd)]
 
 
-def run_hyper_attn(batch_size, head_size, seq_len, dim, causal, smooth_block, warmup=20, rep=100):
-    q, k, v = (torch.randn((batch_size, head_size, seq_len, dim), dtype=torch.bfloat16, device="cuda") for _ in range(3))
+def run_flash_attn(batch_size, head_size, seq_len, dim, causal, mode="fwd", warmup=20, rep=100):
+    q, k, v = (torch.randn((batch_size, seq_len, head_size, dim), dtype=torch.bfloat16, device="cuda",
+                           requires_grad=mode != "fwd") for _ in range(3))
+    return time_mode(lambda: flash_attn_func(q, k, v, None, causal, None)[0], mode, warmup, rep)
+
+
+def run_hyper_attn(batch_size, head_size, seq_len, dim, causal, smooth_block, mode="fwd", warmup=20, rep=100):
+    q, k, v = (torch.randn((batch_size, head_size, seq_len, dim), dtype=torch.bfloat16, device="cuda",
+                           requires_grad=mode != "fwd") for _ in range(3))
     attn = HyperAttention(input_dim=dim, block_size=256, sample_size=256, smooth_block=smooth_block).to(
         device="cuda", dtype=q.dtype)
-    return time_quantiles(lambda: attn(q, k, v, causal=causal), warmup, rep)
+    return time_mode(lambda: attn(q, k, v, causal=causal), mode, warmup, rep)
 
 
 def main(argv=None):
     args = get_arguments(argv)
     for arg_name, arg_var in args.__dict__.items():
         print(f"{arg_name:<16} : {arg_var}")
-    if args.mode != "fwd":
-        sys.exit("only the forward pass is built here: run with --mode fwd")
     if args.attn_method == "flash-cuda":
         sys.exit("flash-cuda is a CUDA package; use --attn_method flash for this library's exact attention")
 
-    seq_lens = [2 ** i for i in range(10, 18)]
+    seq_lens = [2 ** i for i in range(10, args.max_log2_seq + 1)]
     batch_size, head_size, dim = 1, 24, 64
     print(f"mode: {args.mode}, attn_method: {args.attn_method}, batch_size: {batch_size}, head_size: {head_size}, dim: {dim}")
     causal = not args.no_causal
     for seq_len in seq_lens:
         if args.attn_method == "flash":
-            ms = run_flash_attn(batch_size, head_size, seq_len, dim, causal)
+            ms = run_flash_attn(batch_size, head_size, seq_len, dim, causal, args.mode, rep=args.rep)
         else:
-            ms = run_hyper_attn(batch_size, head_size, seq_len, dim, causal, args.smooth_block)
+            ms = run_hyper_attn(batch_size, head_size, seq_len, dim, causal, args.smooth_block, args.mode, rep=args.rep)
         print(f"[{args.mode:<8}], {args.attn_method}, seq_len: {seq_len:<8}, causal: {causal}, "
               f"ms: {ms[0]:.5f} ({ms[1]:.5f}, {ms[2]:.5f}) | ", flush=True)
 

@@ -19,12 +19,15 @@ struct ha_attn_bwd_params {
   const float* lse;    // forward log-sum-exp (natural log), (batch, heads, n_q) by lse_sb / lse_sh
   const float* delta;  // sum_c dO*O per query, fp32, contiguous (batch, heads, n_q)
   void* dq;
-  float *dk32, *dv32;  // fp32 (batch, heads / kv_group, n_k, d) contiguous, added to with atomics
+  void *dk, *dv;       // written directly by the exact pass
+  float *dk32, *dv32;  // fp32 (batch, heads / kv_group, n_k, d) contiguous: the gathered passes' sums
   int64_t q_sb, q_sh, q_sn;
   int64_t k_sb, k_sh, k_sn;
   int64_t v_sb, v_sh, v_sn;
   int64_t do_sb, do_sh, do_sn;
   int64_t dq_sb, dq_sh, dq_sn;
+  int64_t dk_sb, dk_sh, dk_sn;
+  int64_t dv_sb, dv_sh, dv_sn;
   int64_t lse_sb, lse_sh;
   const void *q_idx, *k_idx, *sampled_idx;
   int64_t qi_sb, qi_sh, qi_sn;

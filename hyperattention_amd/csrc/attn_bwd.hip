@@ -20,9 +20,12 @@
 // Both compute S' = Y1 X1^T and dP' = Y2 X2^T (streamed rows as MFMA rows, stationary rows as MFMA
 // columns), so a lane holds 16 streamed rows of ONE stationary row and P', dS' are the B operands of
 // the products that follow, whose A operands (Y^T) come from the transposing LDS reads.  The dQ passes
-// see all keys of a query in one workgroup and store dQ; the dK/dV passes add into fp32 accumulators
-// in HBM with atomics (a key receives contributions from its block, from the sample list, and from
-// every query head of its group), which a last kernel rounds to the output type.
+// see all keys of a query in one workgroup and store dQ.  The dK/dV pass of exact attention sees all
+// queries of a key (of every query head of the key head's group, streamed one head after the other)
+// and stores dK, dV.  With sorted blocks a key gets one contribution from its block (complete in one
+// workgroup: stored as fp32) and, if it is in the sample list, one from every query: those are
+// computed per range of queries and added to the fp32 rows with atomics; a last kernel rounds the
+// fp32 rows to the output type.
 #include "ha_common.h"
 #include "attn_tiles.h"
 #include "attn_fwd.h"
@@ -68,20 +71,36 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_bwd_ker
   rest /= st_tiles;
   const int split = rest % splits;
   const int bh = rest / splits;
-  const int b = bh / p.heads, h = bh - b * p.heads;
-  const int hk = h / p.kv_group;
+  // The dK/dV passes that see every query of a key (exact attention, the blocks) take one workgroup per
+  // KEY head and stream the queries of all the query heads of its group, one head after the other, so
+  // that the sums are complete in registers; the other passes take one workgroup per query head.
+  constexpr bool GROUP_LOOP = PASS == HA_BWD_DKV_EXACT || PASS == HA_BWD_DKV_BLOCK;
   const int kv_heads = p.heads / p.kv_group;
+  int b, h0, hk;
+  if (GROUP_LOOP) {
+    b = bh / kv_heads;
+    hk = bh - b * kv_heads;
+    h0 = hk * p.kv_group;
+  } else {
+    b = bh / p.heads;
+    h0 = bh - b * p.heads;
+    hk = h0 / p.kv_group;
+  }
+  const int n_group = GROUP_LOOP ? p.kv_group : 1;
 
-  const unsigned char* const qb = (const unsigned char*)((const T*)p.q + b * p.q_sb + h * p.q_sh);
+  // query-side tensors of query head h0 + gi
+  auto q_head = [&](int gi) { return (const unsigned char*)((const T*)p.q + b * p.q_sb + (h0 + gi) * p.q_sh); };
+  auto do_head = [&](int gi) { return (const unsigned char*)((const T*)p.dout + b * p.do_sb + (h0 + gi) * p.do_sh); };
+  auto lse_head = [&](int gi) { return p.lse + b * p.lse_sb + (h0 + gi) * p.lse_sh; };
+  auto delta_head = [&](int gi) { return p.delta + (int64_t)(b * p.heads + h0 + gi) * p.n_q; };
+  const int idx_shift = p.idx64 ? 3 : 2;
+  auto q_idx_head = [&](int gi) {
+    return (const unsigned char*)p.q_idx + ((b * p.qi_sb + (h0 + gi) * p.qi_sh) << idx_shift);
+  };
   const unsigned char* const kb = (const unsigned char*)((const T*)p.k + b * p.k_sb + hk * p.k_sh);
   const unsigned char* const vb = (const unsigned char*)((const T*)p.v + b * p.v_sb + hk * p.v_sh);
-  const unsigned char* const dob = (const unsigned char*)((const T*)p.dout + b * p.do_sb + h * p.do_sh);
   const uint32_t q_rb = (uint32_t)p.q_sn * 2, k_rb = (uint32_t)p.k_sn * 2, v_rb = (uint32_t)p.v_sn * 2,
                  do_rb = (uint32_t)p.do_sn * 2;
-  const float* const lse_b = p.lse + b * p.lse_sb + h * p.lse_sh;
-  const float* const delta_b = p.delta + (int64_t)bh * p.n_q;
-  const int idx_shift = p.idx64 ? 3 : 2;
-  const unsigned char* const q_idx = (const unsigned char*)p.q_idx + ((b * p.qi_sb + h * p.qi_sh) << idx_shift);
   const unsigned char* const k_idx = (const unsigned char*)p.k_idx + ((b * p.ki_sb + hk * p.ki_sh) << idx_shift);
   const unsigned char* const s_idx =
       p.sampled_idx ? (const unsigned char*)p.sampled_idx + ((b * p.si_sb + hk * p.si_sh) << idx_shift) : nullptr;
@@ -89,11 +108,9 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_bwd_ker
   const uint32_t si_rb = 1u << idx_shift;
 
   // stationary (X) and streamed (Y) operands of this pass
-  const unsigned char* const x1b = KEY_ST ? kb : qb;
-  const unsigned char* const x2b = KEY_ST ? vb : dob;
+  const unsigned char* const x1b = KEY_ST ? kb : q_head(0);
+  const unsigned char* const x2b = KEY_ST ? vb : do_head(0);
   const uint32_t x1_rb = KEY_ST ? k_rb : q_rb, x2_rb = KEY_ST ? v_rb : do_rb;
-  const unsigned char* const y1b = KEY_ST ? qb : kb;
-  const unsigned char* const y2b = KEY_ST ? dob : vb;
   const uint32_t y1_rb = KEY_ST ? q_rb : k_rb, y2_rb = KEY_ST ? do_rb : v_rb;
   const int n_y = KEY_ST ? p.n_q : p.n_k;  // rows on the streamed side
 
@@ -104,7 +121,7 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_bwd_ker
   {
     const int pos = st_valid ? st_pos : 0;
     if (PASS == HA_BWD_DQ_BLOCK)
-      st_row = *reinterpret_cast<const int*>(row_address(q_idx, pos, qi_rb, 0));
+      st_row = *reinterpret_cast<const int*>(row_address(q_idx_head(0), pos, qi_rb, 0));
     else if (PASS == HA_BWD_DKV_BLOCK)
       st_row = *reinterpret_cast<const int*>(row_address(k_idx, pos, ki_rb, 0));
     else if (PASS == HA_BWD_DKV_SAMPLED)
@@ -120,8 +137,8 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_bwd_ker
   }
   float st_lse2 = 0.f, st_delta = 0.f;  // dQ passes: the lane's query
   if (!KEY_ST) {
-    st_lse2 = lse_b[st_row] * LOG2E;
-    st_delta = delta_b[st_row];
+    st_lse2 = lse_head(0)[st_row] * LOG2E;
+    st_delta = delta_head(0)[st_row];
   }
 
   // ---- the streamed chunks of this workgroup ---------------------------------------------------
@@ -204,7 +221,8 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_bwd_ker
       nc = 2 * lds_ntiles;
     }
   }
-  nc = __builtin_amdgcn_readfirstlane(nc);
+  const int nc_head = __builtin_amdgcn_readfirstlane(nc);  // chunks per query head
+  nc = nc_head * n_group;
 
   // Original row of streamed row r (0..63) of chunk c, clamped to rows that exist; chunks past the
   // end repeat the last one.  Gathered passes read an index array here.
@@ -212,8 +230,11 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_bwd_ker
     if (PASS != HA_BWD_DKV_BLOCK) return 0;
     return p.smooth ? lds_tiles[k] : ((t_first + k) | (int)(3u << 30));
   };
+  auto group_of = [&](int c) -> int { return n_group == 1 ? 0 : (c < nc ? c : nc - 1) / nc_head; };
   auto stream_row = [&](int c, int r) -> int {
     c = c < nc ? c : nc - 1;
+    const int gi = group_of(c);
+    c -= gi * nc_head;
     if (PASS == HA_BWD_DQ_BLOCK) {
       if (c < n_blk) {
         int u = blk_start + c;
@@ -224,7 +245,7 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_bwd_ker
       return s_idx ? *reinterpret_cast<const int*>(row_address(s_idx, s, si_rb, 0)) : s;
     } else if (PASS == HA_BWD_DKV_BLOCK) {
       const int t = attending_tile(c >> 1) & 0x3fffffff;
-      return *reinterpret_cast<const int*>(row_address(q_idx, t * 128 + (c & 1) * YC + r, qi_rb, 0));
+      return *reinterpret_cast<const int*>(row_address(q_idx_head(gi), t * 128 + (c & 1) * YC + r, qi_rb, 0));
     } else {
       const int row = y_first + c * YC + r;
       return row < n_y ? row : n_y - 1;
@@ -233,13 +254,28 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_bwd_ker
 
   if (nc <= 0) {
     // nothing attends (or is attended by) this tile: its gradient is zero
-    if (!KEY_ST && st_valid) {
-      unsigned char* const dqb = (unsigned char*)((T*)p.dq + b * p.dq_sb + h * p.dq_sh) + (int64_t)st_row * p.dq_sn * 2;
+    if (PASS != HA_BWD_DKV_SAMPLED && st_valid) {
       const vec4 zero = {(T)0.f, (T)0.f, (T)0.f, (T)0.f};
+      const f32x4 zero32 = {0.f, 0.f, 0.f, 0.f};
+      unsigned char* const dqb = (unsigned char*)((T*)p.dq + b * p.dq_sb + h0 * p.dq_sh) + (int64_t)st_row * p.dq_sn * 2;
+      unsigned char* const dkb = (unsigned char*)((T*)p.dk + b * p.dk_sb + hk * p.dk_sh) + (int64_t)st_row * p.dk_sn * 2;
+      unsigned char* const dvb = (unsigned char*)((T*)p.dv + b * p.dv_sb + hk * p.dv_sh) + (int64_t)st_row * p.dv_sn * 2;
+      const int64_t head_off = ((int64_t)(b * kv_heads + hk) * p.n_k + st_row) * D;
 #pragma unroll
       for (int db = 0; db < DB; ++db)
 #pragma unroll
-        for (int g = 0; g < 4; ++g) *reinterpret_cast<vec4*>(dqb + (32 * db + 8 * g + 4 * hi) * 2) = zero;
+        for (int g = 0; g < 4; ++g) {
+          const int dd = 32 * db + 8 * g + 4 * hi;
+          if (!KEY_ST) {
+            *reinterpret_cast<vec4*>(dqb + dd * 2) = zero;
+          } else if (PASS == HA_BWD_DKV_EXACT) {
+            *reinterpret_cast<vec4*>(dkb + dd * 2) = zero;
+            *reinterpret_cast<vec4*>(dvb + dd * 2) = zero;
+          } else {
+            *reinterpret_cast<f32x4*>(p.dk32 + head_off + dd) = zero32;
+            *reinterpret_cast<f32x4*>(p.dv32 + head_off + dd) = zero32;
+          }
+        }
     }
     return;
   }
@@ -248,14 +284,18 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_bwd_ker
   const int my_pp = lane % PR;  // physical piece of this lane's LDS slot
   const int my_lr = lane / PR;  // row inside one tile load
   int rows_next[LPW];           // source rows of this wave's loads of the next tile
+  int group_next = 0;           // the query head (within the group) those rows belong to
   int stat_row_next = 0;        // wave 0, dK/dV passes: source row of streamed row `lane` of the next tile
   float stat_lse = 0.f, stat_delta = 0.f;
   auto fetch_rows = [&](int c) {
 #pragma unroll
     for (int j = 0; j < LPW; ++j) rows_next[j] = stream_row(c, (wave_s * LPW + j) * RPL + my_lr);
     if (KEY_ST && wave_s == 0) stat_row_next = stream_row(c, lane);
+    group_next = group_of(c);
   };
   auto load_tile = [&](int buf) {  // the tile whose rows are in rows_next
+    const unsigned char* const y1b = KEY_ST ? q_head(group_next) : kb;
+    const unsigned char* const y2b = KEY_ST ? do_head(group_next) : vb;
 #pragma unroll
     for (int j = 0; j < LPW; ++j) {
       const int r = (wave_s * LPW + j) * RPL + my_lr;
@@ -266,8 +306,8 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_bwd_ker
       global_to_lds_16(row_address(y2b, rows_next[j], y2_rb, piece), dst2);
     }
     if (KEY_ST && wave_s == 0) {
-      stat_lse = lse_b[stat_row_next] * LOG2E;
-      stat_delta = delta_b[stat_row_next];
+      stat_lse = lse_head(group_next)[stat_row_next] * LOG2E;
+      stat_delta = delta_head(group_next)[stat_row_next];
     }
   };
 
@@ -312,8 +352,9 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_bwd_ker
 
     // does this wave take part in the chunk at all (smoothed blocks: the window of a query tile can end
     // between the two 64-key halves of the stationary tile)
+    const int cc = c - group_of(c) * nc_head;  // chunk number within its query head
     bool wave_in = true;
-    if (PASS == HA_BWD_DKV_BLOCK) wave_in = (attending_tile(c >> 1) >> (30 + (wave_s >> 1))) & 1;
+    if (PASS == HA_BWD_DKV_BLOCK) wave_in = (attending_tile(cc >> 1) >> (30 + (wave_s >> 1))) & 1;
 
     if (wave_in) {
       const unsigned char* const y1 = lds_y1[buf];
@@ -352,13 +393,13 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_bwd_ker
             const int i = g * 4 + e;
             bool ok = true;
             if (PASS == HA_BWD_DQ_EXACT) {
-              const int key = c * YC + r0 + e;
+              const int key = cc * YC + r0 + e;
               ok = key < p.n_k && (!CAUSAL || key <= st_pos);
             } else if (PASS == HA_BWD_DKV_EXACT) {
-              const int query = y_first + c * YC + r0 + e;
+              const int query = y_first + cc * YC + r0 + e;
               ok = query < p.n_q && (!CAUSAL || st_pos <= query);
             } else if (PASS == HA_BWD_DKV_SAMPLED) {
-              ok = y_first + c * YC + r0 + e < y_end;
+              ok = y_first + cc * YC + r0 + e < y_end;
             }
             float pv = __builtin_amdgcn_exp2f(__builtin_fmaf(s[rb][i], p.scale_log2, -l4[e]));
             pv = ok ? pv : 0.f;
@@ -387,9 +428,8 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_bwd_ker
   }
 
   // ---- results -------------------------------------------------------------------------------
-  if (!st_valid) return;
-  if (!KEY_ST) {
-    unsigned char* const dqb = (unsigned char*)((T*)p.dq + b * p.dq_sb + h * p.dq_sh) + (int64_t)st_row * p.dq_sn * 2;
+  if (!KEY_ST && st_valid) {
+    unsigned char* const dqb = (unsigned char*)((T*)p.dq + b * p.dq_sb + h0 * p.dq_sh) + (int64_t)st_row * p.dq_sn * 2;
 #pragma unroll
     for (int db = 0; db < DB; ++db)
 #pragma unroll
@@ -399,18 +439,70 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_bwd_ker
         for (int e = 0; e < 4; ++e) o[e] = (T)acc1[db][g * 4 + e];
         *reinterpret_cast<vec4*>(dqb + (32 * db + 8 * g + 4 * hi) * 2) = o;
       }
-  } else {
+  } else if (PASS == HA_BWD_DKV_EXACT && st_valid) {
+    // complete sums: straight to dk, dv
+    unsigned char* const dkb = (unsigned char*)((T*)p.dk + b * p.dk_sb + hk * p.dk_sh) + (int64_t)st_row * p.dk_sn * 2;
+    unsigned char* const dvb = (unsigned char*)((T*)p.dv + b * p.dv_sb + hk * p.dv_sh) + (int64_t)st_row * p.dv_sn * 2;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        vec4 ok_, ov_;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          ok_[e] = (T)acc1[db][g * 4 + e];
+          ov_[e] = (T)acc2[db][g * 4 + e];
+        }
+        *reinterpret_cast<vec4*>(dkb + (32 * db + 8 * g + 4 * hi) * 2) = ok_;
+        *reinterpret_cast<vec4*>(dvb + (32 * db + 8 * g + 4 * hi) * 2) = ov_;
+      }
+  } else if (PASS == HA_BWD_DKV_BLOCK && st_valid) {
+    // every key is in exactly one tile of the sorted order: this is the first write of its fp32 row
     const int64_t head_off = ((int64_t)(b * kv_heads + hk) * p.n_k + st_row) * D;
     float* const dk_row = p.dk32 + head_off;
     float* const dv_row = p.dv32 + head_off;
 #pragma unroll
     for (int db = 0; db < DB; ++db)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const int dd = 32 * db + 8 * (i >> 2) + 4 * hi + (i & 3);
-        unsafeAtomicAdd(dk_row + dd, acc1[db][i]);
-        unsafeAtomicAdd(dv_row + dd, acc2[db][i]);
+      for (int g = 0; g < 4; ++g) {
+        const int dd = 32 * db + 8 * g + 4 * hi;
+        *reinterpret_cast<f32x4*>(dk_row + dd) =
+            f32x4{acc1[db][g * 4], acc1[db][g * 4 + 1], acc1[db][g * 4 + 2], acc1[db][g * 4 + 3]};
+        *reinterpret_cast<f32x4*>(dv_row + dd) =
+            f32x4{acc2[db][g * 4], acc2[db][g * 4 + 1], acc2[db][g * 4 + 2], acc2[db][g * 4 + 3]};
       }
+  }
+  if (PASS == HA_BWD_DKV_SAMPLED) {
+    // Sampled keys: partial sums over one range of queries of one query head, added on top of the rows
+    // with atomics.  Each wave turns its 32 x D results around in LDS (its quarter of the tile buffers,
+    // free once every wave has left the loop) so that one atomic instruction covers 64 consecutive floats
+    // of one row instead of one float of each of 64 rows.
+    __syncthreads();
+    float* const turn = reinterpret_cast<float*>(wave_s < 2 ? lds_y1[wave_s] : lds_y2[wave_s - 2]);
+    const int64_t head_base = (int64_t)(b * kv_heads + hk) * p.n_k * D;
+#pragma unroll
+    for (int which = 0; which < 2; ++which) {
+      float* const dst = (which == 0 ? p.dk32 : p.dv32) + head_base;
+      // [key][D] fp32, the 16-byte pieces of a row XOR-ed with the key number: conflict-free both ways
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const f32x16& a = which == 0 ? acc1[db] : acc2[db];
+          const int piece = (8 * db + 2 * g + hi) ^ (col & 15);
+          *reinterpret_cast<f32x4*>(turn + col * D + piece * 4) = f32x4{a[g * 4], a[g * 4 + 1], a[g * 4 + 2], a[g * 4 + 3]};
+        }
+      for (int r = 0; r < 32; ++r) {
+        const int row = __shfl(st_row, r);
+        const bool valid = __shfl((int)st_valid, r) != 0;
+#pragma unroll
+        for (int part = 0; part < D / 64; ++part) {
+          const int dd = part * 64 + lane;
+          const float val = turn[r * D + (((dd >> 2) ^ (r & 15)) << 2) + (dd & 3)];
+          if (valid) unsafeAtomicAdd(dst + (int64_t)row * D + dd, val);
+        }
+      }
+    }
   }
 }
 
@@ -439,11 +531,6 @@ __global__ __launch_bounds__(256) void ha_bwd_delta_kernel(const T* __restrict__
 #pragma unroll
   for (int m = 1; m < PR; m <<= 1) acc += __shfl_xor(acc, m);
   if (grow < total_rows && piece == 0) delta[grow] = acc;
-}
-
-__global__ __launch_bounds__(256) void ha_bwd_zero_kernel(f32x4* __restrict__ buf, int64_t n4) {
-  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < n4) buf[i] = f32x4{0.f, 0.f, 0.f, 0.f};
 }
 
 // fp32 accumulators (batch, kv_heads, n_k, D) -> dk, dv in the output type, 8 elements per lane
@@ -533,12 +620,14 @@ int check_grads(const ha_attn_operands& t, const ha_attn_grads& g, const char* w
 void fill_bwd_params(const ha_attn_operands& t, const ha_attn_grads& g, const Workspace& w, ha_attn_bwd_params& p) {
   p.q = t.q; p.k = t.k; p.v = t.v; p.dout = g.dout;
   p.lse = t.lse; p.delta = w.delta;
-  p.dq = g.dq; p.dk32 = w.dk32; p.dv32 = w.dv32;
+  p.dq = g.dq; p.dk = g.dk; p.dv = g.dv; p.dk32 = w.dk32; p.dv32 = w.dv32;
   p.q_sb = t.q_stride_b; p.q_sh = t.q_stride_h; p.q_sn = t.q_stride_n;
   p.k_sb = t.k_stride_b; p.k_sh = t.k_stride_h; p.k_sn = t.k_stride_n;
   p.v_sb = t.v_stride_b; p.v_sh = t.v_stride_h; p.v_sn = t.v_stride_n;
   p.do_sb = g.do_stride_b; p.do_sh = g.do_stride_h; p.do_sn = g.do_stride_n;
   p.dq_sb = g.dq_stride_b; p.dq_sh = g.dq_stride_h; p.dq_sn = g.dq_stride_n;
+  p.dk_sb = g.dk_stride_b; p.dk_sh = g.dk_stride_h; p.dk_sn = g.dk_stride_n;
+  p.dv_sb = g.dv_stride_b; p.dv_sh = g.dv_stride_h; p.dv_sn = g.dv_stride_n;
   p.lse_sb = t.lse_stride_b; p.lse_sh = t.lse_stride_h;
   p.q_idx = p.k_idx = p.sampled_idx = nullptr;
   p.qi_sb = p.qi_sh = p.qi_sn = 0;
@@ -552,7 +641,7 @@ void fill_bwd_params(const ha_attn_operands& t, const ha_attn_grads& g, const Wo
   p.scale_log2 = t.scale * LOG2E;
 }
 
-// delta, and zeroed accumulators
+// D_i for every query
 template <typename T, int D>
 int launch_prepare(const ha_attn_operands& t, const ha_attn_grads& g, const Workspace& w, hipStream_t stream) {
   const int64_t rows = t.batch * t.heads * t.n_q;
@@ -560,13 +649,7 @@ int launch_prepare(const ha_attn_operands& t, const ha_attn_grads& g, const Work
   hipLaunchKernelGGL((ha_bwd_delta_kernel<T, D>), dim3((unsigned)((items + 255) / 256)), dim3(256), 0, stream,
                      (const T*)t.out, (const T*)g.dout, w.delta, (int)t.heads, (int)t.n_q, t.o_stride_b, t.o_stride_h,
                      t.o_stride_n, g.do_stride_b, g.do_stride_h, g.do_stride_n, rows);
-  int st = ha_launch_status("attention backward: delta");
-  if (st != HA_OK) return st;
-  // the two accumulators are adjacent up to alignment padding: clear them with one launch each
-  const int64_t n4 = (w.acc_floats + 3) / 4;
-  hipLaunchKernelGGL(ha_bwd_zero_kernel, dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, stream, (f32x4*)w.dk32, n4);
-  hipLaunchKernelGGL(ha_bwd_zero_kernel, dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, stream, (f32x4*)w.dv32, n4);
-  return ha_launch_status("attention backward: clear");
+  return ha_launch_status("attention backward: delta");
 }
 
 template <typename T, int D>
@@ -596,15 +679,16 @@ int run_block_bwd(const ha_block_attn_args& a, const ha_attn_grads& g, hipStream
   p.sample_size = (int)a.sample_size;
   p.smooth = a.smooth_block != 0;
   p.idx64 = a.idx_type == HA_IDX_I64;
-  const int64_t bh = t.batch * t.heads;
+  const int64_t bh = t.batch * t.heads, bhk = t.batch * (t.heads / t.kv_group);
   st = launch_pass<T, D, HA_BWD_DQ_BLOCK, false>(p, bh * (t.n_q / ST_ROWS), stream, "ha_block_attn_bwd: dq");
   if (st != HA_OK) return st;
-  st = launch_pass<T, D, HA_BWD_DKV_BLOCK, false>(p, bh * (t.n_k / ST_ROWS), stream, "ha_block_attn_bwd: dk, dv of the blocks");
+  st = launch_pass<T, D, HA_BWD_DKV_BLOCK, false>(p, bhk * (t.n_k / ST_ROWS), stream, "ha_block_attn_bwd: dk, dv of the blocks");
   if (st != HA_OK) return st;
   if (a.sample_size > 0) {
-    // every query attends every sampled key: cut the queries into ranges so that the grid fills the chip
-    int64_t q_split = 2048;
-    while (q_split > 256 && bh * (a.sample_size / ST_ROWS) * ((t.n_q + q_split - 1) / q_split) < 2048) q_split /= 2;
+    // every query attends every sampled key: the queries are cut into ranges, as long as possible (each
+    // range ends in one atomic add per element of the sampled rows) while two workgroups per CU remain
+    int64_t q_split = 8192;
+    while (q_split > 512 && bh * (a.sample_size / ST_ROWS) * ((t.n_q + q_split - 1) / q_split) < 512) q_split /= 2;
     p.q_split = (int)q_split;
     const int64_t splits = (t.n_q + q_split - 1) / q_split;
     st = launch_pass<T, D, HA_BWD_DKV_SAMPLED, false>(p, bh * (a.sample_size / ST_ROWS) * splits, stream,
@@ -621,19 +705,18 @@ int run_flash_bwd(const ha_attn_operands& t, bool causal, const ha_attn_grads& g
   if (st != HA_OK) return st;
   ha_attn_bwd_params p;
   fill_bwd_params(t, g, w, p);
-  const int64_t bh = t.batch * t.heads;
+  const int64_t bh = t.batch * t.heads, bhk = t.batch * (t.heads / t.kv_group);
   const int64_t q_tiles = (t.n_q + ST_ROWS - 1) / ST_ROWS, k_tiles = (t.n_k + ST_ROWS - 1) / ST_ROWS;
   if (causal) {
     st = launch_pass<T, D, HA_BWD_DQ_EXACT, true>(p, bh * q_tiles, stream, "ha_flash_attn_bwd: dq");
     if (st != HA_OK) return st;
-    st = launch_pass<T, D, HA_BWD_DKV_EXACT, true>(p, bh * k_tiles, stream, "ha_flash_attn_bwd: dk, dv");
+    st = launch_pass<T, D, HA_BWD_DKV_EXACT, true>(p, bhk * k_tiles, stream, "ha_flash_attn_bwd: dk, dv");
   } else {
     st = launch_pass<T, D, HA_BWD_DQ_EXACT, false>(p, bh * q_tiles, stream, "ha_flash_attn_bwd: dq");
     if (st != HA_OK) return st;
-    st = launch_pass<T, D, HA_BWD_DKV_EXACT, false>(p, bh * k_tiles, stream, "ha_flash_attn_bwd: dk, dv");
+    st = launch_pass<T, D, HA_BWD_DKV_EXACT, false>(p, bhk * k_tiles, stream, "ha_flash_attn_bwd: dk, dv");
   }
-  if (st != HA_OK) return st;
-  return launch_round<T, D>(t, g, w, stream);
+  return st;
 }
 
 }  // namespace

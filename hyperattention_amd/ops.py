@@ -304,6 +304,8 @@ class HyperAttnFunc(torch.autograd.Function):
         o, lse = hyper_attn_func(q, k, v, q_sort_idx, k_sort_idx, block_size, sample_size, softmax_scale,
                                  smooth_block, sampled_idx=sampled_idx)
         ctx.save_for_backward(q, k, v, q_sort_idx, k_sort_idx, o, lse)
+        # no gradient is returned for lse: saying so up front keeps autograd from computing one
+        ctx.mark_non_differentiable(lse)
         ctx.sampled_idx = sampled_idx
         ctx.conf = (block_size, sample_size, softmax_scale or 1.0 / math.sqrt(q.shape[-1]), smooth_block)
         return o, lse
@@ -329,6 +331,7 @@ class FlashAttnFunc(torch.autograd.Function):
     def forward(ctx, q, k, v, bias, causal, softmax_scale):
         o, lse = flash_attn_func(q, k, v, bias, causal, softmax_scale)
         ctx.save_for_backward(q, k, v, o, lse)
+        ctx.mark_non_differentiable(lse)
         ctx.conf = (bool(causal), softmax_scale or 1.0 / math.sqrt(q.shape[-1]))
         return o, lse
 

@@ -156,11 +156,11 @@ def test_python_layer_fails_loudly_without_library(monkeypatch, tmp_path):
 
 
 def test_sweep_script_command_line():
-    """The sweep keeps the reference's options (benchmark_single_attention.py:14-22); the modes that
-    need a backward pass stop before touching the GPU."""
+    """The sweep keeps the reference's options (benchmark_single_attention.py:14-22)."""
     from hyperattention_amd import benchmark_single_attention as sweep
     args = sweep.get_arguments(["--no_causal", "--smooth_block", "--mode", "fwd", "--attn_method", "hyper"])
     assert args.no_causal and args.smooth_block and args.mode == "fwd" and args.attn_method == "hyper"
     for mode in ("bwd", "fwd+bwd"):
-        with pytest.raises(SystemExit):
-            sweep.main(["--mode", mode, "--attn_method", "hyper"])
+        assert sweep.get_arguments(["--mode", mode]).mode == mode
+    with pytest.raises(SystemExit):  # a CUDA-only package: stops before touching the GPU
+        sweep.main(["--attn_method", "flash-cuda"])

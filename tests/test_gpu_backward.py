@@ -165,6 +165,51 @@ def test_block_backward_int32_indices_and_sorted_buckets(ha):
         _check(got, want, f"block {name}", dtype)
 
 
+# ------------------------------------------------------------------------- grouped-query heads
+@pytest.mark.parametrize("kind", ["flash", "flash_causal", "block"])
+def test_backward_grouped_query_heads_through_the_c_abi(ha, kind):
+    # 4 query heads on 2 key/value heads, handed to the C entry points as they are (kv_group = 2): the
+    # gradient of a key head is the sum over the query heads of its group
+    import ctypes
+    from hyperattention_amd import _lib, ops
+    dtype, b, h, hk, n, d, block, sample = torch.float16, 1, 4, 2, 512, 64, 256, 128
+    q = _randn((b, h, n, d), 61, dtype)
+    k = _randn((b, hk, n, d), 62, dtype)
+    v = _randn((b, hk, n, d), 63, dtype)
+    do = _randn((b, h, n, d), 64, dtype)
+    qi, ki = _perms(b, h, n, 65), _perms(b, hk, n, 66)
+    expand = lambda x: x.repeat_interleave(h // hk, dim=1)
+    if kind == "block":
+        fn = lambda a, b_, c: O.block_sampled_attention(a, expand(b_), expand(c), qi, expand(ki), block, sample)
+    else:
+        fn = lambda a, b_, c: O.exact_attention(a, expand(b_), expand(c), None, kind == "flash_causal")
+    ref = _oracle_grads(fn, q, k, v, do)
+
+    qg, kg, vg, dog = (x.cuda().transpose(1, 2).contiguous() for x in (q, k, v, do))  # (b,n,heads,d)
+    o = torch.empty_like(qg)
+    lse = torch.empty((b, h, n), device="cuda", dtype=torch.float32)
+    dq, dk, dv = torch.empty_like(qg), torch.empty_like(kg), torch.empty_like(vg)
+    lib = _lib.lib()
+    stream = ops._stream(qg)
+    if kind == "block":
+        qi_g, ki_g = qi.cuda().transpose(1, 2), ki.cuda().transpose(1, 2)
+        a, keep = ops._block_attn_args(qg, kg, vg, o, lse, qi_g, ki_g, block, sample, d ** -0.5, False, None)
+        assert a.t.kv_group == 2
+        _lib.check(lib.ha_block_attn_fwd(ctypes.byref(a), stream))
+        g, ws = ops._attn_grads(a.t, dog, dq, dk, dv)
+        _lib.check(lib.ha_block_attn_bwd(ctypes.byref(a), ctypes.byref(g), stream))
+    else:
+        t = ops._operands(qg, kg, vg, o, lse, d ** -0.5, layout_bnhd=True, lse_row_stride=n)
+        assert t.kv_group == 2
+        causal = int(kind == "flash_causal")
+        _lib.check(lib.ha_flash_attn_fwd(ctypes.byref(t), causal, stream))
+        g, ws = ops._attn_grads(t, dog, dq, dk, dv)
+        _lib.check(lib.ha_flash_attn_bwd(ctypes.byref(t), causal, ctypes.byref(g), stream))
+    torch.cuda.synchronize()
+    for got, want, name in zip((dq, dk, dv), ref, ("dq", "dk", "dv")):
+        _check(got.transpose(1, 2), want, f"{kind} {name}", dtype)
+
+
 # ------------------------------------------------------------------------------- the module
 @pytest.mark.parametrize("causal,n,min_seq_len", [(False, 1024, 256), (True, 1024, 256), (True, 1025, 600)])
 def test_module_backward(ha, causal, n, min_seq_len):
