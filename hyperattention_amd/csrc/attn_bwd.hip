@@ -31,6 +31,8 @@
 #include "attn_fwd.h"
 #include "attn_bwd.h"
 
+#include <type_traits>
+
 namespace {
 
 constexpr int WG_THREADS = 256;
@@ -53,7 +55,7 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_bwd_ker
   __shared__ __attribute__((aligned(1024))) unsigned char lds_y1[2][TILE_BYTES];
   __shared__ __attribute__((aligned(1024))) unsigned char lds_y2[2][TILE_BYTES];
   __shared__ __attribute__((aligned(16))) float lds_lse[2][YC];    // dK/dV passes: L (log2 units) of the streamed queries
-  __shared__ __attribute__((aligned(16))) float lds_delta[2][YC];  // and their D
+  __shared__ __attribute__((aligned(16))) float lds_delta[2][YC];  // and their D * scale
   __shared__ int lds_tiles[PASS == HA_BWD_DKV_BLOCK ? MAX_SMOOTH_TILES : 1];
   __shared__ int lds_ntiles;
 
@@ -135,10 +137,10 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_bwd_ker
     x1f[ks] = *reinterpret_cast<const vec8*>(row_address(x1b, st_row, x1_rb, (ks * 16 + hi * 8) * 2));
     x2f[ks] = *reinterpret_cast<const vec8*>(row_address(x2b, st_row, x2_rb, (ks * 16 + hi * 8) * 2));
   }
-  float st_lse2 = 0.f, st_delta = 0.f;  // dQ passes: the lane's query
+  float st_lse2 = 0.f, st_delta = 0.f;  // dQ passes: L (log2 units) and D * scale of the lane's query
   if (!KEY_ST) {
     st_lse2 = lse_head(0)[st_row] * LOG2E;
-    st_delta = delta_head(0)[st_row];
+    st_delta = delta_head(0)[st_row] * p.scale;
   }
 
   // ---- the streamed chunks of this workgroup ---------------------------------------------------
@@ -307,7 +309,7 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_bwd_ker
     }
     if (KEY_ST && wave_s == 0) {
       stat_lse = lse_head(group_next)[stat_row_next] * LOG2E;
-      stat_delta = delta_head(group_next)[stat_row_next];
+      stat_delta = delta_head(group_next)[stat_row_next] * p.scale;
     }
   };
 
@@ -353,8 +355,21 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_bwd_ker
     // does this wave take part in the chunk at all (smoothed blocks: the window of a query tile can end
     // between the two 64-key halves of the stationary tile)
     const int cc = c - group_of(c) * nc_head;  // chunk number within its query head
-    bool wave_in = true;
-    if (PASS == HA_BWD_DKV_BLOCK) wave_in = (attending_tile(cc >> 1) >> (30 + (wave_s >> 1))) & 1;
+    bool wave_in = true;      // does the wave have any pair in this chunk
+    bool needs_mask = false;  // and are some of its pairs masked
+    const int y_lo = y_first + cc * YC, y_hi = y_lo + YC - 1;             // streamed rows of the chunk (exact, sampled)
+    const int st_lo = tile * ST_ROWS + wave_s * 32, st_hi = st_lo + 31;  // stationary positions of the wave
+    if (PASS == HA_BWD_DKV_BLOCK) {
+      wave_in = (attending_tile(cc >> 1) >> (30 + (wave_s >> 1))) & 1;
+    } else if (PASS == HA_BWD_DQ_EXACT) {
+      wave_in = !CAUSAL || y_lo <= st_hi;
+      needs_mask = y_hi >= p.n_k || (CAUSAL && y_hi > st_lo);
+    } else if (PASS == HA_BWD_DKV_EXACT) {
+      wave_in = !CAUSAL || y_hi >= st_lo;
+      needs_mask = y_hi >= p.n_q || (CAUSAL && y_lo < st_hi);
+    } else if (PASS == HA_BWD_DKV_SAMPLED) {
+      needs_mask = y_hi >= y_end;
+    }
 
     if (wave_in) {
       const unsigned char* const y1 = lds_y1[buf];
@@ -376,38 +391,49 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_bwd_ker
         }
       }
 
-      // P' and dS' of the lane's 32 (streamed row, stationary row) pairs, rounded to the input type
+      // P' and dS' of the lane's 32 (streamed row, stationary row) pairs, rounded to the input type.
+      // Only chunks that touch the diagonal or the end of the sequence pay for the mask.
       vec8 pb[2][2], dsb[2][2];
+      auto softmax_grad = [&](auto masked_tag) {
+        constexpr bool MASKED = decltype(masked_tag)::value;
 #pragma unroll
-      for (int rb = 0; rb < 2; ++rb)
+        for (int rb = 0; rb < 2; ++rb)
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          const int r0 = rb * 32 + g * 8 + hi * 4;  // streamed rows r0..r0+3 of the chunk
-          f32x4 l4 = {st_lse2, st_lse2, st_lse2, st_lse2}, d4 = {st_delta, st_delta, st_delta, st_delta};
-          if (KEY_ST) {
-            l4 = *reinterpret_cast<const f32x4*>(&lds_lse[buf][r0]);
-            d4 = *reinterpret_cast<const f32x4*>(&lds_delta[buf][r0]);
-          }
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const int i = g * 4 + e;
-            bool ok = true;
-            if (PASS == HA_BWD_DQ_EXACT) {
-              const int key = cc * YC + r0 + e;
-              ok = key < p.n_k && (!CAUSAL || key <= st_pos);
-            } else if (PASS == HA_BWD_DKV_EXACT) {
-              const int query = y_first + cc * YC + r0 + e;
-              ok = query < p.n_q && (!CAUSAL || st_pos <= query);
-            } else if (PASS == HA_BWD_DKV_SAMPLED) {
-              ok = y_first + cc * YC + r0 + e < y_end;
+          for (int g = 0; g < 4; ++g) {
+            const int r0 = rb * 32 + g * 8 + hi * 4;  // streamed rows r0..r0+3 of the chunk
+            f32x4 l4 = {st_lse2, st_lse2, st_lse2, st_lse2}, d4 = {st_delta, st_delta, st_delta, st_delta};
+            if (KEY_ST) {
+              l4 = *reinterpret_cast<const f32x4*>(&lds_lse[buf][r0]);
+              d4 = *reinterpret_cast<const f32x4*>(&lds_delta[buf][r0]);
             }
-            float pv = __builtin_amdgcn_exp2f(__builtin_fmaf(s[rb][i], p.scale_log2, -l4[e]));
-            pv = ok ? pv : 0.f;
-            const float dsv = pv * (dp[rb][i] - d4[e]) * p.scale;
-            pb[rb][i >> 3][i & 7] = (T)pv;
-            dsb[rb][i >> 3][i & 7] = (T)dsv;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const int i = g * 4 + e;
+              float pv = __builtin_amdgcn_exp2f(__builtin_fmaf(s[rb][i], p.scale_log2, -l4[e]));
+              if (MASKED) {
+                bool ok = true;
+                if (PASS == HA_BWD_DQ_EXACT) {
+                  const int key = cc * YC + r0 + e;
+                  ok = key < p.n_k && (!CAUSAL || key <= st_pos);
+                } else if (PASS == HA_BWD_DKV_EXACT) {
+                  const int query = y_first + cc * YC + r0 + e;
+                  ok = query < p.n_q && (!CAUSAL || st_pos <= query);
+                } else if (PASS == HA_BWD_DKV_SAMPLED) {
+                  ok = y_first + cc * YC + r0 + e < y_end;
+                }
+                pv = ok ? pv : 0.f;
+              }
+              // d4 holds D * scale: dS = P (dP - D) scale in one FMA and one product
+              const float dsv = pv * __builtin_fmaf(dp[rb][i], p.scale, -d4[e]);
+              pb[rb][i >> 3][i & 7] = (T)pv;
+              dsb[rb][i >> 3][i & 7] = (T)dsv;
+            }
           }
-        }
+      };
+      if (needs_mask)
+        softmax_grad(std::true_type{});
+      else
+        softmax_grad(std::false_type{});
 
       // the products that contract over the streamed rows
 #pragma unroll
