@@ -38,7 +38,50 @@ namespace {
 constexpr int WG_THREADS = 256;
 constexpr int ST_ROWS = 128;       // stationary rows per workgroup
 constexpr int YC = 64;             // streamed rows per LDS tile
+#ifndef BWD_VALU_PER
+#define BWD_VALU_PER 5
+#endif
+#ifndef BWD_TRANS_PER
+#define BWD_TRANS_PER 2
+#endif
 constexpr int MAX_SMOOTH_TILES = 1024;  // query tiles that can attend one 128-key tile (smoothed blocks)
+
+// LDS layout of a streamed tile: row-major [64][D] 2-byte elements, the 16-byte pieces of a row XOR-ed
+// with a function of the row number chosen so that BOTH ways the tile is read are free of bank
+// conflicts (the LDS serves 16 lanes, 64 banks of 4 bytes, at a time):
+//   row reads (ds_read_b128): 16 lanes read the same piece of 16 consecutive rows -> the 16 rows
+//     must land in 16 different 16-byte slots of the 256-byte bank window;
+//   transposing reads (ds_read_b64_tr_b16): 16 lanes read 2 adjacent pieces of 4 consecutive rows
+//     (starting at a multiple of 4) -> the four pairs must differ in a bit above the lowest.
+// d = 64 (a row is half a bank window, so rows of equal parity compete for 8 slots): the bits 1,2,3
+// of the row number, in reversed order.  d = 128 (16 slots per row): the low four bits of the row
+// number with the two pairs of bits exchanged.
+template <int D>
+__device__ __forceinline__ int bwd_swizzle(int row) {
+  if (D == 64) return (((row >> 1) & 1) << 2) | (((row >> 2) & 1) << 1) | ((row >> 3) & 1);
+  return ((row & 3) << 2) | ((row >> 2) & 3);
+}
+template <int D>
+__device__ __forceinline__ int bwd_tile_offset(int row, int piece) {
+  return row * D * 2 + ((piece ^ bwd_swizzle<D>(row)) << 4);
+}
+
+// 8 streamed rows x 1 column, transposed by the LDS unit: rows 0..3 and 8..11 (+4 for the upper lane
+// half) relative to the row the offsets were computed for
+template <typename T>
+__device__ __forceinline__ typename ElemTraits<T>::vec8 bwd_read_tr(const unsigned char* tile, int off_lo, int off_hi) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  typedef short s16x4 __attribute__((ext_vector_type(4)));
+  typedef short s16x8 __attribute__((ext_vector_type(8)));
+  typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+  const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(tile + off_lo));
+  const s16x4 hi8 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(tile + off_hi));
+  const s16x8 both = __builtin_shufflevector(lo, hi8, 0, 1, 2, 3, 4, 5, 6, 7);
+  return __builtin_bit_cast(typename ElemTraits<T>::vec8, both);
+#else
+  return typename ElemTraits<T>::vec8{};
+#endif
+}
 
 template <typename T, int D, int PASS, bool CAUSAL>
 __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_bwd_kernel(const ha_attn_bwd_params p) {
@@ -301,7 +344,7 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_bwd_ker
 #pragma unroll
     for (int j = 0; j < LPW; ++j) {
       const int r = (wave_s * LPW + j) * RPL + my_lr;
-      const uint32_t piece = (uint32_t)((my_pp ^ v_swizzle(r)) << 4);
+      const uint32_t piece = (uint32_t)((my_pp ^ bwd_swizzle<D>(r)) << 4);
       unsigned char* const dst1 = lds_y1[buf] + (wave_s * LPW + j) * 1024;
       unsigned char* const dst2 = lds_y2[buf] + (wave_s * LPW + j) * 1024;
       global_to_lds_16(row_address(y1b, rows_next[j], y1_rb, piece), dst1);
@@ -320,14 +363,19 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_bwd_ker
   // per-lane LDS offsets of the operand reads
   int off_rows[KSTEPS];  // piece of k-step ks of tile row lane%32, 16-byte read
 #pragma unroll
-  for (int ks = 0; ks < KSTEPS; ++ks) off_rows[ks] = v_tile_offset<D>(col, ks * 2 + hi);
-  int off_tr[DB];  // transposing read: streamed rows 0..3 (+4 for the upper lane half), column word of block db
+  for (int ks = 0; ks < KSTEPS; ++ks) off_rows[ks] = bwd_tile_offset<D>(col, ks * 2 + hi);
+  // transposing read: lane s = 4j + w of a 16-lane group addresses streamed row j (+4 for the upper lane
+  // half), 8-byte word w of the 16 columns of its group; a second read takes the rows 8 further on
+  int off_tr_lo[DB], off_tr_hi[DB];
   {
     const int g = lane >> 4, sl = lane & 15;
     const int key = (g >> 1) * 4 + (sl >> 2);
     const int w = sl & 3;
 #pragma unroll
-    for (int db = 0; db < DB; ++db) off_tr[db] = v_tile_offset<D>(key, db * 4 + (g & 1) * 2 + (w >> 1)) + (w & 1) * 8;
+    for (int db = 0; db < DB; ++db) {
+      off_tr_lo[db] = bwd_tile_offset<D>(key, db * 4 + (g & 1) * 2 + (w >> 1)) + (w & 1) * 8;
+      off_tr_hi[db] = bwd_tile_offset<D>(key + 8, db * 4 + (g & 1) * 2 + (w >> 1)) + (w & 1) * 8;
+    }
   }
 
   f32x16 acc1[DB], acc2[DB];  // dQ^T, or dK^T and dV^T: rows = head dim, column = the lane's stationary row
@@ -371,7 +419,10 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_bwd_ker
       needs_mask = y_hi >= y_end;
     }
 
-    if (wave_in) {
+    // One chunk of one wave as straight-line code (one copy with the mask, one without), so that the
+    // scheduler can mix the soft-max arithmetic of one 32-row half with the MFMAs of the other.
+    auto chunk_body = [&](auto masked_tag) {
+      constexpr bool MASKED = decltype(masked_tag)::value;
       const unsigned char* const y1 = lds_y1[buf];
       const unsigned char* const y2 = lds_y2[buf];
       f32x16 s[2], dp[2];
@@ -394,8 +445,7 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_bwd_ker
       // P' and dS' of the lane's 32 (streamed row, stationary row) pairs, rounded to the input type.
       // Only chunks that touch the diagonal or the end of the sequence pay for the mask.
       vec8 pb[2][2], dsb[2][2];
-      auto softmax_grad = [&](auto masked_tag) {
-        constexpr bool MASKED = decltype(masked_tag)::value;
+      {
 #pragma unroll
         for (int rb = 0; rb < 2; ++rb)
 #pragma unroll
@@ -429,11 +479,7 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_bwd_ker
               dsb[rb][i >> 3][i & 7] = (T)dsv;
             }
           }
-      };
-      if (needs_mask)
-        softmax_grad(std::true_type{});
-      else
-        softmax_grad(std::false_type{});
+      }
 
       // the products that contract over the streamed rows
 #pragma unroll
@@ -443,13 +489,29 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_bwd_ker
 #pragma unroll
           for (int db = 0; db < DB; ++db) {
             const int row_off = (rb * 32 + kk * 16) * D * 2;
-            const vec8 t1 = lds_read_vt<T>(y1, off_tr[db] + row_off, D * 2);
+            const vec8 t1 = bwd_read_tr<T>(y1, off_tr_lo[db] + row_off, off_tr_hi[db] + row_off);
             acc1[db] = Mfma<T>::run(t1, dsb[rb][kk], acc1[db]);
             if (KEY_ST) {
-              const vec8 t2 = lds_read_vt<T>(y2, off_tr[db] + row_off, D * 2);
+              const vec8 t2 = bwd_read_tr<T>(y2, off_tr_lo[db] + row_off, off_tr_hi[db] + row_off);
               acc2[db] = Mfma<T>::run(t2, pb[rb][kk], acc2[db]);
             }
           }
+      // Issue order: every MFMA of the chunk is followed by a share of the vector arithmetic that is
+      // ready by then (none behind the first half's S' and dP' MFMAs, the first half's soft-max behind
+      // the second half's, and so on), instead of all MFMAs first and all arithmetic after.
+      constexpr int N_MFMA = 4 * KSTEPS + 4 * DB * (KEY_ST ? 2 : 1);
+#pragma unroll
+      for (int g = 0; g < N_MFMA; ++g) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);            // one MFMA
+        __builtin_amdgcn_sched_group_barrier(0x002, BWD_VALU_PER, 0); // vector instructions
+        __builtin_amdgcn_sched_group_barrier(0x400, BWD_TRANS_PER, 0);  // exponentials
+      }
+    };
+    if (wave_in) {
+      if (needs_mask)
+        chunk_body(std::true_type{});
+      else
+        chunk_body(std::false_type{});
     }
   }
 

@@ -7,10 +7,10 @@ the closed formulas.  A gradient arriving for the log-sum-exp output is ignored 
 in the reference (src/hyper_attn_triton.py:922-945, src/flash_attn_triton.py:1014-1040): the loss used
 here depends on the attention output only.
 
-Tolerances: norm-wise ||g - ref|| <= tol ||ref|| per gradient tensor, tol = 3e-3 for fp16 and 1e-2 for
+Tolerances: norm-wise ||g - ref|| <= tol ||ref|| per gradient tensor, tol = 3e-3 for fp16 and 5e-3 for
 bf16.  They are wider than the forward's because P and dS are rounded to the input type before the
 products, as the reference does (src/hyper_attn_triton.py:345,367), and dS has twice the relative
-error of P.
+error of P (150 random configurations stay below 1.6e-3 in fp16 and 3.1e-3 in bf16).
 """
 import numpy as np
 import pytest
@@ -22,7 +22,7 @@ pytestmark = pytest.mark.gpu
 
 from _util import _gen, _randn
 
-TOL = {torch.float16: 3e-3, torch.bfloat16: 1e-2}
+TOL = {torch.float16: 3e-3, torch.bfloat16: 5e-3}
 
 
 @pytest.fixture(scope="module")
