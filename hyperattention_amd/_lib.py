@@ -104,6 +104,7 @@ class AttnGrads(ctypes.Structure):
         ("dk_stride_b", ctypes.c_int64), ("dk_stride_h", ctypes.c_int64), ("dk_stride_n", ctypes.c_int64),
         ("dv_stride_b", ctypes.c_int64), ("dv_stride_h", ctypes.c_int64), ("dv_stride_n", ctypes.c_int64),
         ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_int64),
+        ("accumulate", ctypes.c_int),
     ]
 
 

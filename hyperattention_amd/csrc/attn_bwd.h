@@ -38,6 +38,7 @@ struct ha_attn_bwd_params {
   int block_tiles;  // ceil(block_size / 128)
   int sample_size;
   int smooth, idx64;
+  int accumulate;  // add to dq / dk / dv instead of overwriting them
   int q_split;  // sampled-key pass: queries per workgroup
   float scale, scale_log2;
 };

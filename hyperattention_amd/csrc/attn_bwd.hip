@@ -38,6 +38,9 @@ namespace {
 constexpr int WG_THREADS = 256;
 constexpr int ST_ROWS = 128;       // stationary rows per workgroup
 constexpr int YC = 64;             // streamed rows per LDS tile
+#ifndef BWD_INTERLEAVE
+#define BWD_INTERLEAVE 1
+#endif
 #ifndef BWD_VALU_PER
 #define BWD_VALU_PER 5
 #endif
@@ -312,10 +315,12 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_bwd_ker
         for (int g = 0; g < 4; ++g) {
           const int dd = 32 * db + 8 * g + 4 * hi;
           if (!KEY_ST) {
-            *reinterpret_cast<vec4*>(dqb + dd * 2) = zero;
+            if (!p.accumulate) *reinterpret_cast<vec4*>(dqb + dd * 2) = zero;
           } else if (PASS == HA_BWD_DKV_EXACT) {
-            *reinterpret_cast<vec4*>(dkb + dd * 2) = zero;
-            *reinterpret_cast<vec4*>(dvb + dd * 2) = zero;
+            if (!p.accumulate) {
+              *reinterpret_cast<vec4*>(dkb + dd * 2) = zero;
+              *reinterpret_cast<vec4*>(dvb + dd * 2) = zero;
+            }
           } else {
             *reinterpret_cast<f32x4*>(p.dk32 + head_off + dd) = zero32;
             *reinterpret_cast<f32x4*>(p.dv32 + head_off + dd) = zero32;
@@ -499,7 +504,7 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_bwd_ker
       // Issue order: every MFMA of the chunk is followed by a share of the vector arithmetic that is
       // ready by then (none behind the first half's S' and dP' MFMAs, the first half's soft-max behind
       // the second half's, and so on), instead of all MFMAs first and all arithmetic after.
-      constexpr int N_MFMA = 4 * KSTEPS + 4 * DB * (KEY_ST ? 2 : 1);
+      constexpr int N_MFMA = BWD_INTERLEAVE ? 4 * KSTEPS + 4 * DB * (KEY_ST ? 2 : 1) : 0;
 #pragma unroll
       for (int g = 0; g < N_MFMA; ++g) {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);            // one MFMA
@@ -522,10 +527,17 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_bwd_ker
     for (int db = 0; db < DB; ++db)
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
+        vec4* const dst = reinterpret_cast<vec4*>(dqb + (32 * db + 8 * g + 4 * hi) * 2);
         vec4 o;
+        if (p.accumulate) {
+          const vec4 old = *dst;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) o[e] = (T)acc1[db][g * 4 + e];
-        *reinterpret_cast<vec4*>(dqb + (32 * db + 8 * g + 4 * hi) * 2) = o;
+          for (int e = 0; e < 4; ++e) o[e] = (T)(acc1[db][g * 4 + e] + (float)old[e]);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) o[e] = (T)acc1[db][g * 4 + e];
+        }
+        *dst = o;
       }
   } else if (PASS == HA_BWD_DKV_EXACT && st_valid) {
     // complete sums: straight to dk, dv
@@ -535,14 +547,25 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_bwd_ker
     for (int db = 0; db < DB; ++db)
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
+        vec4* const dst_k = reinterpret_cast<vec4*>(dkb + (32 * db + 8 * g + 4 * hi) * 2);
+        vec4* const dst_v = reinterpret_cast<vec4*>(dvb + (32 * db + 8 * g + 4 * hi) * 2);
         vec4 ok_, ov_;
+        if (p.accumulate) {
+          const vec4 old_k = *dst_k, old_v = *dst_v;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          ok_[e] = (T)acc1[db][g * 4 + e];
-          ov_[e] = (T)acc2[db][g * 4 + e];
+          for (int e = 0; e < 4; ++e) {
+            ok_[e] = (T)(acc1[db][g * 4 + e] + (float)old_k[e]);
+            ov_[e] = (T)(acc2[db][g * 4 + e] + (float)old_v[e]);
+          }
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            ok_[e] = (T)acc1[db][g * 4 + e];
+            ov_[e] = (T)acc2[db][g * 4 + e];
+          }
         }
-        *reinterpret_cast<vec4*>(dkb + (32 * db + 8 * g + 4 * hi) * 2) = ok_;
-        *reinterpret_cast<vec4*>(dvb + (32 * db + 8 * g + 4 * hi) * 2) = ov_;
+        *dst_k = ok_;
+        *dst_v = ov_;
       }
   } else if (PASS == HA_BWD_DKV_BLOCK && st_valid) {
     // every key is in exactly one tile of the sorted order: this is the first write of its fp32 row
@@ -626,7 +649,8 @@ template <typename T, int D>
 __global__ __launch_bounds__(256) void ha_bwd_round_kernel(const float* __restrict__ dk32, const float* __restrict__ dv32,
                                                            T* __restrict__ dk, T* __restrict__ dv, int kv_heads, int n_k,
                                                            int64_t dk_sb, int64_t dk_sh, int64_t dk_sn, int64_t dv_sb,
-                                                           int64_t dv_sh, int64_t dv_sn, int64_t total_rows) {
+                                                           int64_t dv_sh, int64_t dv_sn, int64_t total_rows,
+                                                           int accumulate) {
   typedef typename ElemTraits<T>::vec8 vec8;
   constexpr int PR = D / 8;
   const int64_t item = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -647,8 +671,20 @@ __global__ __launch_bounds__(256) void ha_bwd_round_kernel(const float* __restri
     ov[e] = (T)v0[e];
     ov[4 + e] = (T)v1[e];
   }
-  *reinterpret_cast<vec8*>(dk + b * dk_sb + h * dk_sh + row * dk_sn + piece * 8) = ok;
-  *reinterpret_cast<vec8*>(dv + b * dv_sb + h * dv_sh + row * dv_sn + piece * 8) = ov;
+  vec8* const dst_k = reinterpret_cast<vec8*>(dk + b * dk_sb + h * dk_sh + row * dk_sn + piece * 8);
+  vec8* const dst_v = reinterpret_cast<vec8*>(dv + b * dv_sb + h * dv_sh + row * dv_sn + piece * 8);
+  if (accumulate) {
+    const vec8 old_k = *dst_k, old_v = *dst_v;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      ok[e] = (T)(k0[e] + (float)old_k[e]);
+      ok[4 + e] = (T)(k1[e] + (float)old_k[4 + e]);
+      ov[e] = (T)(v0[e] + (float)old_v[e]);
+      ov[4 + e] = (T)(v1[e] + (float)old_v[4 + e]);
+    }
+  }
+  *dst_k = ok;
+  *dst_v = ov;
 }
 
 template <typename T, int D, int PASS, bool CAUSAL>
@@ -724,6 +760,7 @@ void fill_bwd_params(const ha_attn_operands& t, const ha_attn_grads& g, const Wo
   p.batch = (int)t.batch; p.heads = (int)t.heads; p.kv_group = (int)t.kv_group;
   p.n_q = (int)t.n_q; p.n_k = (int)t.n_k;
   p.block_tiles = 1; p.sample_size = 0; p.smooth = 0; p.idx64 = 0;
+  p.accumulate = g.accumulate != 0;
   p.q_split = (int)t.n_q;
   p.scale = t.scale;
   p.scale_log2 = t.scale * LOG2E;
@@ -747,7 +784,7 @@ int launch_round(const ha_attn_operands& t, const ha_attn_grads& g, const Worksp
   const int64_t items = rows * (D / 8);
   hipLaunchKernelGGL((ha_bwd_round_kernel<T, D>), dim3((unsigned)((items + 255) / 256)), dim3(256), 0, stream, w.dk32,
                      w.dv32, (T*)g.dk, (T*)g.dv, (int)kv_heads, (int)t.n_k, g.dk_stride_b, g.dk_stride_h, g.dk_stride_n,
-                     g.dv_stride_b, g.dv_stride_h, g.dv_stride_n, rows);
+                     g.dv_stride_b, g.dv_stride_h, g.dv_stride_n, rows, g.accumulate != 0);
   return ha_launch_status("attention backward: round");
 }
 

@@ -8,10 +8,143 @@ the same HIP operators, following the reference's recursion step by step.
 """
 from __future__ import annotations
 
+import ctypes
+
 import torch
 
-from . import ops
+from . import _lib, ops
 from .angular_lsh import AngularLSH
+
+
+class _CausalRecursionFunc(torch.autograd.Function):
+    """The causal divide-and-conquer (hyper_attention.py:51-96) with its gradient, for lengths that stay
+    even down to the leaves.
+
+    Same arithmetic as the reference's recursion under autograd: exact causal attention on the leaves,
+    one un-masked call per level on (second-half queries, first-half keys/values), merges with the
+    weight rounded to the attention's type (src/attn_utils.py:21-23), and log-sum-exps that carry no
+    gradient (src/hyper_attn_triton.py:922-945).  What differs is the bookkeeping: every call reads and
+    writes strided views of the (batch, heads, n, d) tensors through the C entry points, the merges
+    run in place, and in the backward the gradients of the calls are accumulated by the kernels
+    (`accumulate`), so there are no concatenations, zero-padded slice gradients or gradient additions.
+    """
+
+    @staticmethod
+    def forward(ctx, module, scale, query, key, value):
+        b, h, n, d = query.shape
+        lens = [n]
+        while lens[-1] > module.min_seq_len:
+            lens.append(lens[-1] // 2)
+        levels = len(lens) - 1
+        lib, stream = _lib.lib(), ops._stream(query)
+        f32 = dict(device=query.device, dtype=torch.float32)
+        heads = lambda x, j: x.view(b, h << j, lens[j], x.shape[-1])
+
+        with torch.cuda.device(query.device):
+            # leaves: exact causal attention on every segment of lens[levels] rows
+            o_leaf, lse_leaf = torch.empty_like(query), torch.empty((b, h, n), **f32)
+            t = ops._operands(heads(query, levels), heads(key, levels), heads(value, levels), heads(o_leaf, levels),
+                              lse_leaf.view(b, h << levels, lens[levels]), scale, layout_bnhd=False,
+                              lse_row_stride=lens[levels])
+            _lib.check(lib.ha_flash_attn_fwd(ctypes.byref(t), 1, stream))
+            out, lse = o_leaf.clone(), lse_leaf.clone()
+
+            per_level = []
+            for j in reversed(range(levels)):  # deepest level first, as the recursion returns
+                H, half = h << j, lens[j + 1]
+                q2 = query.view(b, H, 2, half, d)[:, :, 1]
+                k1 = key.view(b, H, 2, half, d)[:, :, 0]
+                v1 = value.view(b, H, 2, half, d)[:, :, 0]
+                o_un, lse_un = torch.empty((b, H, half, d), device=query.device, dtype=query.dtype), torch.empty((b, H, half), **f32)
+                if module.min_seq_len > half:  # hyper_attention.py:109
+                    q_idx = k_idx = None
+                    t = ops._operands(q2, k1, v1, o_un, lse_un, scale, layout_bnhd=False, lse_row_stride=half)
+                    _lib.check(lib.ha_flash_attn_fwd(ctypes.byref(t), 0, stream))
+                else:
+                    num_keys = 1 << module.lsh_num_projs
+                    q_idx = ops.bucket_argsort(module.lsh.hash(q2), num_keys)
+                    k_idx = ops.bucket_argsort(module.lsh.hash(k1), num_keys)
+                    a, keep = ops._block_attn_args(q2, k1, v1, o_un, lse_un, q_idx, k_idx, module.block_size,
+                                                   module.sample_size, scale, module.smooth_block, module.sampled_idx,
+                                                   layout_bnhd=False)
+                    _lib.check(lib.ha_block_attn_fwd(ctypes.byref(a), stream))
+                # merge into the second halves, in place
+                out2 = out.view(b, H, 2, half, d)[:, :, 1]
+                lse2 = lse.view(b, H, 2, half)[:, :, 1]
+                c = torch.sigmoid(lse2 - lse_un).unsqueeze(-1).to(query.dtype)
+                out2.mul_(c).add_((1 - c) * o_un)
+                lse2.sub_((c + torch.finfo(torch.float32).eps).log().squeeze(-1))
+                per_level.append((j, o_un, lse_un, c, q_idx, k_idx))
+
+        tensors = [query, key, value, o_leaf, lse_leaf]
+        layout = []
+        for j, o_un, lse_un, c, q_idx, k_idx in per_level:
+            layout.append((j, q_idx is not None))
+            tensors += [o_un, lse_un, c] + ([q_idx, k_idx] if q_idx is not None else [])
+        ctx.save_for_backward(*tensors)
+        ctx.layout, ctx.lens, ctx.module, ctx.scale = layout, lens, module, scale
+        lse = lse.unsqueeze(-1)
+        ctx.mark_non_differentiable(lse)
+        return out, lse
+
+    @staticmethod
+    def backward(ctx, dout, dlse=None):
+        saved = list(ctx.saved_tensors)
+        query, key, value, o_leaf, lse_leaf = saved[:5]
+        rest = saved[5:]
+        module, scale, lens = ctx.module, ctx.scale, ctx.lens
+        b, h, n, d = query.shape
+        levels = len(lens) - 1
+        lib, stream = _lib.lib(), ops._stream(query)
+        heads = lambda x, j: x.view(b, h << j, lens[j], x.shape[-1])
+
+        per_level = {}
+        for j, hashed in ctx.layout:
+            o_un, lse_un, c = rest[:3]
+            q_idx, k_idx = (rest[3], rest[4]) if hashed else (None, None)
+            rest = rest[5:] if hashed else rest[3:]
+            per_level[j] = (o_un, lse_un, c, q_idx, k_idx)
+
+        with torch.cuda.device(query.device):
+            # the gradient of the output splits at every merge, from the top level down: (1 - c) of it
+            # goes to the un-masked call of the level, c of it further down
+            do_cur = dout.contiguous().clone()
+            do_un = {}
+            for j in range(levels):
+                H, half = h << j, lens[j + 1]
+                c = per_level[j][2]
+                do2 = do_cur.view(b, H, 2, half, d)[:, :, 1]
+                do_un[j] = (1 - c) * do2
+                do2.mul_(c)
+
+            dq, dk, dv = torch.empty_like(query), torch.empty_like(key), torch.empty_like(value)
+            # leaves first: they write every row of dq, dk, dv; the levels then add to their views
+            t = ops._operands(heads(query, levels), heads(key, levels), heads(value, levels), heads(o_leaf, levels),
+                              lse_leaf.view(b, h << levels, lens[levels]), scale, layout_bnhd=False,
+                              lse_row_stride=lens[levels])
+            g, ws = ops._attn_grads(t, heads(do_cur, levels), heads(dq, levels), heads(dk, levels), heads(dv, levels),
+                                    layout_bnhd=False)
+            _lib.check(lib.ha_flash_attn_bwd(ctypes.byref(t), 1, ctypes.byref(g), stream))
+            for j in range(levels):
+                H, half = h << j, lens[j + 1]
+                o_un, lse_un, c, q_idx, k_idx = per_level[j]
+                q2 = query.view(b, H, 2, half, d)[:, :, 1]
+                k1 = key.view(b, H, 2, half, d)[:, :, 0]
+                v1 = value.view(b, H, 2, half, d)[:, :, 0]
+                dq2 = dq.view(b, H, 2, half, d)[:, :, 1]
+                dk1 = dk.view(b, H, 2, half, d)[:, :, 0]
+                dv1 = dv.view(b, H, 2, half, d)[:, :, 0]
+                if q_idx is None:
+                    t = ops._operands(q2, k1, v1, o_un, lse_un, scale, layout_bnhd=False, lse_row_stride=half)
+                    g, ws = ops._attn_grads(t, do_un[j], dq2, dk1, dv1, layout_bnhd=False, accumulate=True)
+                    _lib.check(lib.ha_flash_attn_bwd(ctypes.byref(t), 0, ctypes.byref(g), stream))
+                else:
+                    a, keep = ops._block_attn_args(q2, k1, v1, o_un, lse_un, q_idx, k_idx, module.block_size,
+                                                   module.sample_size, scale, module.smooth_block, module.sampled_idx,
+                                                   layout_bnhd=False)
+                    g, ws = ops._attn_grads(a.t, do_un[j], dq2, dk1, dv1, layout_bnhd=False, accumulate=True)
+                    _lib.check(lib.ha_block_attn_bwd(ctypes.byref(a), ctypes.byref(g), stream))
+        return None, None, dq, dk, dv
 
 
 class HyperAttention(torch.nn.Module):
@@ -91,7 +224,13 @@ class HyperAttention(torch.nn.Module):
                 # wants as many k/v heads as q heads (hyper_attention.py:43,67-68)
                 group = query.shape[1] // key.shape[1]
                 key, value = key.repeat_interleave(group, dim=1), value.repeat_interleave(group, dim=1)
-            attn, lse = self._forward_composed(query.contiguous(), key.contiguous(), value.contiguous(), scale, causal)
+            query, key, value = query.contiguous(), key.contiguous(), value.contiguous()
+            if (causal is not False and n_key > self.min_seq_len and ops._wants_grad(query, key, value)
+                    and ops.forward_plan_supported(n_key, self.min_seq_len, True, 8)):
+                # every level has an even length: the recursion and its gradient on views, in place
+                attn, lse = _CausalRecursionFunc.apply(self, scale, query, key, value)
+            else:
+                attn, lse = self._forward_composed(query, key, value, scale, causal)
 
         if not return_lse:
             return attn

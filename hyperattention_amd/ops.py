@@ -137,15 +137,21 @@ def padded_head_dim(d):
 
 
 def _block_attn_args(q, k, v, o, lse, q_sort_idx, k_sort_idx, block_size, sample_size, softmax_scale,
-                     smooth_block, sampled_idx, accumulate=False):
-    """BlockAttnArgs for (b,n,h,d) tensors; the second result keeps the device copy of sampled_idx alive."""
-    batch, seqlen_q, nheads, _ = q.shape
+                     smooth_block, sampled_idx, accumulate=False, layout_bnhd=True):
+    """BlockAttnArgs for (b,n,h,d) tensors with (b,n,h) index tensors [layout_bnhd] or (b,h,n,d) tensors
+    with (b,h,n) index tensors; the second result keeps the device copy of sampled_idx alive."""
+    if layout_bnhd:
+        batch, seqlen_q, nheads, _ = q.shape
+        sn, sh = 1, 2
+    else:
+        batch, nheads, seqlen_q, _ = q.shape
+        sn, sh = 2, 1
     a = BlockAttnArgs()
-    a.t = _operands(q, k, v, o, lse, softmax_scale, layout_bnhd=True, lse_row_stride=seqlen_q)
+    a.t = _operands(q, k, v, o, lse, softmax_scale, layout_bnhd=layout_bnhd, lse_row_stride=seqlen_q)
     a.q_idx, a.k_idx = q_sort_idx.data_ptr(), k_sort_idx.data_ptr()
     a.idx_type = _idx_code(q_sort_idx)
-    a.q_idx_stride_b, a.q_idx_stride_h, a.q_idx_stride_n = q_sort_idx.stride(0), q_sort_idx.stride(2), q_sort_idx.stride(1)
-    a.k_idx_stride_b, a.k_idx_stride_h, a.k_idx_stride_n = k_sort_idx.stride(0), k_sort_idx.stride(2), k_sort_idx.stride(1)
+    a.q_idx_stride_b, a.q_idx_stride_h, a.q_idx_stride_n = q_sort_idx.stride(0), q_sort_idx.stride(sh), q_sort_idx.stride(sn)
+    a.k_idx_stride_b, a.k_idx_stride_h, a.k_idx_stride_n = k_sort_idx.stride(0), k_sort_idx.stride(sh), k_sort_idx.stride(sn)
     keep = None
     a.sampled_stride_b = a.sampled_stride_h = 0
     if sampled_idx is not None:
@@ -278,14 +284,16 @@ def _wants_grad(*tensors):
     return torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in tensors)
 
 
-def _attn_grads(t, dout, dq, dk, dv):
-    """AttnGrads for (b,n,h,d) gradient tensors plus the workspace the C side asks for."""
+def _attn_grads(t, dout, dq, dk, dv, layout_bnhd=True, accumulate=False):
+    """AttnGrads for (b,n,h,d) [layout_bnhd] or (b,h,n,d) gradient tensors plus the workspace the C side asks for."""
+    sn, sh = (1, 2) if layout_bnhd else (2, 1)
     g = AttnGrads()
     g.dout, g.dq, g.dk, g.dv = dout.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr()
-    g.do_stride_b, g.do_stride_h, g.do_stride_n = dout.stride(0), dout.stride(2), dout.stride(1)
-    g.dq_stride_b, g.dq_stride_h, g.dq_stride_n = dq.stride(0), dq.stride(2), dq.stride(1)
-    g.dk_stride_b, g.dk_stride_h, g.dk_stride_n = dk.stride(0), dk.stride(2), dk.stride(1)
-    g.dv_stride_b, g.dv_stride_h, g.dv_stride_n = dv.stride(0), dv.stride(2), dv.stride(1)
+    g.do_stride_b, g.do_stride_h, g.do_stride_n = dout.stride(0), dout.stride(sh), dout.stride(sn)
+    g.dq_stride_b, g.dq_stride_h, g.dq_stride_n = dq.stride(0), dq.stride(sh), dq.stride(sn)
+    g.dk_stride_b, g.dk_stride_h, g.dk_stride_n = dk.stride(0), dk.stride(sh), dk.stride(sn)
+    g.dv_stride_b, g.dv_stride_h, g.dv_stride_n = dv.stride(0), dv.stride(sh), dv.stride(sn)
+    g.accumulate = int(bool(accumulate))
     nbytes = _lib.lib().ha_attn_bwd_workspace_bytes(ctypes.byref(t))
     if nbytes <= 0:
         _lib.check(int(nbytes) if nbytes < 0 else -3)

@@ -153,7 +153,9 @@ int ha_flash_attn_fwd(const ha_attn_operands* t, int causal, void* stream);
  * holding the forward's results (read only here); a gradient for `lse` is not taken, as in the
  * reference (HyperAttnFunc.backward / FlashAttnFunc.backward ignore it).
  * dq: like q; dk, dv: like k, v, i.e. (batch, heads / kv_group, n_k, d): with grouped queries every
- * query head of a group adds into its key head.  All in dtype, last dim contiguous, written in full.
+ * query head of a group adds into its key head.  All in dtype, last dim contiguous, written in full
+ * (or, with accumulate, added to in full: a caller that differentiates several attention calls on
+ * views of the same tensors, like the causal recursion, sums their gradients without extra passes).
  * Only whole heads: segs == 1 and zero segment offsets.
  * workspace: ha_attn_bwd_workspace_bytes(t) bytes, 256-byte aligned (row statistics and fp32
  * accumulators of dk, dv; cleared by the call).
@@ -169,6 +171,7 @@ typedef struct {
   int64_t dv_stride_b, dv_stride_h, dv_stride_n;
   void* workspace;
   int64_t workspace_bytes;
+  int accumulate;    /* != 0: dq, dk, dv hold gradients already and the results are added to them   */
 } ha_attn_grads;
 
 int64_t ha_attn_bwd_workspace_bytes(const ha_attn_operands* t);
