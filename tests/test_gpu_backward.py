@@ -211,20 +211,30 @@ def test_backward_grouped_query_heads_through_the_c_abi(ha, kind):
 
 
 # ------------------------------------------------------------------------------- the module
-@pytest.mark.parametrize("causal,n,min_seq_len", [(False, 1024, 256), (True, 1024, 256), (True, 1025, 600)])
-def test_module_backward(ha, causal, n, min_seq_len):
+@pytest.mark.parametrize("causal,n,min_seq_len,block,sample,smooth,kv_heads", [
+    (False, 1024, 256, 128, 128, False, 2),
+    (True, 1024, 256, 128, 128, False, 2),    # two hashed levels, on views with accumulated gradients
+    (True, 1025, 600, 128, 128, False, 2),    # odd length: the operator-by-operator recursion, padded
+    (True, 2048, 512, 256, 256, True, 2),     # smoothed blocks
+    (True, 1024, 600, 128, 128, False, 2),    # the off-diagonal call is exact (min_seq_len > n/2)
+    (True, 2048, 256, 128, 128, False, 1),    # three levels; two query heads on one key/value head
+])
+def test_module_backward(ha, causal, n, min_seq_len, block, sample, smooth, kv_heads):
     # the module under autograd: operators with their own backward, merges as tensor arithmetic;
     # log-sum-exps carry no gradient (detach_lse), as the reference's operators return none for them
     dtype, b, h, d = torch.float16, 1, 2, 64
     q = _randn((b, h, n, d), 51, dtype)
-    k = _randn((b, h, n, d), 52, dtype)
-    v = _randn((b, h, n, d), 53, dtype)
+    k = _randn((b, kv_heads, n, d), 52, dtype)
+    v = _randn((b, kv_heads, n, d), 53, dtype)
     do = _randn((b, h, n, d), 54, dtype)
-    m = ha.HyperAttention(input_dim=d, block_size=128, sample_size=128, min_seq_len=min_seq_len, rng=_gen(55))
+    m = ha.HyperAttention(input_dim=d, block_size=block, sample_size=sample, min_seq_len=min_seq_len, smooth_block=smooth,
+                          rng=_gen(55))
     m = m.to(device="cuda", dtype=dtype)
     proj = m.lsh.proj_dir[0, 0].cpu()
-    ref = _oracle_grads(lambda a, b_, c: O.hyper_forward(a, b_, c, proj, causal=causal, block_size=128, sample_size=128,
-                                                         min_seq_len=min_seq_len, detach_lse=True), q, k, v, do)
+    expand = lambda x: x.repeat_interleave(h // kv_heads, dim=1)
+    ref = _oracle_grads(lambda a, b_, c: O.hyper_forward(a, expand(b_), expand(c), proj, causal=causal, block_size=block,
+                                                         sample_size=sample, min_seq_len=min_seq_len, smooth_block=smooth,
+                                                         detach_lse=True), q, k, v, do)
     qg, kg, vg = (x.cuda().requires_grad_() for x in (q, k, v))
     out = m(qg, kg, vg, causal=causal)
     with torch.no_grad():
@@ -235,3 +245,20 @@ def test_module_backward(ha, causal, n, min_seq_len):
     torch.cuda.synchronize()
     for got, want, name in zip((qg.grad, kg.grad, vg.grad), ref, ("dq", "dk", "dv")):
         _check(got, want, f"module {name}", dtype)
+
+
+def test_module_backward_twice_and_retain_graph(ha):
+    # the backward neither consumes nor disturbs what it saved: two passes over one graph agree
+    dtype, b, h, n, d = torch.bfloat16, 1, 2, 1024, 64
+    q, k, v, do = (_randn((b, h, n, d), 70 + i, dtype).cuda() for i in range(4))
+    m = ha.HyperAttention(input_dim=d, block_size=128, sample_size=128, min_seq_len=256, rng=_gen(75)).to(device="cuda", dtype=dtype)
+    qg, kg, vg = (x.clone().requires_grad_() for x in (q, k, v))
+    out = m(qg, kg, vg, causal=True)
+    out.backward(do, retain_graph=True)
+    first = [x.grad.clone() for x in (qg, kg, vg)]
+    for x in (qg, kg, vg):
+        x.grad = None
+    out.backward(do)
+    for a, b_ in zip(first, (qg.grad, kg.grad, vg.grad)):
+        # the sampled keys' sums are accumulated with atomics, in an order that can differ between runs
+        assert ((a.double() - b_.double()).norm() / a.double().norm()).item() < 1e-3
