@@ -106,28 +106,36 @@ class _CausalRecursionFunc(torch.autograd.Function):
             per_level[j] = (o_un, lse_un, c, q_idx, k_idx)
 
         with torch.cuda.device(query.device):
-            # the gradient of the output splits at every merge, from the top level down: (1 - c) of it
-            # goes to the un-masked call of the level, c of it further down
-            do_cur = dout.contiguous().clone()
-            do_un = {}
+            # The gradient of the output splits at every merge, from the top level down: (1 - c) of it goes
+            # to the un-masked call of the level, c of it further down.  A call's gradients are linear in
+            # the output gradient it is given, and that enters only through P = exp(s - lse): weighting a
+            # row's output gradient by w equals giving the call the log-sum-exp lse - log(w) for that row
+            # (w = 0: lse = +inf, P = 0).  So every call gets the output gradient as it is and a shifted
+            # copy of its small log-sum-exp array, and no weighted copy of the gradient is ever made.
+            dout = dout.contiguous()
+            log_w = torch.zeros((b, h, n), device=query.device, dtype=torch.float32)
+            lse_shifted = {}
             for j in range(levels):
                 H, half = h << j, lens[j + 1]
-                c = per_level[j][2]
-                do2 = do_cur.view(b, H, 2, half, d)[:, :, 1]
-                do_un[j] = (1 - c) * do2
-                do2.mul_(c)
+                lse_un, c = per_level[j][1], per_level[j][2].squeeze(-1).float()
+                log_w2 = log_w.view(b, H, 2, half)[:, :, 1]
+                lse_shifted[j] = lse_un - torch.log1p(-c) - log_w2
+                log_w2.add_(torch.log(c))
+            lse_leaf = lse_leaf - log_w
 
             dq, dk, dv = torch.empty_like(query), torch.empty_like(key), torch.empty_like(value)
             # leaves first: they write every row of dq, dk, dv; the levels then add to their views
             t = ops._operands(heads(query, levels), heads(key, levels), heads(value, levels), heads(o_leaf, levels),
                               lse_leaf.view(b, h << levels, lens[levels]), scale, layout_bnhd=False,
                               lse_row_stride=lens[levels])
-            g, ws = ops._attn_grads(t, heads(do_cur, levels), heads(dq, levels), heads(dk, levels), heads(dv, levels),
+            g, ws = ops._attn_grads(t, heads(dout, levels), heads(dq, levels), heads(dk, levels), heads(dv, levels),
                                     layout_bnhd=False)
             _lib.check(lib.ha_flash_attn_bwd(ctypes.byref(t), 1, ctypes.byref(g), stream))
             for j in range(levels):
                 H, half = h << j, lens[j + 1]
-                o_un, lse_un, c, q_idx, k_idx = per_level[j]
+                o_un, _, _, q_idx, k_idx = per_level[j]
+                lse_un = lse_shifted[j]
+                do2 = dout.view(b, H, 2, half, d)[:, :, 1]
                 q2 = query.view(b, H, 2, half, d)[:, :, 1]
                 k1 = key.view(b, H, 2, half, d)[:, :, 0]
                 v1 = value.view(b, H, 2, half, d)[:, :, 0]
@@ -136,13 +144,13 @@ class _CausalRecursionFunc(torch.autograd.Function):
                 dv1 = dv.view(b, H, 2, half, d)[:, :, 0]
                 if q_idx is None:
                     t = ops._operands(q2, k1, v1, o_un, lse_un, scale, layout_bnhd=False, lse_row_stride=half)
-                    g, ws = ops._attn_grads(t, do_un[j], dq2, dk1, dv1, layout_bnhd=False, accumulate=True)
+                    g, ws = ops._attn_grads(t, do2, dq2, dk1, dv1, layout_bnhd=False, accumulate=True)
                     _lib.check(lib.ha_flash_attn_bwd(ctypes.byref(t), 0, ctypes.byref(g), stream))
                 else:
                     a, keep = ops._block_attn_args(q2, k1, v1, o_un, lse_un, q_idx, k_idx, module.block_size,
                                                    module.sample_size, scale, module.smooth_block, module.sampled_idx,
                                                    layout_bnhd=False)
-                    g, ws = ops._attn_grads(a.t, do_un[j], dq2, dk1, dv1, layout_bnhd=False, accumulate=True)
+                    g, ws = ops._attn_grads(a.t, do2, dq2, dk1, dv1, layout_bnhd=False, accumulate=True)
                     _lib.check(lib.ha_block_attn_bwd(ctypes.byref(a), ctypes.byref(g), stream))
         return None, None, dq, dk, dv
 
