@@ -148,7 +148,7 @@ def _declare(lib):
     lib.ha_flash_attn_fwd.restype = ci
     lib.ha_flash_attn_fwd.argtypes = [ctypes.POINTER(AttnOperands), ci, vp]
     lib.ha_attn_bwd_workspace_bytes.restype = i64
-    lib.ha_attn_bwd_workspace_bytes.argtypes = [ctypes.POINTER(AttnOperands)]
+    lib.ha_attn_bwd_workspace_bytes.argtypes = [ctypes.POINTER(AttnOperands), i64]
     lib.ha_block_attn_bwd.restype = ci
     lib.ha_block_attn_bwd.argtypes = [ctypes.POINTER(BlockAttnArgs), ctypes.POINTER(AttnGrads), vp]
     lib.ha_flash_attn_bwd.restype = ci

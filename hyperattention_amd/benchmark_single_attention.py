@@ -26,6 +26,7 @@ def get_arguments(argv=None):
     parser.add_argument("--smooth_block", action="store_true")
     parser.add_argument("--mode", type=str, default="fwd", choices=["fwd", "bwd", "fwd+bwd"])
     parser.add_argument("--attn_method", type=str, default="flash", choices=["flash", "flash-cuda", "hyper"])
+    parser.add_argument("--min_log2_seq", type=int, default=10, help="first sequence length of the sweep (2^k)")
     parser.add_argument("--max_log2_seq", type=int, default=17, help="last sequence length of the sweep (2^k)")
     parser.add_argument("--rep", type=int, default=100)
     return parser.parse_args(argv)
@@ -78,7 +79,7 @@ def main(argv=None):
     if args.attn_method == "flash-cuda":
         sys.exit("flash-cuda is a CUDA package; use --attn_method flash for this library's exact attention")
 
-    seq_lens = [2 ** i for i in range(10, args.max_log2_seq + 1)]
+    seq_lens = [2 ** i for i in range(args.min_log2_seq, args.max_log2_seq + 1)]
     batch_size, head_size, dim = 1, 24, 64
     print(f"mode: {args.mode}, attn_method: {args.attn_method}, batch_size: {batch_size}, head_size: {head_size}, dim: {dim}")
     causal = not args.no_causal

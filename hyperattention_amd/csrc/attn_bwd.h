@@ -19,8 +19,8 @@ struct ha_attn_bwd_params {
   const float* lse;    // forward log-sum-exp (natural log), (batch, heads, n_q) by lse_sb / lse_sh
   const float* delta;  // sum_c dO*O per query, fp32, contiguous (batch, heads, n_q)
   void* dq;
-  void *dk, *dv;       // written directly by the exact pass
-  float *dk32, *dv32;  // fp32 (batch, heads / kv_group, n_k, d) contiguous: the gathered passes' sums
+  void *dk, *dv;       // written directly by the exact and the block passes
+  float *dk32, *dv32;  // fp32 (batch, heads / kv_group, sample_size, d): sums of the sampled keys, by slot
   int64_t q_sb, q_sh, q_sn;
   int64_t k_sb, k_sh, k_sn;
   int64_t v_sb, v_sh, v_sn;

@@ -23,9 +23,9 @@
 // see all keys of a query in one workgroup and store dQ.  The dK/dV pass of exact attention sees all
 // queries of a key (of every query head of the key head's group, streamed one head after the other)
 // and stores dK, dV.  With sorted blocks a key gets one contribution from its block (complete in one
-// workgroup: stored as fp32) and, if it is in the sample list, one from every query: those are
-// computed per range of queries and added to the fp32 rows with atomics; a last kernel rounds the
-// fp32 rows to the output type.
+// workgroup: stored like the exact pass's) and, if it is in the sample list, one from every query:
+// those are computed per range of queries and summed with atomics in small fp32 rows, one per slot of
+// the sample list, which a last kernel adds to the keys' rows of dK, dV.
 #include "ha_common.h"
 #include "attn_tiles.h"
 #include "attn_fwd.h"
@@ -304,11 +304,9 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_bwd_ker
     // nothing attends (or is attended by) this tile: its gradient is zero
     if (PASS != HA_BWD_DKV_SAMPLED && st_valid) {
       const vec4 zero = {(T)0.f, (T)0.f, (T)0.f, (T)0.f};
-      const f32x4 zero32 = {0.f, 0.f, 0.f, 0.f};
       unsigned char* const dqb = (unsigned char*)((T*)p.dq + b * p.dq_sb + h0 * p.dq_sh) + (int64_t)st_row * p.dq_sn * 2;
       unsigned char* const dkb = (unsigned char*)((T*)p.dk + b * p.dk_sb + hk * p.dk_sh) + (int64_t)st_row * p.dk_sn * 2;
       unsigned char* const dvb = (unsigned char*)((T*)p.dv + b * p.dv_sb + hk * p.dv_sh) + (int64_t)st_row * p.dv_sn * 2;
-      const int64_t head_off = ((int64_t)(b * kv_heads + hk) * p.n_k + st_row) * D;
 #pragma unroll
       for (int db = 0; db < DB; ++db)
 #pragma unroll
@@ -316,14 +314,9 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_bwd_ker
           const int dd = 32 * db + 8 * g + 4 * hi;
           if (!KEY_ST) {
             if (!p.accumulate) *reinterpret_cast<vec4*>(dqb + dd * 2) = zero;
-          } else if (PASS == HA_BWD_DKV_EXACT) {
-            if (!p.accumulate) {
-              *reinterpret_cast<vec4*>(dkb + dd * 2) = zero;
-              *reinterpret_cast<vec4*>(dvb + dd * 2) = zero;
-            }
-          } else {
-            *reinterpret_cast<f32x4*>(p.dk32 + head_off + dd) = zero32;
-            *reinterpret_cast<f32x4*>(p.dv32 + head_off + dd) = zero32;
+          } else if (!p.accumulate) {
+            *reinterpret_cast<vec4*>(dkb + dd * 2) = zero;
+            *reinterpret_cast<vec4*>(dvb + dd * 2) = zero;
           }
         }
     }
@@ -539,8 +532,8 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_bwd_ker
         }
         *dst = o;
       }
-  } else if (PASS == HA_BWD_DKV_EXACT && st_valid) {
-    // complete sums: straight to dk, dv
+  } else if ((PASS == HA_BWD_DKV_EXACT || PASS == HA_BWD_DKV_BLOCK) && st_valid) {
+    // complete sums (of the blocks: every key is in exactly one tile of the sorted order): straight to dk, dv
     unsigned char* const dkb = (unsigned char*)((T*)p.dk + b * p.dk_sb + hk * p.dk_sh) + (int64_t)st_row * p.dk_sn * 2;
     unsigned char* const dvb = (unsigned char*)((T*)p.dv + b * p.dv_sb + hk * p.dv_sh) + (int64_t)st_row * p.dv_sn * 2;
 #pragma unroll
@@ -567,30 +560,16 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_bwd_ker
         *dst_k = ok_;
         *dst_v = ov_;
       }
-  } else if (PASS == HA_BWD_DKV_BLOCK && st_valid) {
-    // every key is in exactly one tile of the sorted order: this is the first write of its fp32 row
-    const int64_t head_off = ((int64_t)(b * kv_heads + hk) * p.n_k + st_row) * D;
-    float* const dk_row = p.dk32 + head_off;
-    float* const dv_row = p.dv32 + head_off;
-#pragma unroll
-    for (int db = 0; db < DB; ++db)
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const int dd = 32 * db + 8 * g + 4 * hi;
-        *reinterpret_cast<f32x4*>(dk_row + dd) =
-            f32x4{acc1[db][g * 4], acc1[db][g * 4 + 1], acc1[db][g * 4 + 2], acc1[db][g * 4 + 3]};
-        *reinterpret_cast<f32x4*>(dv_row + dd) =
-            f32x4{acc2[db][g * 4], acc2[db][g * 4 + 1], acc2[db][g * 4 + 2], acc2[db][g * 4 + 3]};
-      }
   }
   if (PASS == HA_BWD_DKV_SAMPLED) {
-    // Sampled keys: partial sums over one range of queries of one query head, added on top of the rows
-    // with atomics.  Each wave turns its 32 x D results around in LDS (its quarter of the tile buffers,
-    // free once every wave has left the loop) so that one atomic instruction covers 64 consecutive floats
-    // of one row instead of one float of each of 64 rows.
+    // Sampled keys: partial sums over one range of queries of one query head, added with atomics to the
+    // fp32 row of the key's SLOT in the sample list (batch, kv_heads, sample_size, D).  Each wave turns its
+    // 32 x D results around in LDS (its quarter of the tile buffers, free once every wave has left the
+    // loop) so that one atomic instruction covers 64 consecutive floats of one row instead of one float of
+    // each of 64 rows.
     __syncthreads();
     float* const turn = reinterpret_cast<float*>(wave_s < 2 ? lds_y1[wave_s] : lds_y2[wave_s - 2]);
-    const int64_t head_base = (int64_t)(b * kv_heads + hk) * p.n_k * D;
+    const int64_t head_base = (int64_t)(b * kv_heads + hk) * p.sample_size * D;
 #pragma unroll
     for (int which = 0; which < 2; ++which) {
       float* const dst = (which == 0 ? p.dk32 : p.dv32) + head_base;
@@ -604,13 +583,12 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_bwd_ker
           *reinterpret_cast<f32x4*>(turn + col * D + piece * 4) = f32x4{a[g * 4], a[g * 4 + 1], a[g * 4 + 2], a[g * 4 + 3]};
         }
       for (int r = 0; r < 32; ++r) {
-        const int row = __shfl(st_row, r);
-        const bool valid = __shfl((int)st_valid, r) != 0;
+        const int slot = tile * ST_ROWS + wave_s * 32 + r;  // < sample_size: a multiple of 128
 #pragma unroll
         for (int part = 0; part < D / 64; ++part) {
           const int dd = part * 64 + lane;
           const float val = turn[r * D + (((dd >> 2) ^ (r & 15)) << 2) + (dd & 3)];
-          if (valid) unsafeAtomicAdd(dst + (int64_t)row * D + dd, val);
+          unsafeAtomicAdd(dst + (int64_t)slot * D + dd, val);
         }
       }
     }
@@ -644,44 +622,61 @@ __global__ __launch_bounds__(256) void ha_bwd_delta_kernel(const T* __restrict__
   if (grow < total_rows && piece == 0) delta[grow] = acc;
 }
 
-// fp32 accumulators (batch, kv_heads, n_k, D) -> dk, dv in the output type, 8 elements per lane
+__global__ __launch_bounds__(256) void ha_bwd_zero_kernel(f32x4* __restrict__ buf, int64_t n4) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n4) buf[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+}
+
+// Sums of the sampled keys (fp32, one row per slot of the sample list) added to the rows of dk, dv, 8
+// elements per lane.  A row that is listed several times is handled by its first slot alone, which adds
+// the sums of all of them: no two lanes write the same row, whatever the list holds.
 template <typename T, int D>
-__global__ __launch_bounds__(256) void ha_bwd_round_kernel(const float* __restrict__ dk32, const float* __restrict__ dv32,
-                                                           T* __restrict__ dk, T* __restrict__ dv, int kv_heads, int n_k,
-                                                           int64_t dk_sb, int64_t dk_sh, int64_t dk_sn, int64_t dv_sb,
-                                                           int64_t dv_sh, int64_t dv_sn, int64_t total_rows,
-                                                           int accumulate) {
+__global__ __launch_bounds__(256) void ha_bwd_add_samples_kernel(const float* __restrict__ sk32, const float* __restrict__ sv32,
+                                                                 T* __restrict__ dk, T* __restrict__ dv,
+                                                                 const void* __restrict__ sampled_idx, int idx64,
+                                                                 int64_t si_sb, int64_t si_sh, int kv_heads, int sample_size,
+                                                                 int64_t dk_sb, int64_t dk_sh, int64_t dk_sn, int64_t dv_sb,
+                                                                 int64_t dv_sh, int64_t dv_sn, int64_t total_slots) {
   typedef typename ElemTraits<T>::vec8 vec8;
   constexpr int PR = D / 8;
   const int64_t item = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  const int64_t grow = item / PR;
+  const int64_t gslot = item / PR;
   const int piece = (int)(item % PR);
-  if (grow >= total_rows) return;
-  const int64_t bh = grow / n_k;
-  const int row = (int)(grow - bh * n_k);
+  if (gslot >= total_slots) return;
+  const int64_t bh = gslot / sample_size;
+  const int slot = (int)(gslot - bh * sample_size);
   const int64_t b = bh / kv_heads, h = bh - b * kv_heads;
-  const f32x4* const sk = reinterpret_cast<const f32x4*>(dk32 + grow * D + piece * 8);
-  const f32x4* const sv = reinterpret_cast<const f32x4*>(dv32 + grow * D + piece * 8);
-  const f32x4 k0 = sk[0], k1 = sk[1], v0 = sv[0], v1 = sv[1];
-  vec8 ok, ov;
+  int row = slot;
+  float sum_k[8], sum_v[8];
+  const float* const bk = sk32 + (bh * sample_size) * D + piece * 8;
+  const float* const bv = sv32 + (bh * sample_size) * D + piece * 8;
+  auto add_slot = [&](int s2) {
 #pragma unroll
-  for (int e = 0; e < 4; ++e) {
-    ok[e] = (T)k0[e];
-    ok[4 + e] = (T)k1[e];
-    ov[e] = (T)v0[e];
-    ov[4 + e] = (T)v1[e];
+    for (int e = 0; e < 8; ++e) {
+      sum_k[e] += bk[(int64_t)s2 * D + e];
+      sum_v[e] += bv[(int64_t)s2 * D + e];
+    }
+  };
+#pragma unroll
+  for (int e = 0; e < 8; ++e) sum_k[e] = sum_v[e] = 0.f;
+  if (sampled_idx) {
+    const int64_t list = b * si_sb + h * si_sh;
+    row = ha_load_idx(sampled_idx, list + slot, idx64);
+    for (int s2 = 0; s2 < slot; ++s2)
+      if (ha_load_idx(sampled_idx, list + s2, idx64) == row) return;  // an earlier slot owns this row
+    add_slot(slot);
+    for (int s2 = slot + 1; s2 < sample_size; ++s2)
+      if (ha_load_idx(sampled_idx, list + s2, idx64) == row) add_slot(s2);
+  } else {
+    add_slot(slot);
   }
   vec8* const dst_k = reinterpret_cast<vec8*>(dk + b * dk_sb + h * dk_sh + row * dk_sn + piece * 8);
   vec8* const dst_v = reinterpret_cast<vec8*>(dv + b * dv_sb + h * dv_sh + row * dv_sn + piece * 8);
-  if (accumulate) {
-    const vec8 old_k = *dst_k, old_v = *dst_v;
+  vec8 ok = *dst_k, ov = *dst_v;
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      ok[e] = (T)(k0[e] + (float)old_k[e]);
-      ok[4 + e] = (T)(k1[e] + (float)old_k[4 + e]);
-      ov[e] = (T)(v0[e] + (float)old_v[e]);
-      ov[4 + e] = (T)(v1[e] + (float)old_v[4 + e]);
-    }
+  for (int e = 0; e < 8; ++e) {
+    ok[e] = (T)((float)ok[e] + sum_k[e]);
+    ov[e] = (T)((float)ov[e] + sum_v[e]);
   }
   *dst_k = ok;
   *dst_v = ov;
@@ -699,16 +694,16 @@ inline int64_t align256(int64_t v) { return (v + 255) & ~(int64_t)255; }
 
 struct Workspace {
   float* delta;
-  float* dk32;
+  float* dk32;  // sums of the sampled keys, (batch, kv_heads, sample_size, d) fp32
   float* dv32;
   int64_t acc_floats;  // per accumulator
   int64_t bytes;
 };
 
-Workspace carve(const ha_attn_operands& t, void* base) {
+Workspace carve(const ha_attn_operands& t, int64_t sample_size, void* base) {
   Workspace w;
   const int64_t delta_bytes = align256(t.batch * t.heads * t.n_q * 4);
-  w.acc_floats = t.batch * (t.heads / t.kv_group) * t.n_k * t.d;
+  w.acc_floats = t.batch * (t.heads / t.kv_group) * sample_size * t.d;
   const int64_t acc_bytes = align256(w.acc_floats * 4);
   w.delta = (float*)base;
   w.dk32 = (float*)((char*)base + delta_bytes);
@@ -717,7 +712,7 @@ Workspace carve(const ha_attn_operands& t, void* base) {
   return w;
 }
 
-int check_grads(const ha_attn_operands& t, const ha_attn_grads& g, const char* who) {
+int check_grads(const ha_attn_operands& t, int64_t sample_size, const ha_attn_grads& g, const char* who) {
   HA_REQUIRE(g.dout && g.dq && g.dk && g.dv, HA_ERR_NULL, "%s: null gradient pointer", who);
   HA_REQUIRE(t.segs == 1 && t.q_seg_offset == 0 && t.k_seg_offset == 0, HA_ERR_UNSUPPORTED,
              "%s: the backward takes whole heads (segs == 1, no segment offsets)", who);
@@ -735,7 +730,7 @@ int check_grads(const ha_attn_operands& t, const ha_attn_grads& g, const char* w
     HA_REQUIRE((row_counts[i] - 1) * row_strides[i] * 2 + t.d * 2 <= (1ll << 32), HA_ERR_UNSUPPORTED,
                "%s: one head of a gradient tensor may span 4 GiB at most", who);
   }
-  const Workspace w = carve(t, nullptr);
+  const Workspace w = carve(t, sample_size, nullptr);
   HA_REQUIRE(g.workspace && g.workspace_bytes >= w.bytes && ((uintptr_t)g.workspace % 256) == 0, HA_ERR_WORKSPACE,
              "%s: workspace of %lld bytes (256-byte aligned) required", who, (long long)w.bytes);
   return HA_OK;
@@ -777,21 +772,24 @@ int launch_prepare(const ha_attn_operands& t, const ha_attn_grads& g, const Work
   return ha_launch_status("attention backward: delta");
 }
 
+// the sampled keys' sums onto their rows of dk, dv
 template <typename T, int D>
-int launch_round(const ha_attn_operands& t, const ha_attn_grads& g, const Workspace& w, hipStream_t stream) {
+int launch_add_samples(const ha_block_attn_args& a, const ha_attn_grads& g, const Workspace& w, hipStream_t stream) {
+  const ha_attn_operands& t = a.t;
   const int64_t kv_heads = t.heads / t.kv_group;
-  const int64_t rows = t.batch * kv_heads * t.n_k;
-  const int64_t items = rows * (D / 8);
-  hipLaunchKernelGGL((ha_bwd_round_kernel<T, D>), dim3((unsigned)((items + 255) / 256)), dim3(256), 0, stream, w.dk32,
-                     w.dv32, (T*)g.dk, (T*)g.dv, (int)kv_heads, (int)t.n_k, g.dk_stride_b, g.dk_stride_h, g.dk_stride_n,
-                     g.dv_stride_b, g.dv_stride_h, g.dv_stride_n, rows, g.accumulate != 0);
-  return ha_launch_status("attention backward: round");
+  const int64_t slots = t.batch * kv_heads * a.sample_size;
+  const int64_t items = slots * (D / 8);
+  hipLaunchKernelGGL((ha_bwd_add_samples_kernel<T, D>), dim3((unsigned)((items + 255) / 256)), dim3(256), 0, stream,
+                     w.dk32, w.dv32, (T*)g.dk, (T*)g.dv, a.sampled_idx, (int)(a.idx_type == HA_IDX_I64),
+                     a.sampled_stride_b, a.sampled_stride_h, (int)kv_heads, (int)a.sample_size, g.dk_stride_b,
+                     g.dk_stride_h, g.dk_stride_n, g.dv_stride_b, g.dv_stride_h, g.dv_stride_n, slots);
+  return ha_launch_status("attention backward: sampled keys");
 }
 
 template <typename T, int D>
 int run_block_bwd(const ha_block_attn_args& a, const ha_attn_grads& g, hipStream_t stream) {
   const ha_attn_operands& t = a.t;
-  const Workspace w = carve(t, g.workspace);
+  const Workspace w = carve(t, a.sample_size, g.workspace);
   int st = launch_prepare<T, D>(t, g, w, stream);
   if (st != HA_OK) return st;
   ha_attn_bwd_params p;
@@ -810,6 +808,11 @@ int run_block_bwd(const ha_block_attn_args& a, const ha_attn_grads& g, hipStream
   st = launch_pass<T, D, HA_BWD_DKV_BLOCK, false>(p, bhk * (t.n_k / ST_ROWS), stream, "ha_block_attn_bwd: dk, dv of the blocks");
   if (st != HA_OK) return st;
   if (a.sample_size > 0) {
+    const int64_t n4 = (w.acc_floats + 3) / 4;
+    hipLaunchKernelGGL(ha_bwd_zero_kernel, dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, stream, (f32x4*)w.dk32, n4);
+    hipLaunchKernelGGL(ha_bwd_zero_kernel, dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, stream, (f32x4*)w.dv32, n4);
+    st = ha_launch_status("attention backward: clear");
+    if (st != HA_OK) return st;
     // every query attends every sampled key: the queries are cut into ranges, as long as possible (each
     // range ends in one atomic add per element of the sampled rows) while two workgroups per CU remain
     int64_t q_split = 8192;
@@ -819,13 +822,14 @@ int run_block_bwd(const ha_block_attn_args& a, const ha_attn_grads& g, hipStream
     st = launch_pass<T, D, HA_BWD_DKV_SAMPLED, false>(p, bh * (a.sample_size / ST_ROWS) * splits, stream,
                                                       "ha_block_attn_bwd: dk, dv of the sampled keys");
     if (st != HA_OK) return st;
+    return launch_add_samples<T, D>(a, g, w, stream);
   }
-  return launch_round<T, D>(t, g, w, stream);
+  return HA_OK;
 }
 
 template <typename T, int D>
 int run_flash_bwd(const ha_attn_operands& t, bool causal, const ha_attn_grads& g, hipStream_t stream) {
-  const Workspace w = carve(t, g.workspace);
+  const Workspace w = carve(t, 0, g.workspace);
   int st = launch_prepare<T, D>(t, g, w, stream);
   if (st != HA_OK) return st;
   ha_attn_bwd_params p;
@@ -846,11 +850,11 @@ int run_flash_bwd(const ha_attn_operands& t, bool causal, const ha_attn_grads& g
 
 }  // namespace
 
-extern "C" int64_t ha_attn_bwd_workspace_bytes(const ha_attn_operands* t) {
+extern "C" int64_t ha_attn_bwd_workspace_bytes(const ha_attn_operands* t, int64_t sample_size) {
   if (!t || t->batch <= 0 || t->heads <= 0 || t->n_q <= 0 || t->n_k <= 0 || t->d <= 0 || t->kv_group <= 0 ||
-      t->heads % t->kv_group != 0)
+      t->heads % t->kv_group != 0 || sample_size < 0)
     return ha_fail(HA_ERR_SHAPE, "ha_attn_bwd_workspace_bytes: sizes must be positive, kv_group dividing heads");
-  return carve(*t, nullptr).bytes;
+  return carve(*t, sample_size, nullptr).bytes;
 }
 
 extern "C" int ha_block_attn_bwd(const ha_block_attn_args* args, const ha_attn_grads* grads, void* stream) {
@@ -858,7 +862,7 @@ extern "C" int ha_block_attn_bwd(const ha_block_attn_args* args, const ha_attn_g
   const ha_block_attn_args& a = *args;
   int st = ha_check_block_attn_args(a, "ha_block_attn_bwd");
   if (st != HA_OK) return st;
-  st = check_grads(a.t, *grads, "ha_block_attn_bwd");
+  st = check_grads(a.t, a.sample_size, *grads, "ha_block_attn_bwd");
   if (st != HA_OK) return st;
   HA_REQUIRE(!a.accumulate, HA_ERR_UNSUPPORTED, "ha_block_attn_bwd: no backward of the fused merge (accumulate)");
   HA_REQUIRE(!a.smooth_block || a.block_size <= 128 * (MAX_SMOOTH_TILES - 1), HA_ERR_UNSUPPORTED,
@@ -872,7 +876,7 @@ extern "C" int ha_flash_attn_bwd(const ha_attn_operands* t, int causal, const ha
   HA_REQUIRE(t && grads, HA_ERR_NULL, "ha_flash_attn_bwd: null argument");
   int st = ha_check_operands(*t, "ha_flash_attn_bwd");
   if (st != HA_OK) return st;
-  st = check_grads(*t, *grads, "ha_flash_attn_bwd");
+  st = check_grads(*t, 0, *grads, "ha_flash_attn_bwd");
   if (st != HA_OK) return st;
   hipStream_t s = (hipStream_t)stream;
   if (t->dtype == HA_F16)

@@ -150,7 +150,8 @@ class _CausalRecursionFunc(torch.autograd.Function):
                     a, keep = ops._block_attn_args(q2, k1, v1, o_un, lse_un, q_idx, k_idx, module.block_size,
                                                    module.sample_size, scale, module.smooth_block, module.sampled_idx,
                                                    layout_bnhd=False)
-                    g, ws = ops._attn_grads(a.t, do2, dq2, dk1, dv1, layout_bnhd=False, accumulate=True)
+                    g, ws = ops._attn_grads(a.t, do2, dq2, dk1, dv1, layout_bnhd=False, accumulate=True,
+                                            sample_size=module.sample_size)
                     _lib.check(lib.ha_block_attn_bwd(ctypes.byref(a), ctypes.byref(g), stream))
         return None, None, dq, dk, dv
 

@@ -284,7 +284,7 @@ def _wants_grad(*tensors):
     return torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in tensors)
 
 
-def _attn_grads(t, dout, dq, dk, dv, layout_bnhd=True, accumulate=False):
+def _attn_grads(t, dout, dq, dk, dv, layout_bnhd=True, accumulate=False, sample_size=0):
     """AttnGrads for (b,n,h,d) [layout_bnhd] or (b,h,n,d) gradient tensors plus the workspace the C side asks for."""
     sn, sh = (1, 2) if layout_bnhd else (2, 1)
     g = AttnGrads()
@@ -294,7 +294,7 @@ def _attn_grads(t, dout, dq, dk, dv, layout_bnhd=True, accumulate=False):
     g.dk_stride_b, g.dk_stride_h, g.dk_stride_n = dk.stride(0), dk.stride(sh), dk.stride(sn)
     g.dv_stride_b, g.dv_stride_h, g.dv_stride_n = dv.stride(0), dv.stride(sh), dv.stride(sn)
     g.accumulate = int(bool(accumulate))
-    nbytes = _lib.lib().ha_attn_bwd_workspace_bytes(ctypes.byref(t))
+    nbytes = _lib.lib().ha_attn_bwd_workspace_bytes(ctypes.byref(t), sample_size)
     if nbytes <= 0:
         _lib.check(int(nbytes) if nbytes < 0 else -3)
     ws = torch.empty((nbytes,), device=dout.device, dtype=torch.uint8)
@@ -326,7 +326,7 @@ class HyperAttnFunc(torch.autograd.Function):
         dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
         a, keep = _block_attn_args(q, k, v, o, lse, q_sort_idx, k_sort_idx, block_size, sample_size, softmax_scale,
                                    smooth_block, ctx.sampled_idx)
-        g, ws = _attn_grads(a.t, do, dq, dk, dv)
+        g, ws = _attn_grads(a.t, do, dq, dk, dv, sample_size=sample_size)
         with torch.cuda.device(q.device):
             _lib.check(_lib.lib().ha_block_attn_bwd(ctypes.byref(a), ctypes.byref(g), _stream(q)))
         return dq, dk, dv, None, None, None, None, None, None, None

@@ -157,8 +157,8 @@ int ha_flash_attn_fwd(const ha_attn_operands* t, int causal, void* stream);
  * (or, with accumulate, added to in full: a caller that differentiates several attention calls on
  * views of the same tensors, like the causal recursion, sums their gradients without extra passes).
  * Only whole heads: segs == 1 and zero segment offsets.
- * workspace: ha_attn_bwd_workspace_bytes(t) bytes, 256-byte aligned (row statistics and fp32
- * accumulators of dk, dv; cleared by the call).
+ * workspace: ha_attn_bwd_workspace_bytes(t, sample_size) bytes (sample_size = 0 for exact attention),
+ * 256-byte aligned: one float per query, and fp32 sums of the sampled keys, cleared by the call.
  */
 typedef struct {
   const void* dout;  /* (.., n_q, dv)                          */
@@ -174,7 +174,7 @@ typedef struct {
   int accumulate;    /* != 0: dq, dk, dv hold gradients already and the results are added to them   */
 } ha_attn_grads;
 
-int64_t ha_attn_bwd_workspace_bytes(const ha_attn_operands* t);
+int64_t ha_attn_bwd_workspace_bytes(const ha_attn_operands* t, int64_t sample_size);
 
 /* replaces: HyperAttnFunc.backward -> _hyper_attn_backward with _bwd_preprocess_do_o_dot,
  *           _bwd_permuted_block_diagonal_kernel, _bwd_sampled_col_kernel

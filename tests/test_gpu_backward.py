@@ -7,10 +7,11 @@ the closed formulas.  A gradient arriving for the log-sum-exp output is ignored 
 in the reference (src/hyper_attn_triton.py:922-945, src/flash_attn_triton.py:1014-1040): the loss used
 here depends on the attention output only.
 
-Tolerances: norm-wise ||g - ref|| <= tol ||ref|| per gradient tensor, tol = 3e-3 for fp16 and 5e-3 for
+Tolerances: norm-wise ||g - ref|| <= tol ||ref|| per gradient tensor, tol = 3e-3 for fp16 and 8e-3 for
 bf16.  They are wider than the forward's because P and dS are rounded to the input type before the
 products, as the reference does (src/hyper_attn_triton.py:345,367), and dS has twice the relative
-error of P (150 random configurations stay below 1.6e-3 in fp16 and 3.1e-3 in bf16).
+error of P, and gradients that several calls add to are rounded once per call (350 random
+configurations stay below 1.6e-3 in fp16 and 5.4e-3 in bf16).
 """
 import numpy as np
 import pytest
@@ -22,7 +23,7 @@ pytestmark = pytest.mark.gpu
 
 from _util import _gen, _randn
 
-TOL = {torch.float16: 3e-3, torch.bfloat16: 5e-3}
+TOL = {torch.float16: 3e-3, torch.bfloat16: 8e-3}
 
 
 @pytest.fixture(scope="module")
@@ -196,7 +197,7 @@ def test_backward_grouped_query_heads_through_the_c_abi(ha, kind):
         a, keep = ops._block_attn_args(qg, kg, vg, o, lse, qi_g, ki_g, block, sample, d ** -0.5, False, None)
         assert a.t.kv_group == 2
         _lib.check(lib.ha_block_attn_fwd(ctypes.byref(a), stream))
-        g, ws = ops._attn_grads(a.t, dog, dq, dk, dv)
+        g, ws = ops._attn_grads(a.t, dog, dq, dk, dv, sample_size=sample)
         _lib.check(lib.ha_block_attn_bwd(ctypes.byref(a), ctypes.byref(g), stream))
     else:
         t = ops._operands(qg, kg, vg, o, lse, d ** -0.5, layout_bnhd=True, lse_row_stride=n)
