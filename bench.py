@@ -14,6 +14,8 @@ Besides the whole-forward time the line carries
                 launch stream, against the MI355X dense fp16/bf16 MFMA peak;
   kernels       the same figure for the other kernels of the path (hash, sort: HBM; exact leaves: MFMA);
   exact_flash   our exact MFMA flash-attention forward at the same shape (the 20x comparison);
+  backward      forward under autograd + backward of the module at the same shape, and of the exact
+                attention, as the reference's sweep script times them (not part of `value`);
   cpu_baseline  the CPU oracle (float32, torch) on a bounded sample of the same workload.
 """
 import argparse
@@ -123,6 +125,7 @@ def main():
     ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-exact", action="store_true", help="skip timing the exact flash kernel at the same shape")
+    ap.add_argument("--no-backward", action="store_true", help="skip timing forward + backward under autograd")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run three plain device copies of Q (a kernel of known traffic, to scale HBM byte "
                          "counters collected with rocprofv3 --pmc)")
@@ -289,6 +292,28 @@ def main():
                  "frac_of_mfma_peak": round(exact_flops / ms / 1e9 / MFMA_PEAK_TFLOPS, 4),
                  "speedup_of_hyper": round(ms / ms_per_step, 2)}
 
+    backward = None
+    if not args.no_backward:
+        def fwd_bwd_ms(fn, tensors, reps):
+            """(ms of the forward under autograd, ms of the backward), each the mean over reps calls"""
+            leaves = [x.detach().clone().requires_grad_() for x in tensors]
+            o = fn(*leaves)
+            do = torch.randn_like(o)
+            o.backward(do)
+            f = time_events(lambda: fn(*leaves), reps, torch)
+            o = fn(*leaves)
+            bw = time_events(lambda: o.backward(do, retain_graph=True), reps, torch)
+            return f, bw
+
+        f_ms, b_ms = fwd_bwd_ms(lambda a, b_, c: m(a, b_, c, causal=w["causal"]), (q, k, v), 5)
+        backward = {"fwd_autograd_ms": round(f_ms, 3), "bwd_ms": round(b_ms, 3), "fwd_bwd_ms": round(f_ms + b_ms, 3)}
+        if not args.no_exact and hk == h:
+            ef, eb = fwd_bwd_ms(lambda a, b_, c: ops.flash_attn_func(a.transpose(1, 2), b_.transpose(1, 2), c.transpose(1, 2),
+                                                                    None, w["causal"], scale)[0], (q, k, v), 2)
+            backward["exact_fwd_bwd_ms"] = round(ef + eb, 3)
+            backward["speedup_of_hyper"] = round((ef + eb) / (f_ms + b_ms), 2)
+        torch.cuda.empty_cache()
+
     result = {
         "metric": METRIC if args.workload == "c3" else f"HyperAttention fwd ms ({args.workload})",
         "value": round(ms_per_step, 4), "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -300,7 +325,7 @@ def main():
                    "seed": seed},
         "algorithmic_TFLOPs": round(algo_flops / ms_per_step / 1e9, 1),
         "exact_equivalent_TFLOPs": round(exact_flops / ms_per_step / 1e9, 1),
-        "roofline": roofline, "kernels": kernels, "exact_flash": exact,
+        "roofline": roofline, "kernels": kernels, "exact_flash": exact, "backward": backward,
     }
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(w, seed)
