@@ -49,6 +49,10 @@ class _CausalRecursionFunc(torch.autograd.Function):
             _lib.check(lib.ha_flash_attn_fwd(ctypes.byref(t), 1, stream))
             out, lse = o_leaf.clone(), lse_leaf.clone()
 
+            # a row's bucket does not depend on the level: hash once, sort per level
+            hashed = [j for j in range(levels) if not module.min_seq_len > lens[j + 1]]
+            if hashed:
+                buckets_q, buckets_k = module.lsh.hash(query), module.lsh.hash(key)
             per_level = []
             for j in reversed(range(levels)):  # deepest level first, as the recursion returns
                 H, half = h << j, lens[j + 1]
@@ -62,8 +66,8 @@ class _CausalRecursionFunc(torch.autograd.Function):
                     _lib.check(lib.ha_flash_attn_fwd(ctypes.byref(t), 0, stream))
                 else:
                     num_keys = 1 << module.lsh_num_projs
-                    q_idx = ops.bucket_argsort(module.lsh.hash(q2), num_keys)
-                    k_idx = ops.bucket_argsort(module.lsh.hash(k1), num_keys)
+                    q_idx = ops.bucket_argsort(buckets_q.view(b, H, 2, half)[:, :, 1], num_keys, torch.int32)
+                    k_idx = ops.bucket_argsort(buckets_k.view(b, H, 2, half)[:, :, 0], num_keys, torch.int32)
                     a, keep = ops._block_attn_args(q2, k1, v1, o_un, lse_un, q_idx, k_idx, module.block_size,
                                                    module.sample_size, scale, module.smooth_block, module.sampled_idx,
                                                    layout_bnhd=False)
