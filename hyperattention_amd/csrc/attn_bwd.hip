@@ -38,15 +38,6 @@ namespace {
 constexpr int WG_THREADS = 256;
 constexpr int ST_ROWS = 128;       // stationary rows per workgroup
 constexpr int YC = 64;             // streamed rows per LDS tile
-#ifndef BWD_INTERLEAVE
-#define BWD_INTERLEAVE 1
-#endif
-#ifndef BWD_VALU_PER
-#define BWD_VALU_PER 5
-#endif
-#ifndef BWD_TRANS_PER
-#define BWD_TRANS_PER 2
-#endif
 constexpr int MAX_SMOOTH_TILES = 1024;  // query tiles that can attend one 128-key tile (smoothed blocks)
 
 // LDS layout of a streamed tile: row-major [64][D] 2-byte elements, the 16-byte pieces of a row XOR-ed
@@ -417,8 +408,9 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_bwd_ker
       needs_mask = y_hi >= y_end;
     }
 
-    // One chunk of one wave as straight-line code (one copy with the mask, one without), so that the
-    // scheduler can mix the soft-max arithmetic of one 32-row half with the MFMAs of the other.
+    // One chunk of one wave as straight-line code, one copy with the mask and one without: the
+    // scheduler is free to mix the soft-max arithmetic of one 32-row half with the MFMAs of the other
+    // (forcing a particular interleave with scheduling groups made no difference).
     auto chunk_body = [&](auto masked_tag) {
       constexpr bool MASKED = decltype(masked_tag)::value;
       const unsigned char* const y1 = lds_y1[buf];
@@ -494,16 +486,6 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_bwd_ker
               acc2[db] = Mfma<T>::run(t2, pb[rb][kk], acc2[db]);
             }
           }
-      // Issue order: every MFMA of the chunk is followed by a share of the vector arithmetic that is
-      // ready by then (none behind the first half's S' and dP' MFMAs, the first half's soft-max behind
-      // the second half's, and so on), instead of all MFMAs first and all arithmetic after.
-      constexpr int N_MFMA = BWD_INTERLEAVE ? 4 * KSTEPS + 4 * DB * (KEY_ST ? 2 : 1) : 0;
-#pragma unroll
-      for (int g = 0; g < N_MFMA; ++g) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);            // one MFMA
-        __builtin_amdgcn_sched_group_barrier(0x002, BWD_VALU_PER, 0); // vector instructions
-        __builtin_amdgcn_sched_group_barrier(0x400, BWD_TRANS_PER, 0);  // exponentials
-      }
     };
     if (wave_in) {
       if (needs_mask)
