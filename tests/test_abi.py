@@ -48,6 +48,8 @@ int main(void) {
          offsetof(ha_forward_args, workspace_bytes));
   printf("%zu %zu %zu\n", offsetof(ha_block_attn_args, q_idx), offsetof(ha_forward_args, scale),
          offsetof(ha_forward_args, v_stride_n));
+  printf("%zu %zu %zu\n", sizeof(ha_attn_grads), offsetof(ha_attn_grads, workspace_bytes),
+         offsetof(ha_attn_grads, accumulate));
   return 0;
 }''')
     exe = tmp_path / "layout"
@@ -57,7 +59,8 @@ int main(void) {
     want = [ctypes.sizeof(_lib.AttnOperands), ctypes.sizeof(_lib.BlockAttnArgs), ctypes.sizeof(_lib.ForwardArgs),
             _lib.AttnOperands.scale.offset, _lib.BlockAttnArgs.accumulate.offset,
             _lib.ForwardArgs.workspace_bytes.offset, _lib.BlockAttnArgs.q_idx.offset, _lib.ForwardArgs.scale.offset,
-            _lib.ForwardArgs.v_stride_n.offset]
+            _lib.ForwardArgs.v_stride_n.offset,
+            ctypes.sizeof(_lib.AttnGrads), _lib.AttnGrads.workspace_bytes.offset, _lib.AttnGrads.accumulate.offset]
     assert got == want
 
 
@@ -146,6 +149,20 @@ def test_forward_plan_and_workspace(lib):
     f.n, f.min_seq_len = 1000, 2048  # exact path: no workspace needed beyond the minimum
     assert lib.ha_forward_workspace_bytes(ctypes.byref(f)) == 256
     assert lib.ha_forward(ctypes.byref(f), None) == -1  # null tensors
+
+
+def test_backward_argument_errors_before_any_launch(lib):
+    t = _lib.AttnOperands()
+    g = _lib.AttnGrads()
+    assert lib.ha_flash_attn_bwd(None, 0, None, None) == -1
+    assert lib.ha_flash_attn_bwd(ctypes.byref(t), 0, ctypes.byref(g), None) == -1  # null tensors
+    assert lib.ha_attn_bwd_workspace_bytes(ctypes.byref(t), 0) == -3                # zero sizes
+    t.batch, t.heads, t.n_q, t.n_k, t.d, t.dv, t.kv_group = 2, 4, 300, 200, 64, 64, 2
+    # one float per query (256-byte aligned) + two fp32 (batch, kv_heads, sample_size, d) arrays
+    assert lib.ha_attn_bwd_workspace_bytes(ctypes.byref(t), 0) == 9728
+    assert lib.ha_attn_bwd_workspace_bytes(ctypes.byref(t), 128) == 9728 + 2 * (2 * 2 * 128 * 64 * 4)
+    a = _lib.BlockAttnArgs()
+    assert lib.ha_block_attn_bwd(ctypes.byref(a), ctypes.byref(g), None) == -1
 
 
 def test_python_layer_fails_loudly_without_library(monkeypatch, tmp_path):
