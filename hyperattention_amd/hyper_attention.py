@@ -5,6 +5,11 @@ Contiguous inputs whose causal recursion only meets even lengths take one librar
 (ha_forward: hash once, all sorts in one batch, leaves, then each level merged in place).  Other
 shapes (an odd length somewhere in the recursion, more than 8 projections) are composed here from
 the same HIP operators, following the reference's recursion step by step.
+
+With inputs that require grad the forward keeps what the backward needs: the non-causal case is one
+differentiable operator call, the causal recursion with even lengths runs on views of the tensors
+with the calls' gradients accumulated by the kernels (_CausalRecursionFunc), anything else operator
+by operator under torch autograd.
 """
 from __future__ import annotations
 

@@ -5,9 +5,11 @@ Reference interfaces mirrored here:
   hash            <- AngularLSHTriton.hash_triton           src/angular_lsh_triton.py:99-145,181-182
   bucket_argsort  <- torch.sort(..., dim=2, stable=True)[1] hyper_attention.py:116-117
   indexing        <- indexing                               src/attn_utils.py:27-50
-  hyper_attn_func <- hyper_attn_func (forward)              src/hyper_attn_triton.py:668-742,895-920
-  flash_attn_func <- flash_attn_func (forward, no bias)     src/flash_attn_triton.py:795-872,995-1012
+  hyper_attn_func <- hyper_attn_func                        src/hyper_attn_triton.py:668-742,895-945
+  flash_attn_func <- flash_attn_func (no bias)              src/flash_attn_triton.py:795-872,995-1040
   add_self_attentions <- add_self_attentions                src/attn_utils.py:6-24
+The two attention operators are differentiable in q, k, v (HyperAttnFunc, FlashAttnFunc below: torch
+autograd functions over ha_block_attn_bwd / ha_flash_attn_bwd), as the reference's are.
 """
 from __future__ import annotations
 
