@@ -105,9 +105,12 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_bwd_ker
   const int st_total = PASS == HA_BWD_DKV_SAMPLED ? p.sample_size : (KEY_ST ? p.n_k : p.n_q);
   const int st_tiles = (st_total + ST_ROWS - 1) / ST_ROWS;
   const int splits = PASS == HA_BWD_DKV_SAMPLED ? (p.n_q + p.q_split - 1) / p.q_split : 1;
-  int rest = blockIdx.x;
-  const int tile = rest % st_tiles;
+  int rest = xcd_contiguous_id(blockIdx.x, gridDim.x);
+  int tile = rest % st_tiles;
   rest /= st_tiles;
+  // causal dq: the tiles with the most keys first, so that the last workgroups of the grid are short
+  // (the dk/dv tiles are in that order as they come: the first key tile streams the most queries)
+  if (PASS == HA_BWD_DQ_EXACT && CAUSAL) tile = st_tiles - 1 - tile;
   const int split = rest % splits;
   const int bh = rest / splits;
   // The dK/dV passes that see every query of a key (exact attention, the blocks) take one workgroup per

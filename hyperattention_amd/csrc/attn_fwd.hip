@@ -48,22 +48,12 @@ constexpr int WG_THREADS = 256;
 constexpr int WG_QUERIES = 256;  // sorted query positions per workgroup
 constexpr int KC = 64;           // keys per LDS tile
 constexpr float HALF_SUM_LIMIT = 16384.f;  // 2^14: a lane's half-step sum below this has no fp16 overflow
-constexpr int NUM_XCD = 8;
 
 // Head dims whose kernel needs more than 256 registers keep the S^T accumulators in VGPRs by hand.
 template <int D>
 struct S_IN_VGPR {
   static constexpr bool value = D > 64;
 };
-
-// Workgroups are handed to the 8 XCDs round-robin by their linear id, and each XCD has its own L2.
-// Re-number them so that every XCD works through one contiguous range of (head, query tile): the
-// query tiles that share a head's K/V then meet in the same L2.
-__device__ __forceinline__ int xcd_contiguous_id(int linear, int total) {
-  const int xcd = (unsigned)linear % NUM_XCD, k = (unsigned)linear / NUM_XCD;
-  const int q = (unsigned)total / NUM_XCD, r = (unsigned)total % NUM_XCD;
-  return xcd * q + (xcd < r ? xcd : r) + k;
-}
 
 // x / y for 0 <= x < 2^31 by the divisor's multiply-and-shift constants
 __device__ __forceinline__ int fast_div(int x, ha_divisor y) { return (int)(((uint64_t)(uint32_t)x * y.magic) >> y.shift); }

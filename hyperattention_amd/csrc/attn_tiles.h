@@ -9,6 +9,17 @@ namespace {
 
 constexpr float LOG2E = 1.4426950408889634f;
 constexpr float LN2 = 0.6931471805599453f;
+constexpr int NUM_XCD = 8;
+
+// Workgroups are handed to the 8 XCDs round-robin by their linear id, and each XCD has its own L2.
+// Re-number them so that every XCD works through one contiguous range of (head, tile): the
+// tiles that share a head's rows then meet in the same L2.
+__device__ __forceinline__ int xcd_contiguous_id(int linear, int total) {
+  const int xcd = (unsigned)linear % NUM_XCD, k = (unsigned)linear / NUM_XCD;
+  const int q = (unsigned)total / NUM_XCD, r = (unsigned)total % NUM_XCD;
+  return xcd * q + (xcd < r ? xcd : r) + k;
+}
+
 
 template <typename T>
 struct Mfma;
