@@ -322,12 +322,13 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_bwd_ker
   const int my_lr = lane / PR;  // row inside one tile load
   int rows_next[LPW];           // source rows of this wave's loads of the next tile
   int group_next = 0;           // the query head (within the group) those rows belong to
-  int stat_row_next = 0;        // wave 0, dK/dV passes: source row of streamed row `lane` of the next tile
+  int stat_row_next = 0;        // dK/dV passes: source row of streamed row 16 * wave + lane % 16 of the next tile
+                                // (every wave fetches the statistics of 16 rows: no wave has more to do)
   float stat_lse = 0.f, stat_delta = 0.f;
   auto fetch_rows = [&](int c) {
 #pragma unroll
     for (int j = 0; j < LPW; ++j) rows_next[j] = stream_row(c, (wave_s * LPW + j) * RPL + my_lr);
-    if (KEY_ST && wave_s == 0) stat_row_next = stream_row(c, lane);
+    if (KEY_ST) stat_row_next = stream_row(c, wave_s * 16 + (lane & 15));
     group_next = group_of(c);
   };
   auto load_tile = [&](int buf) {  // the tile whose rows are in rows_next
@@ -342,7 +343,7 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_bwd_ker
       global_to_lds_16(row_address(y1b, rows_next[j], y1_rb, piece), dst1);
       global_to_lds_16(row_address(y2b, rows_next[j], y2_rb, piece), dst2);
     }
-    if (KEY_ST && wave_s == 0) {
+    if (KEY_ST) {
       stat_lse = lse_head(group_next)[stat_row_next] * LOG2E;
       stat_delta = delta_head(group_next)[stat_row_next] * p.scale;
     }
@@ -381,9 +382,9 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_bwd_ker
 
   for (int c = 0; c < nc; ++c) {
     const int buf = c & 1;
-    if (KEY_ST && wave_s == 0) {
-      lds_lse[buf][lane] = stat_lse;
-      lds_delta[buf][lane] = stat_delta;
+    if (KEY_ST && lane < 16) {
+      lds_lse[buf][wave_s * 16 + lane] = stat_lse;
+      lds_delta[buf][wave_s * 16 + lane] = stat_delta;
     }
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's part of tile c has landed
     __syncthreads();
