@@ -263,3 +263,25 @@ def test_module_backward_twice_and_retain_graph(ha):
     for a, b_ in zip(first, (qg.grad, kg.grad, vg.grad)):
         # the sampled keys' sums are accumulated with atomics, in an order that can differ between runs
         assert ((a.double() - b_.double()).norm() / a.double().norm()).item() < 1e-3
+
+
+def test_module_backward_on_views_agrees_with_operator_by_operator_at_length_32768(ha):
+    # two routes to the same gradient at a length the CPU oracle does not reach: the recursion on views
+    # with accumulated gradients, and the reference's recursion operator by operator under torch autograd
+    dtype, b, h, n, d = torch.bfloat16, 1, 4, 32768, 64
+    q, k, v, do = (_randn((b, h, n, d), 80 + i, dtype).cuda() for i in range(4))
+    m = ha.HyperAttention(input_dim=d, block_size=256, sample_size=256, min_seq_len=2048, rng=_gen(85)).to(device="cuda", dtype=dtype)
+    grads = []
+    for route in ("views", "operators"):
+        qg, kg, vg = (x.clone().requires_grad_() for x in (q, k, v))
+        if route == "views":
+            out = m(qg, kg, vg, causal=True)
+        else:
+            out, _ = m._forward_composed(qg, kg, vg, d ** -0.5, True)
+        out.backward(do)
+        grads.append((out.detach(), qg.grad, kg.grad, vg.grad))
+    torch.cuda.synchronize()
+    for a, b_, name in zip(grads[0], grads[1], ("out", "dq", "dk", "dv")):
+        rel = ((a.double() - b_.double()).norm() / b_.double().norm()).item()
+        # both round to bf16, the operator route once per level more (its gradients are added by torch)
+        assert rel < 8e-3, f"{name}: {rel:.3e}"
