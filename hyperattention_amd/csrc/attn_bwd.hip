@@ -78,7 +78,7 @@ __device__ __forceinline__ typename ElemTraits<T>::vec8 bwd_read_tr(const unsign
 }
 
 template <typename T, int D, int PASS, bool CAUSAL>
-__global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_bwd_kernel(const ha_attn_bwd_params p) {
+__global__ __launch_bounds__(WG_THREADS, (D <= 64 || PASS == HA_BWD_DQ_BLOCK ? 2 : 1)) void ha_attn_bwd_kernel(const ha_attn_bwd_params p) {
   typedef typename ElemTraits<T>::vec8 vec8;
   typedef typename ElemTraits<T>::vec4 vec4;
   constexpr bool KEY_ST = PASS == HA_BWD_DKV_EXACT || PASS == HA_BWD_DKV_BLOCK || PASS == HA_BWD_DKV_SAMPLED;
