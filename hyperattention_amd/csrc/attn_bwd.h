@@ -5,6 +5,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "ha_common.h"
+
 // which gradient a launch computes, and over which (query, key) pairs
 enum ha_bwd_pass {
   HA_BWD_DQ_EXACT = 0,     // dq of exact attention
@@ -16,8 +18,7 @@ enum ha_bwd_pass {
 
 struct ha_attn_bwd_params {
   const void *q, *k, *v, *dout;
-  const float* lse;    // forward log-sum-exp (natural log), (batch, heads, n_q) by lse_sb / lse_sh
-  const float* delta;  // sum_c dO*O per query, fp32, contiguous (batch, heads, n_q)
+  const f32x2* stats;  // per query {log-sum-exp * log2(e), scale * sum_c dO*O}, contiguous (batch, heads, n_q)
   void* dq;
   void *dk, *dv;       // written directly by the exact and the block passes
   float *dk32, *dv32;  // fp32 (batch, heads / kv_group, sample_size, d): sums of the sampled keys, by slot
@@ -28,7 +29,6 @@ struct ha_attn_bwd_params {
   int64_t dq_sb, dq_sh, dq_sn;
   int64_t dk_sb, dk_sh, dk_sn;
   int64_t dv_sb, dv_sh, dv_sn;
-  int64_t lse_sb, lse_sh;
   const void *q_idx, *k_idx, *sampled_idx;
   int64_t qi_sb, qi_sh, qi_sn;
   int64_t ki_sb, ki_sh, ki_sn;

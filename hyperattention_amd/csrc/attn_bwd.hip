@@ -133,8 +133,8 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 || PASS == HA_BWD_DQ_BLOCK ? 2
   // query-side tensors of query head h0 + gi
   auto q_head = [&](int gi) { return (const unsigned char*)((const T*)p.q + b * p.q_sb + (h0 + gi) * p.q_sh); };
   auto do_head = [&](int gi) { return (const unsigned char*)((const T*)p.dout + b * p.do_sb + (h0 + gi) * p.do_sh); };
-  auto lse_head = [&](int gi) { return p.lse + b * p.lse_sb + (h0 + gi) * p.lse_sh; };
-  auto delta_head = [&](int gi) { return p.delta + (int64_t)(b * p.heads + h0 + gi) * p.n_q; };
+  // per query: {L in log2 units, D * scale}, written by the preparation kernel
+  auto stats_head = [&](int gi) { return p.stats + (int64_t)(b * p.heads + h0 + gi) * p.n_q; };
   const int idx_shift = p.idx64 ? 3 : 2;
   auto q_idx_head = [&](int gi) {
     return (const unsigned char*)p.q_idx + ((b * p.qi_sb + (h0 + gi) * p.qi_sh) << idx_shift);
@@ -179,8 +179,9 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 || PASS == HA_BWD_DQ_BLOCK ? 2
   }
   float st_lse2 = 0.f, st_delta = 0.f;  // dQ passes: L (log2 units) and D * scale of the lane's query
   if (!KEY_ST) {
-    st_lse2 = lse_head(0)[st_row] * LOG2E;
-    st_delta = delta_head(0)[st_row] * p.scale;
+    const f32x2 sd = stats_head(0)[st_row];
+    st_lse2 = sd[0];
+    st_delta = sd[1];
   }
 
   // ---- the streamed chunks of this workgroup ---------------------------------------------------
@@ -344,8 +345,9 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 || PASS == HA_BWD_DQ_BLOCK ? 2
       global_to_lds_16(row_address(y2b, rows_next[j], y2_rb, piece), dst2);
     }
     if (KEY_ST) {
-      stat_lse = lse_head(group_next)[stat_row_next] * LOG2E;
-      stat_delta = delta_head(group_next)[stat_row_next] * p.scale;
+      const f32x2 sd = stats_head(group_next)[stat_row_next];
+      stat_lse = sd[0];
+      stat_delta = sd[1];
     }
   };
 
@@ -581,23 +583,28 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 || PASS == HA_BWD_DQ_BLOCK ? 2
   }
 }
 
-// D_i = sum_c dO_ic O_ic (src/hyper_attn_triton.py:195-226): one 16-byte piece per lane, a row per
-// group of D/8 lanes
+// Per query {L * log2(e), D * scale} with D_i = sum_c dO_ic O_ic (src/hyper_attn_triton.py:195-226): what
+// the passes need of a query besides its rows, in one 8-byte word.  One 16-byte piece per lane, a row per
+// group of D/8 lanes.
 template <typename T, int D>
-__global__ __launch_bounds__(256) void ha_bwd_delta_kernel(const T* __restrict__ out, const T* __restrict__ dout,
-                                                           float* __restrict__ delta, int heads, int n_q, int64_t o_sb,
-                                                           int64_t o_sh, int64_t o_sn, int64_t do_sb, int64_t do_sh,
-                                                           int64_t do_sn, int64_t total_rows) {
+__global__ __launch_bounds__(256) void ha_bwd_stats_kernel(const T* __restrict__ out, const T* __restrict__ dout,
+                                                           const float* __restrict__ lse, f32x2* __restrict__ stats,
+                                                           int heads, int n_q, int64_t o_sb, int64_t o_sh, int64_t o_sn,
+                                                           int64_t do_sb, int64_t do_sh, int64_t do_sn, int64_t lse_sb,
+                                                           int64_t lse_sh, float scale, int64_t total_rows) {
   typedef typename ElemTraits<T>::vec8 vec8;
   constexpr int PR = D / 8;
   const int64_t item = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   const int64_t grow = item / PR;
   const int piece = (int)(item % PR);
   float acc = 0.f;
+  int64_t b = 0, h = 0;
+  int row = 0;
   if (grow < total_rows) {
     const int64_t bh = grow / n_q;
-    const int row = (int)(grow - bh * n_q);
-    const int64_t b = bh / heads, h = bh - b * heads;
+    row = (int)(grow - bh * n_q);
+    b = bh / heads;
+    h = bh - b * heads;
     const vec8 o = *reinterpret_cast<const vec8*>(out + b * o_sb + h * o_sh + row * o_sn + piece * 8);
     const vec8 g = *reinterpret_cast<const vec8*>(dout + b * do_sb + h * do_sh + row * do_sn + piece * 8);
 #pragma unroll
@@ -605,7 +612,7 @@ __global__ __launch_bounds__(256) void ha_bwd_delta_kernel(const T* __restrict__
   }
 #pragma unroll
   for (int m = 1; m < PR; m <<= 1) acc += __shfl_xor(acc, m);
-  if (grow < total_rows && piece == 0) delta[grow] = acc;
+  if (grow < total_rows && piece == 0) stats[grow] = f32x2{lse[b * lse_sb + h * lse_sh + row] * LOG2E, acc * scale};
 }
 
 __global__ __launch_bounds__(256) void ha_bwd_zero_kernel(f32x4* __restrict__ buf, int64_t n4) {
@@ -679,7 +686,7 @@ int launch_pass(const ha_attn_bwd_params& p, int64_t grid, hipStream_t stream, c
 inline int64_t align256(int64_t v) { return (v + 255) & ~(int64_t)255; }
 
 struct Workspace {
-  float* delta;
+  f32x2* stats;  // per query {L * log2(e), D * scale}
   float* dk32;  // sums of the sampled keys, (batch, kv_heads, sample_size, d) fp32
   float* dv32;
   int64_t acc_floats;  // per accumulator
@@ -688,10 +695,10 @@ struct Workspace {
 
 Workspace carve(const ha_attn_operands& t, int64_t sample_size, void* base) {
   Workspace w;
-  const int64_t delta_bytes = align256(t.batch * t.heads * t.n_q * 4);
+  const int64_t delta_bytes = align256(t.batch * t.heads * t.n_q * 8);
   w.acc_floats = t.batch * (t.heads / t.kv_group) * sample_size * t.d;
   const int64_t acc_bytes = align256(w.acc_floats * 4);
-  w.delta = (float*)base;
+  w.stats = (f32x2*)base;
   w.dk32 = (float*)((char*)base + delta_bytes);
   w.dv32 = (float*)((char*)base + delta_bytes + acc_bytes);
   w.bytes = delta_bytes + 2 * acc_bytes;
@@ -724,7 +731,7 @@ int check_grads(const ha_attn_operands& t, int64_t sample_size, const ha_attn_gr
 
 void fill_bwd_params(const ha_attn_operands& t, const ha_attn_grads& g, const Workspace& w, ha_attn_bwd_params& p) {
   p.q = t.q; p.k = t.k; p.v = t.v; p.dout = g.dout;
-  p.lse = t.lse; p.delta = w.delta;
+  p.stats = w.stats;
   p.dq = g.dq; p.dk = g.dk; p.dv = g.dv; p.dk32 = w.dk32; p.dv32 = w.dv32;
   p.q_sb = t.q_stride_b; p.q_sh = t.q_stride_h; p.q_sn = t.q_stride_n;
   p.k_sb = t.k_stride_b; p.k_sh = t.k_stride_h; p.k_sn = t.k_stride_n;
@@ -733,7 +740,6 @@ void fill_bwd_params(const ha_attn_operands& t, const ha_attn_grads& g, const Wo
   p.dq_sb = g.dq_stride_b; p.dq_sh = g.dq_stride_h; p.dq_sn = g.dq_stride_n;
   p.dk_sb = g.dk_stride_b; p.dk_sh = g.dk_stride_h; p.dk_sn = g.dk_stride_n;
   p.dv_sb = g.dv_stride_b; p.dv_sh = g.dv_stride_h; p.dv_sn = g.dv_stride_n;
-  p.lse_sb = t.lse_stride_b; p.lse_sh = t.lse_stride_h;
   p.q_idx = p.k_idx = p.sampled_idx = nullptr;
   p.qi_sb = p.qi_sh = p.qi_sn = 0;
   p.ki_sb = p.ki_sh = p.ki_sn = 0;
@@ -747,15 +753,16 @@ void fill_bwd_params(const ha_attn_operands& t, const ha_attn_grads& g, const Wo
   p.scale_log2 = t.scale * LOG2E;
 }
 
-// D_i for every query
+// {L, D} for every query
 template <typename T, int D>
 int launch_prepare(const ha_attn_operands& t, const ha_attn_grads& g, const Workspace& w, hipStream_t stream) {
   const int64_t rows = t.batch * t.heads * t.n_q;
   const int64_t items = rows * (D / 8);
-  hipLaunchKernelGGL((ha_bwd_delta_kernel<T, D>), dim3((unsigned)((items + 255) / 256)), dim3(256), 0, stream,
-                     (const T*)t.out, (const T*)g.dout, w.delta, (int)t.heads, (int)t.n_q, t.o_stride_b, t.o_stride_h,
-                     t.o_stride_n, g.do_stride_b, g.do_stride_h, g.do_stride_n, rows);
-  return ha_launch_status("attention backward: delta");
+  hipLaunchKernelGGL((ha_bwd_stats_kernel<T, D>), dim3((unsigned)((items + 255) / 256)), dim3(256), 0, stream,
+                     (const T*)t.out, (const T*)g.dout, t.lse, w.stats, (int)t.heads, (int)t.n_q, t.o_stride_b, t.o_stride_h,
+                     t.o_stride_n, g.do_stride_b, g.do_stride_h, g.do_stride_n, t.lse_stride_b, t.lse_stride_h, t.scale,
+                     rows);
+  return ha_launch_status("attention backward: row statistics");
 }
 
 // the sampled keys' sums onto their rows of dk, dv

@@ -158,7 +158,7 @@ int ha_flash_attn_fwd(const ha_attn_operands* t, int causal, void* stream);
  * views of the same tensors, like the causal recursion, sums their gradients without extra passes).
  * Only whole heads: segs == 1 and zero segment offsets.
  * workspace: ha_attn_bwd_workspace_bytes(t, sample_size) bytes (sample_size = 0 for exact attention),
- * 256-byte aligned: one float per query, and fp32 sums of the sampled keys, cleared by the call.
+ * 256-byte aligned: two floats per query, and fp32 sums of the sampled keys, cleared by the call.
  */
 typedef struct {
   const void* dout;  /* (.., n_q, dv)                          */

@@ -158,9 +158,9 @@ def test_backward_argument_errors_before_any_launch(lib):
     assert lib.ha_flash_attn_bwd(ctypes.byref(t), 0, ctypes.byref(g), None) == -1  # null tensors
     assert lib.ha_attn_bwd_workspace_bytes(ctypes.byref(t), 0) == -3                # zero sizes
     t.batch, t.heads, t.n_q, t.n_k, t.d, t.dv, t.kv_group = 2, 4, 300, 200, 64, 64, 2
-    # one float per query (256-byte aligned) + two fp32 (batch, kv_heads, sample_size, d) arrays
-    assert lib.ha_attn_bwd_workspace_bytes(ctypes.byref(t), 0) == 9728
-    assert lib.ha_attn_bwd_workspace_bytes(ctypes.byref(t), 128) == 9728 + 2 * (2 * 2 * 128 * 64 * 4)
+    # two floats per query (256-byte aligned) + two fp32 (batch, kv_heads, sample_size, d) arrays
+    assert lib.ha_attn_bwd_workspace_bytes(ctypes.byref(t), 0) == 19200
+    assert lib.ha_attn_bwd_workspace_bytes(ctypes.byref(t), 128) == 19200 + 2 * (2 * 2 * 128 * 64 * 4)
     a = _lib.BlockAttnArgs()
     assert lib.ha_block_attn_bwd(ctypes.byref(a), ctypes.byref(g), None) == -1
 
