@@ -93,6 +93,8 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 || PASS == HA_BWD_DQ_BLOCK ? 2
   __shared__ __attribute__((aligned(1024))) unsigned char lds_y2[2][TILE_BYTES];
   __shared__ __attribute__((aligned(16))) float lds_lse[2][YC];    // dK/dV passes: L (log2 units) of the streamed queries
   __shared__ __attribute__((aligned(16))) float lds_delta[2][YC];  // and their D * scale
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_x1[KEY_ST ? ST_ROWS * D * 2 : 16];  // staging of the
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_x2[KEY_ST ? ST_ROWS * D * 2 : 16];  // stationary rows
   __shared__ int lds_tiles[PASS == HA_BWD_DKV_BLOCK ? MAX_SMOOTH_TILES : 1];
   __shared__ int lds_ntiles;
 
@@ -171,19 +173,6 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 || PASS == HA_BWD_DQ_BLOCK ? 2
     else
       st_row = pos;
   }
-  vec8 x1f[KSTEPS], x2f[KSTEPS];
-#pragma unroll
-  for (int ks = 0; ks < KSTEPS; ++ks) {
-    x1f[ks] = *reinterpret_cast<const vec8*>(row_address(x1b, st_row, x1_rb, (ks * 16 + hi * 8) * 2));
-    x2f[ks] = *reinterpret_cast<const vec8*>(row_address(x2b, st_row, x2_rb, (ks * 16 + hi * 8) * 2));
-  }
-  float st_lse2 = 0.f, st_delta = 0.f;  // dQ passes: L (log2 units) and D * scale of the lane's query
-  if (!KEY_ST) {
-    const f32x2 sd = stats_head(0)[st_row];
-    st_lse2 = sd[0];
-    st_delta = sd[1];
-  }
-
   // ---- the streamed chunks of this workgroup ---------------------------------------------------
   const int T_blk = p.block_tiles;
   const int nkc = p.n_k / YC;  // gathered passes: n_k % 128 == 0
@@ -351,7 +340,44 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 || PASS == HA_BWD_DQ_BLOCK ? 2
     }
   };
 
+  // the row numbers of the first tile are asked for before the stationary rows, so that the two chains
+  // index -> rows run side by side
   fetch_rows(0);
+  vec8 x1f[KSTEPS], x2f[KSTEPS];
+  float st_lse2 = 0.f, st_delta = 0.f;  // dQ passes: L (log2 units) and D * scale of the lane's query
+  if (!KEY_ST) {
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) {
+      x1f[ks] = *reinterpret_cast<const vec8*>(row_address(x1b, st_row, x1_rb, (ks * 16 + hi * 8) * 2));
+      x2f[ks] = *reinterpret_cast<const vec8*>(row_address(x2b, st_row, x2_rb, (ks * 16 + hi * 8) * 2));
+    }
+    const f32x2 sd = stats_head(0)[st_row];
+    st_lse2 = sd[0];
+    st_delta = sd[1];
+  } else {
+    // The dK/dV passes fetch their stationary rows through LDS: whole rows per 8 or 16 consecutive lanes
+    // (one 128- or 256-byte request per row) instead of one 16-byte piece of 64 different rows per
+    // instruction.  Each wave stages its own 32 rows, so only the wave itself has to wait.
+    constexpr int ROWS_PER_LOAD = 64 / PR;
+    const int row_in_load = lane / PR, phys_piece = lane % PR;
+#pragma unroll
+    for (int j = 0; j < 32 / ROWS_PER_LOAD; ++j) {
+      const int r = j * ROWS_PER_LOAD + row_in_load;  // 0..31: a stationary row of this wave
+      const int row = __shfl(st_row, r);
+      const uint32_t piece = (uint32_t)((phys_piece ^ bwd_swizzle<D>(r)) << 4);
+      const int dst = (wave_s * 32 + j * ROWS_PER_LOAD) * D * 2;
+      global_to_lds_16(row_address(x1b, row, x1_rb, piece), lds_x1 + dst);
+      global_to_lds_16(row_address(x2b, row, x2_rb, piece), lds_x2 + dst);
+    }
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): these rows, and the row numbers of the first tile
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) {
+      const int off = bwd_tile_offset<D>(wave_s * 32 + col, ks * 2 + hi);
+      x1f[ks] = lds_read_k<T>(lds_x1, off);
+      x2f[ks] = lds_read_k<T>(lds_x2, off);
+    }
+  }
+
   load_tile(0);
   fetch_rows(1);
 
