@@ -10,8 +10,10 @@ here depends on the attention output only.
 Tolerances: norm-wise ||g - ref|| <= tol ||ref|| per gradient tensor, tol = 3e-3 for fp16 and 8e-3 for
 bf16.  They are wider than the forward's because P and dS are rounded to the input type before the
 products, as the reference does (src/hyper_attn_triton.py:345,367), and dS has twice the relative
-error of P, and gradients that several calls add to are rounded once per call (350 random
-configurations stay below 1.6e-3 in fp16 and 5.4e-3 in bf16).
+error of P, and gradients that several calls add to are rounded once per call.  500 random
+configurations with the default soft-max scale stay below 1.6e-3 in fp16 and 5.4e-3 in bf16; with
+scales up to 0.2 (peaked soft-max: dP - D cancels, and D comes from the rounded output) fp16 reaches
+3.0e-3.
 """
 import numpy as np
 import pytest
