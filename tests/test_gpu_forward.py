@@ -245,3 +245,32 @@ def test_grouped_query_heads(ha):
                                       lsh_num_projs=8, block_size=256, sample_size=256, min_seq_len=1024,
                                       smooth_block=False)
     assert torch.equal(native, attn) and torch.equal(lse_n.unsqueeze(-1), lse)
+
+
+def test_forward_is_capturable_in_a_hip_graph(ha):
+    # The library neither allocates, nor synchronises, nor records memsets: one forward (hash, sorts,
+    # leaves, levels) can be captured into a HIP graph and replayed on new data.  Every replay is
+    # compared with the eager result, with eager work and synchronisations between the replays.
+    dtype, b, h, n, d = torch.float16, 1, 4, 4096, 64
+    m = ha.HyperAttention(input_dim=d, block_size=256, sample_size=256, min_seq_len=1024, rng=_gen(90)).to(
+        device="cuda", dtype=dtype)
+    q, k, v = (_randn((b, h, n, d), 91 + i, dtype).cuda() for i in range(3))
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):  # warm-up on a side stream, as graph capture asks for
+        for _ in range(2):
+            m(q, k, v, causal=True)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = m(q, k, v, causal=True)
+    for it in range(3):
+        fresh = [_randn((b, h, n, d), 100 + 3 * it + i, dtype).cuda() for i in range(3)]
+        for dst, src in zip((q, k, v), fresh):
+            dst.copy_(src)
+        graph.replay()
+        torch.cuda.synchronize()
+        want = m(*fresh, causal=True)
+        torch.cuda.synchronize()
+        assert torch.equal(out, want), f"replay {it} differs from the eager forward"
