@@ -74,6 +74,8 @@ def _gpu_grads(fn, q, k, v, do):
     (torch.bfloat16, 1, 2, 200, 517, 128, False),    # more keys than queries
     (torch.float16, 1, 1, 640, 130, 64, False),      # more queries than keys
     (torch.float16, 1, 2, 1, 1, 64, True),           # a single row
+    (torch.float16, 1, 2, 300, 130, 64, True),       # causal with fewer keys than queries (mask row >= col)
+    (torch.bfloat16, 1, 2, 200, 517, 128, True),     # causal with more keys: the last keys get no gradient
 ])
 def test_flash_backward(ha, dtype, b, h, nq, nk, d, causal):
     q = _randn((b, h, nq, d), 11, dtype)
