@@ -528,7 +528,54 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 || PASS == HA_BWD_DQ_BLOCK ? 2
   }
 
   // ---- results -------------------------------------------------------------------------------
-  if (!KEY_ST && st_valid) {
+  // A lane holds 4 consecutive elements of 16 pieces of ONE row.  In the gathered passes, whose rows lie
+  // all over the head, each wave turns its 32 x D results around in LDS (its quarter of the first tile
+  // buffer pair, free once every wave has left the loop), so that 8 or 16 consecutive lanes write one
+  // whole row, 16 bytes each, instead of every lane 8 bytes of its own row per instruction (3.5 %; the
+  // exact passes, whose rows are neighbours anyway, lose 1-3 % to the extra barrier and registers).
+  constexpr bool TURN_RESULTS = PASS == HA_BWD_DQ_BLOCK || PASS == HA_BWD_DKV_BLOCK;
+  if (TURN_RESULTS) {
+    __syncthreads();
+    unsigned char* const turn = lds_y1[0] + wave_s * (32 * D * 2);
+    constexpr int ROWS_PER_STORE = 64 / PR;
+    const int row_in_store = lane / PR, out_piece = lane % PR;
+    auto store_rows = [&](const f32x16 (&acc)[DB], unsigned char* base, int64_t row_stride_bytes) {
+      // [row][D] in the output type, 16-byte pieces XOR-ed with the row number
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          vec4 o;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) o[e] = (T)acc[db][g * 4 + e];
+          const int piece = (4 * db + g) ^ (col & (PR - 1));
+          *reinterpret_cast<vec4*>(turn + col * (D * 2) + piece * 16 + hi * 8) = o;
+        }
+#pragma unroll
+      for (int j = 0; j < 32 / ROWS_PER_STORE; ++j) {
+        const int r = j * ROWS_PER_STORE + row_in_store;
+        const int row = __shfl(st_row, r);
+        const bool valid = __shfl((int)st_valid, r) != 0;
+        vec8 o = *reinterpret_cast<const vec8*>(turn + r * (D * 2) + ((out_piece ^ (r & (PR - 1))) << 4));
+        if (valid) {
+          vec8* const dst = reinterpret_cast<vec8*>(base + row * row_stride_bytes + out_piece * 16);
+          if (p.accumulate) {
+            const vec8 old = *dst;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) o[e] = (T)((float)o[e] + (float)old[e]);
+          }
+          *dst = o;
+        }
+      }
+    };
+    if (!KEY_ST) {
+      store_rows(acc1, (unsigned char*)((T*)p.dq + b * p.dq_sb + h0 * p.dq_sh), p.dq_sn * 2);
+    } else {
+      store_rows(acc1, (unsigned char*)((T*)p.dk + b * p.dk_sb + hk * p.dk_sh), p.dk_sn * 2);
+      store_rows(acc2, (unsigned char*)((T*)p.dv + b * p.dv_sb + hk * p.dv_sh), p.dv_sn * 2);
+    }
+  }
+  if (!TURN_RESULTS && !KEY_ST && st_valid) {
     unsigned char* const dqb = (unsigned char*)((T*)p.dq + b * p.dq_sb + h0 * p.dq_sh) + (int64_t)st_row * p.dq_sn * 2;
 #pragma unroll
     for (int db = 0; db < DB; ++db)
@@ -546,7 +593,7 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 || PASS == HA_BWD_DQ_BLOCK ? 2
         }
         *dst = o;
       }
-  } else if ((PASS == HA_BWD_DKV_EXACT || PASS == HA_BWD_DKV_BLOCK) && st_valid) {
+  } else if (!TURN_RESULTS && (PASS == HA_BWD_DKV_EXACT || PASS == HA_BWD_DKV_BLOCK) && st_valid) {
     // complete sums (of the blocks: every key is in exactly one tile of the sorted order): straight to dk, dv
     unsigned char* const dkb = (unsigned char*)((T*)p.dk + b * p.dk_sb + hk * p.dk_sh) + (int64_t)st_row * p.dk_sn * 2;
     unsigned char* const dvb = (unsigned char*)((T*)p.dv + b * p.dv_sb + hk * p.dv_sh) + (int64_t)st_row * p.dv_sn * 2;
