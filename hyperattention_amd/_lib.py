@@ -30,6 +30,7 @@ SYMBOLS = [
     "ha_abi_version", "ha_last_error", "ha_lsh_hash", "ha_bucket_argsort_workspace_bytes",
     "ha_bucket_argsort", "ha_gather_rows", "ha_block_attn_fwd", "ha_flash_attn_fwd",
     "ha_attn_bwd_workspace_bytes", "ha_block_attn_bwd", "ha_flash_attn_bwd", "ha_lse_merge",
+    "ha_lse_merge_segments",
     "ha_forward_workspace_bytes", "ha_forward",
 ]
 
@@ -155,6 +156,8 @@ def _declare(lib):
     lib.ha_flash_attn_bwd.argtypes = [ctypes.POINTER(AttnOperands), ci, ctypes.POINTER(AttnGrads), vp]
     lib.ha_lse_merge.restype = ci
     lib.ha_lse_merge.argtypes = [vp] * 6 + [i64] * 8 + [ci, vp]
+    lib.ha_lse_merge_segments.restype = ci
+    lib.ha_lse_merge_segments.argtypes = [vp] * 7 + [i64] * 13 + [ci, vp]
     lib.ha_forward_workspace_bytes.restype = i64
     lib.ha_forward_workspace_bytes.argtypes = [ctypes.POINTER(ForwardArgs)]
     lib.ha_forward.restype = ci

@@ -77,12 +77,15 @@ class _CausalRecursionFunc(torch.autograd.Function):
                                                    module.sample_size, scale, module.smooth_block, module.sampled_idx,
                                                    layout_bnhd=False)
                     _lib.check(lib.ha_block_attn_fwd(ctypes.byref(a), stream))
-                # merge into the second halves, in place
+                # merge into the second halves, in place; c: the weight of what was there (fp32 copy of the
+                # weight rounded to the attention's type)
                 out2 = out.view(b, H, 2, half, d)[:, :, 1]
                 lse2 = lse.view(b, H, 2, half)[:, :, 1]
-                c = torch.sigmoid(lse2 - lse_un).unsqueeze(-1).to(query.dtype)
-                out2.mul_(c).add_((1 - c) * o_un)
-                lse2.sub_((c + torch.finfo(torch.float32).eps).log().squeeze(-1))
+                c = torch.empty((b, H, half), **f32)
+                _lib.check(lib.ha_lse_merge_segments(
+                    out2.data_ptr(), lse2.data_ptr(), o_un.data_ptr(), lse_un.data_ptr(), out2.data_ptr(),
+                    lse2.data_ptr(), c.data_ptr(), b * H, half, d, 2 * half * d, d, half * d, d, 2 * half * d, d,
+                    2 * half, half, 2 * half, half, ops._dtype_code(query), stream))
                 per_level.append((j, o_un, lse_un, c, q_idx, k_idx))
 
         tensors = [query, key, value, o_leaf, lse_leaf]
@@ -126,7 +129,7 @@ class _CausalRecursionFunc(torch.autograd.Function):
             lse_shifted = {}
             for j in range(levels):
                 H, half = h << j, lens[j + 1]
-                lse_un, c = per_level[j][1], per_level[j][2].squeeze(-1).float()
+                lse_un, c = per_level[j][1], per_level[j][2]
                 log_w2 = log_w.view(b, H, 2, half)[:, :, 1]
                 lse_shifted[j] = lse_un - torch.log1p(-c) - log_w2
                 log_w2.add_(torch.log(c))

@@ -200,6 +200,23 @@ int ha_lse_merge(const void* attn1, const float* lse1, const void* attn2, const 
                  int64_t lse1_stride, int64_t lse2_stride, int64_t lse_out_stride,
                  int dtype, void* stream);
 
+/* The same merge for rows that come in `segs` equal segments of `seg_len` rows, each tensor with its own
+ * segment and row strides (in elements; lse and weight arrays: segment strides, rows contiguous): e.g. the
+ * second halves of all heads of a (batch, heads, n, d) tensor, in place when the output aliases the
+ * first input.  The weight c of the first input (rounded to dtype first, src/attn_utils.py:21) is used
+ * for the merge and, if weight_out is not NULL, written out as fp32: a caller that differentiates the
+ * merge needs it (d attn1 = c * d attn, d attn2 = (1 - c) * d attn).  No counterpart in the reference
+ * beyond add_self_attentions itself; it serves the causal recursion (hyper_attention.py:86-89).
+ */
+int ha_lse_merge_segments(const void* attn1, const float* lse1, const void* attn2, const float* lse2,
+                          void* attn_out, float* lse_out, float* weight_out,
+                          int64_t segs, int64_t seg_len, int64_t d,
+                          int64_t attn1_seg_stride, int64_t attn1_row_stride,
+                          int64_t attn2_seg_stride, int64_t attn2_row_stride,
+                          int64_t out_seg_stride, int64_t out_row_stride,
+                          int64_t lse1_seg_stride, int64_t lse2_seg_stride, int64_t lse_out_seg_stride,
+                          int64_t weight_seg_stride, int dtype, void* stream);
+
 /* ---------------------------------------------------------------------------------------------
  * Whole forward pass of the module for (batch, heads, n, d) tensors, one call, no host
  * synchronisation and no tensor copies.

@@ -82,6 +82,9 @@ def test_argument_errors_before_any_launch(lib):
     assert lib.ha_gather_rows(one, one, 0, one, 1, 1, 8, 8, 8, 3, 0, 0, 3, 2, None) == -4
     # merge
     assert lib.ha_lse_merge(one, one, one, one, one, one, 8, 12, 12, 12, 12, 1, 1, 1, 0, None) == -3
+    assert lib.ha_lse_merge_segments(one, one, one, one, one, one, None, 2, 8, 12, 96, 12, 96, 12, 96, 12, 8, 8, 8, 8, 0, None) == -3
+    assert lib.ha_lse_merge_segments(one, one, one, one, one, one, None, 2, 8, 16, 128, 16, 128, 16, 128, 16, 8, 8, 8, 8, 5, None) == -2
+    assert lib.ha_lse_merge_segments(one, None, one, one, one, one, None, 2, 8, 16, 128, 16, 128, 16, 128, 16, 8, 8, 8, 8, 0, None) == -1
 
 
 def _operands(**kw):

@@ -350,3 +350,39 @@ def test_add_self_attentions(ha, dtype):
     # and against the exact attention over the union of the two key sets
     ro, rl = O.exact_attention(q, k, v)
     assert_close(got, ro, "merge vs union", dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_merge_segments_in_place(ha, dtype):
+    """ha_lse_merge_segments on the second halves of every head, in place, with the weight written out:
+    the merge of one level of the causal recursion (hyper_attention.py:86-89)."""
+    import ctypes
+    from hyperattention_amd import _lib
+    b, h, n, d = 2, 3, 256, 64
+    half = n // 2
+    q, k, v = (_randn((b, h, n, d), s, dtype) for s in (60, 61, 62))
+    q2 = q[:, :, half:]
+    a1, l1 = O.exact_attention(q2, k[:, :, half:], v[:, :, half:])          # what the second halves hold
+    a2, l2 = O.exact_attention(q2, k[:, :, :half], v[:, :, :half])          # the un-masked call of the level
+    out = torch.zeros((b, h, n, d), dtype=dtype).cuda()
+    lse = torch.zeros((b, h, n), dtype=torch.float32).cuda()
+    out[:, :, half:] = a1.to(dtype).cuda()
+    lse[:, :, half:] = l1.float().cuda()
+    o_un, lse_un = a2.to(dtype).cuda().contiguous(), l2.float().cuda().contiguous()
+    w = torch.empty((b, h, half), dtype=torch.float32, device="cuda")
+    out2, lse2 = out[:, :, half:], lse[:, :, half:]
+    lib = _lib.lib()
+    _lib.check(lib.ha_lse_merge_segments(
+        out2.data_ptr(), lse2.data_ptr(), o_un.data_ptr(), lse_un.data_ptr(), out2.data_ptr(), lse2.data_ptr(),
+        w.data_ptr(), b * h, half, d, n * d, d, half * d, d, n * d, d, n, half, n, half,
+        0 if dtype == torch.float16 else 1, ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)))
+    torch.cuda.synchronize()
+    want, wlse = O.add_self_attentions(a1.to(dtype).double(), l1.float().double().unsqueeze(-1),
+                                       a2.to(dtype).double(), l2.float().double().unsqueeze(-1))
+    assert_close(out[:, :, half:], want, "segment merge out", dtype)
+    assert_close(lse[:, :, half:], wlse.squeeze(-1), "segment merge lse")
+    ro, rl = O.exact_attention(q2, k, v)
+    assert_close(out[:, :, half:], ro, "segment merge vs union", dtype)
+    assert float(out[:, :, :half].abs().max()) == 0 and float(lse[:, :, :half].abs().max()) == 0  # first halves untouched
+    c = torch.sigmoid(l1.float() - l2.float()).to(dtype).float()
+    assert float((w.cpu() - c).abs().max()) <= 2 * torch.finfo(dtype).eps
