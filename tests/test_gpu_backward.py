@@ -289,3 +289,46 @@ def test_module_backward_on_views_agrees_with_operator_by_operator_at_length_327
         rel = ((a.double() - b_.double()).norm() / b_.double().norm()).item()
         # both round to bf16, the operator route once per level more (its gradients are added by torch)
         assert rel < 8e-3, f"{name}: {rel:.3e}"
+
+
+def test_full_size_causal_backward_properties(ha):
+    """Benchmark shape (batch 1, 32 heads, seq 131072, d 64, fp16, causal), too long for the oracle's
+    autograd: what the mathematics fixes at any size.
+
+    Every call of the recursion is soft-max attention over some set of keys, merged with weights that sum
+    to one per query, and the scores enter as q.k only.  So per head
+      sum_i <q_i, dq_i> = sum_ij S_ij dS_ij = sum_j <k_j, dk_j>,
+      sum_j dv_j = sum_i dout_i                        (every query's weights over all its keys sum to one),
+    the gradients are linear in dout, and a query of the first leaf only ever meets exact causal
+    attention, so its dq is the exact attention's on that leaf (checked against the oracle)."""
+    b, h, n, d = 1, 32, 131072, 64
+    g = torch.Generator(device="cuda").manual_seed(190)
+    q, k, v = (torch.randn((b, h, n, d), generator=g, device="cuda", dtype=torch.float16).requires_grad_()
+               for _ in range(3))
+    dout = torch.randn((b, h, n, d), generator=g, device="cuda", dtype=torch.float16)
+    m = ha.HyperAttention(input_dim=d, block_size=256, sample_size=256, min_seq_len=2048,
+                          rng=torch.Generator().manual_seed(191)).to(device="cuda", dtype=torch.float16)
+    out = m(q, k, v, causal=True)
+    dq, dk, dv = torch.autograd.grad(out, (q, k, v), dout, retain_graph=True)
+    assert all(torch.isfinite(x).all() for x in (dq, dk, dv))
+
+    qdq, kdk = (q.detach().float() * dq.float()), (k.detach().float() * dk.float())
+    a, c = qdq.double().sum((0, 2, 3)), kdk.double().sum((0, 2, 3))
+    noise = qdq.double().pow(2).sum((0, 2, 3)).sqrt() + kdk.double().pow(2).sum((0, 2, 3)).sqrt()
+    assert float(((a - c).abs() / noise).max()) < 3e-3, ((a - c).abs() / noise).max()  # measured 6e-4
+
+    sv, so = dv.double().sum(2), dout.double().sum(2)
+    rel = (sv - so).norm() / so.norm()
+    assert float(rel) < 2e-4, rel  # measured 2e-5
+
+    dq2, dk2, dv2 = torch.autograd.grad(out, (q, k, v), 2 * dout, retain_graph=True)
+    for x2, x, what in ((dq2, dq, "dq"), (dk2, dk, "dk"), (dv2, dv, "dv")):
+        rel = (x2.double() - 2 * x.double()).norm() / x.double().norm()
+        assert float(rel) < 1e-3, (what, rel)  # measured 3e-4: P and dS are rounded, small values lose bits
+
+    # queries of the first leaf: exact causal attention only
+    leaf = slice(0, 2048)
+    ql, kl, vl = (x[:, :2, leaf].detach().double().cpu().requires_grad_() for x in (q, k, v))
+    ro, _ = O.exact_attention(ql, kl, vl, None, True)
+    (rdq,) = torch.autograd.grad(ro, (ql,), dout[:, :2, leaf].double().cpu())
+    _check(dq[:, :2, leaf], rdq, "dq of the first leaf", torch.float16)
