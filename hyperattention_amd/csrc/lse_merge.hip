@@ -8,9 +8,8 @@
 namespace {
 
 template <typename T>
-__global__ __launch_bounds__(256) void lse_merge_kernel(const T* __restrict__ a1, const float* __restrict__ l1,
-                                                        const T* __restrict__ a2, const float* __restrict__ l2,
-                                                        T* __restrict__ ao, float* __restrict__ lo, int64_t rows,
+__global__ __launch_bounds__(256) void lse_merge_kernel(const T* a1, const float* l1, const T* a2, const float* l2,
+                                                        T* ao, float* lo, int64_t rows,
                                                         int pieces, int64_t s1, int64_t s2, int64_t so,
                                                         int64_t ls1, int64_t ls2, int64_t lso) {
   typedef typename ElemTraits<T>::vec8 vec8;
@@ -43,6 +42,12 @@ extern "C" int ha_lse_merge(const void* attn1, const float* lse1, const void* at
              HA_ERR_SHAPE, "ha_lse_merge: rows must be 16-byte aligned");
   const int pieces = (int)(d / 8);
   const int64_t items = rows * pieces;
+  // In place, the lanes of a row read its log-sum-exps before one of them writes the merged one: that
+  // holds inside a wave, so a row's d/8 lanes must not straddle two waves.
+  const bool in_place = lse_out == lse1 || lse_out == lse2 || attn_out == attn1 || attn_out == attn2;
+  HA_REQUIRE(!in_place || 64 % pieces == 0, HA_ERR_UNSUPPORTED,
+             "ha_lse_merge: in place needs a head dimension of 8, 16, 32, 64, 128, 256 or 512");
+  HA_REQUIRE((items + 255) / 256 < (1ll << 31), HA_ERR_SHAPE, "ha_lse_merge: too many rows");
   dim3 grid((unsigned)((items + 255) / 256));
   hipStream_t s = (hipStream_t)stream;
   if (dtype == HA_F16)
@@ -63,9 +68,9 @@ extern "C" int ha_lse_merge(const void* attn1, const float* lse1, const void* at
 namespace {
 
 template <typename T>
-__global__ __launch_bounds__(256) void lse_merge_segments_kernel(const T* __restrict__ a1, const float* __restrict__ l1,
-                                                                 const T* __restrict__ a2, const float* __restrict__ l2,
-                                                                 T* ao, float* lo, float* __restrict__ wo, int64_t rows,
+__global__ __launch_bounds__(256) void lse_merge_segments_kernel(const T* a1, const float* l1, const T* a2,
+                                                                 const float* l2, T* ao, float* lo,
+                                                                 float* __restrict__ wo, int64_t rows,
                                                                  int64_t seg_len, int pieces, int64_t a1_ss, int64_t a1_rs,
                                                                  int64_t a2_ss, int64_t a2_rs, int64_t ao_ss, int64_t ao_rs,
                                                                  int64_t l1_ss, int64_t l2_ss, int64_t lo_ss, int64_t wo_ss) {
@@ -108,6 +113,11 @@ extern "C" int ha_lse_merge_segments(const void* attn1, const float* lse1, const
   const int pieces = (int)(d / 8);
   const int64_t rows = segs * seg_len, items = rows * pieces;
   HA_REQUIRE((items + 255) / 256 < (1ll << 31), HA_ERR_SHAPE, "ha_lse_merge_segments: too many rows");
+  // In place, the lanes of a row read its log-sum-exps before one of them writes the merged one: that
+  // holds inside a wave, so a row's d/8 lanes must not straddle two waves.
+  const bool in_place = lse_out == lse1 || lse_out == lse2 || attn_out == attn1 || attn_out == attn2;
+  HA_REQUIRE(!in_place || 64 % pieces == 0, HA_ERR_UNSUPPORTED,
+             "ha_lse_merge_segments: in place needs a head dimension of 8, 16, 32, 64, 128, 256 or 512");
   dim3 grid((unsigned)((items + 255) / 256));
   hipStream_t s = (hipStream_t)stream;
   if (dtype == HA_F16)

@@ -192,7 +192,8 @@ int ha_flash_attn_bwd(const ha_attn_operands* t, int causal, const ha_attn_grads
 /* Merge of two partial attentions.
  * replaces: add_self_attentions (src/attn_utils.py:6-24)
  * rows = batch*heads*n flattened; attn*: (rows, d) with row strides; lse*: fp32 with element
- * strides.  Outputs may alias the first inputs.
+ * strides.  An output may be the very tensor of an input (same pointer and strides) when d is 8, 16,
+ * 32, 64, 128, 256 or 512 (HA_ERR_UNSUPPORTED otherwise); partly overlapping tensors are not allowed.
  */
 int ha_lse_merge(const void* attn1, const float* lse1, const void* attn2, const float* lse2,
                  void* attn_out, float* lse_out, int64_t rows, int64_t d,
@@ -202,8 +203,8 @@ int ha_lse_merge(const void* attn1, const float* lse1, const void* attn2, const 
 
 /* The same merge for rows that come in `segs` equal segments of `seg_len` rows, each tensor with its own
  * segment and row strides (in elements; lse and weight arrays: segment strides, rows contiguous): e.g. the
- * second halves of all heads of a (batch, heads, n, d) tensor, in place when the output aliases the
- * first input.  The weight c of the first input (rounded to dtype first, src/attn_utils.py:21) is used
+ * second halves of all heads of a (batch, heads, n, d) tensor, in place when the output is the very
+ * tensor of an input (same rule as ha_lse_merge).  The weight c of the first input (rounded to dtype first, src/attn_utils.py:21) is used
  * for the merge and, if weight_out is not NULL, written out as fp32: a caller that differentiates the
  * merge needs it (d attn1 = c * d attn, d attn2 = (1 - c) * d attn).  No counterpart in the reference
  * beyond add_self_attentions itself; it serves the causal recursion (hyper_attention.py:86-89).

@@ -82,6 +82,10 @@ def test_argument_errors_before_any_launch(lib):
     assert lib.ha_gather_rows(one, one, 0, one, 1, 1, 8, 8, 8, 3, 0, 0, 3, 2, None) == -4
     # merge
     assert lib.ha_lse_merge(one, one, one, one, one, one, 8, 12, 12, 12, 12, 1, 1, 1, 0, None) == -3
+    two = ctypes.c_void_p(32)
+    assert lib.ha_lse_merge(one, one, two, two, one, one, 8, 24, 24, 24, 24, 1, 1, 1, 0, None) == -5  # in place, d = 24
+    assert b"in place" in lib.ha_last_error()
+    assert lib.ha_lse_merge_segments(one, one, two, two, one, one, None, 2, 8, 24, 192, 24, 192, 24, 192, 24, 8, 8, 8, 8, 0, None) == -5
     assert lib.ha_lse_merge_segments(one, one, one, one, one, one, None, 2, 8, 12, 96, 12, 96, 12, 96, 12, 8, 8, 8, 8, 0, None) == -3
     assert lib.ha_lse_merge_segments(one, one, one, one, one, one, None, 2, 8, 16, 128, 16, 128, 16, 128, 16, 8, 8, 8, 8, 5, None) == -2
     assert lib.ha_lse_merge_segments(one, None, one, one, one, one, None, 2, 8, 16, 128, 16, 128, 16, 128, 16, 8, 8, 8, 8, 0, None) == -1
