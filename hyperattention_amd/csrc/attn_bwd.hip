@@ -93,8 +93,9 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 || PASS == HA_BWD_DQ_BLOCK ? 2
   __shared__ __attribute__((aligned(1024))) unsigned char lds_y2[2][TILE_BYTES];
   __shared__ __attribute__((aligned(16))) float lds_lse[2][YC];    // dK/dV passes: L (log2 units) of the streamed queries
   __shared__ __attribute__((aligned(16))) float lds_delta[2][YC];  // and their D * scale
-  __shared__ __attribute__((aligned(1024))) unsigned char lds_x1[KEY_ST ? ST_ROWS * D * 2 : 16];  // staging of the
-  __shared__ __attribute__((aligned(1024))) unsigned char lds_x2[KEY_ST ? ST_ROWS * D * 2 : 16];  // stationary rows
+  constexpr bool STAGE_X = KEY_ST || D <= 64;
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_x1[STAGE_X ? ST_ROWS * D * 2 : 16];  // staging of the
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_x2[STAGE_X ? ST_ROWS * D * 2 : 16];  // stationary rows
   __shared__ int lds_tiles[PASS == HA_BWD_DKV_BLOCK ? MAX_SMOOTH_TILES : 1];
   __shared__ int lds_ntiles;
 
@@ -346,18 +347,21 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 || PASS == HA_BWD_DQ_BLOCK ? 2
   vec8 x1f[KSTEPS], x2f[KSTEPS];
   float st_lse2 = 0.f, st_delta = 0.f;  // dQ passes: L (log2 units) and D * scale of the lane's query
   if (!KEY_ST) {
+    const f32x2 sd = stats_head(0)[st_row];
+    st_lse2 = sd[0];
+    st_delta = sd[1];
+  }
+  if (!STAGE_X) {
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ++ks) {
       x1f[ks] = *reinterpret_cast<const vec8*>(row_address(x1b, st_row, x1_rb, (ks * 16 + hi * 8) * 2));
       x2f[ks] = *reinterpret_cast<const vec8*>(row_address(x2b, st_row, x2_rb, (ks * 16 + hi * 8) * 2));
     }
-    const f32x2 sd = stats_head(0)[st_row];
-    st_lse2 = sd[0];
-    st_delta = sd[1];
   } else {
-    // The dK/dV passes fetch their stationary rows through LDS: whole rows per 8 or 16 consecutive lanes
-    // (one 128- or 256-byte request per row) instead of one 16-byte piece of 64 different rows per
-    // instruction.  Each wave stages its own 32 rows, so only the wave itself has to wait.
+    // The stationary rows come through LDS (dK/dV passes; dQ passes at d = 64, where the 32 KB fit beside
+    // two workgroups per CU): whole rows per 8 or 16 consecutive lanes (one 128- or 256-byte request per
+    // row) instead of one 16-byte piece of 64 different rows per instruction.  Each wave stages its own
+    // 32 rows, so only the wave itself has to wait.
     constexpr int ROWS_PER_LOAD = 64 / PR;
     const int row_in_load = lane / PR, phys_piece = lane % PR;
 #pragma unroll
