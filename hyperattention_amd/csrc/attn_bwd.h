@@ -18,7 +18,10 @@ enum ha_bwd_pass {
 
 struct ha_attn_bwd_params {
   const void *q, *k, *v, *dout;
-  const f32x2* stats;  // per query {log-sum-exp * log2(e), scale * sum_c dO*O}, contiguous (batch, heads, n_q)
+  const void* out;   // the forward's output and log-sum-exp: read by the dq passes, which write `stats`
+  const float* lse;
+  f32x2* stats;  // per query {log-sum-exp * log2(e), scale * sum_c dO*O}, contiguous (batch, heads, n_q): written
+                 // by the dq pass of a call for the dk/dv passes that follow it
   void* dq;
   void *dk, *dv;       // written directly by the exact and the block passes
   float *dk32, *dv32;  // fp32 (batch, heads / kv_group, sample_size, d): sums of the sampled keys, by slot
@@ -26,6 +29,8 @@ struct ha_attn_bwd_params {
   int64_t k_sb, k_sh, k_sn;
   int64_t v_sb, v_sh, v_sn;
   int64_t do_sb, do_sh, do_sn;
+  int64_t o_sb, o_sh, o_sn;
+  int64_t lse_sb, lse_sh;
   int64_t dq_sb, dq_sh, dq_sn;
   int64_t dk_sb, dk_sh, dk_sn;
   int64_t dv_sb, dv_sh, dv_sn;

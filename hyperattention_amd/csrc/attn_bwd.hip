@@ -136,7 +136,8 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 || PASS == HA_BWD_DQ_BLOCK ? 2
   // query-side tensors of query head h0 + gi
   auto q_head = [&](int gi) { return (const unsigned char*)((const T*)p.q + b * p.q_sb + (h0 + gi) * p.q_sh); };
   auto do_head = [&](int gi) { return (const unsigned char*)((const T*)p.dout + b * p.do_sb + (h0 + gi) * p.do_sh); };
-  // per query: {L in log2 units, D * scale}, written by the preparation kernel
+  // per query: {L in log2 units, D * scale} with D_i = sum_c dO_ic O_ic (src/hyper_attn_triton.py:195-226),
+  // written by the dq pass of the call
   auto stats_head = [&](int gi) { return p.stats + (int64_t)(b * p.heads + h0 + gi) * p.n_q; };
   const int idx_shift = p.idx64 ? 3 : 2;
   auto q_idx_head = [&](int gi) {
@@ -346,10 +347,14 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 || PASS == HA_BWD_DQ_BLOCK ? 2
   fetch_rows(0);
   vec8 x1f[KSTEPS], x2f[KSTEPS];
   float st_lse2 = 0.f, st_delta = 0.f;  // dQ passes: L (log2 units) and D * scale of the lane's query
+  vec8 of[KSTEPS];  // dQ passes: the lane's pieces of its query's output row
   if (!KEY_ST) {
-    const f32x2 sd = stats_head(0)[st_row];
-    st_lse2 = sd[0];
-    st_delta = sd[1];
+    const unsigned char* const ob = (const unsigned char*)((const T*)p.out + b * p.o_sb + h0 * p.o_sh);
+    const uint32_t o_rb = (uint32_t)p.o_sn * 2;
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks)
+      of[ks] = *reinterpret_cast<const vec8*>(row_address(ob, st_row, o_rb, (ks * 16 + hi * 8) * 2));
+    st_lse2 = p.lse[b * p.lse_sb + h0 * p.lse_sh + st_row] * LOG2E;
   }
   if (!STAGE_X) {
 #pragma unroll
@@ -384,6 +389,18 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 || PASS == HA_BWD_DQ_BLOCK ? 2
 
   load_tile(0);
   fetch_rows(1);
+
+  if (!KEY_ST) {
+    // D = sum_c dO * O of the lane's query: the two lanes of a column hold complementary pieces of the row.
+    // The dK/dV passes of the call read both statistics from the workspace.
+    float part = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) part = __builtin_fmaf((float)of[ks][e], (float)x2f[ks][e], part);
+    st_delta = (part + __shfl_xor(part, 32)) * p.scale;
+    if (hi == 0 && st_valid) p.stats[(int64_t)(b * p.heads + h0) * p.n_q + st_row] = f32x2{st_lse2, st_delta};
+  }
 
   // per-lane LDS offsets of the operand reads
   int off_rows[KSTEPS];  // piece of k-step ks of tile row lane%32, 16-byte read
@@ -660,38 +677,6 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 || PASS == HA_BWD_DQ_BLOCK ? 2
   }
 }
 
-// Per query {L * log2(e), D * scale} with D_i = sum_c dO_ic O_ic (src/hyper_attn_triton.py:195-226): what
-// the passes need of a query besides its rows, in one 8-byte word.  One 16-byte piece per lane, a row per
-// group of D/8 lanes.
-template <typename T, int D>
-__global__ __launch_bounds__(256) void ha_bwd_stats_kernel(const T* __restrict__ out, const T* __restrict__ dout,
-                                                           const float* __restrict__ lse, f32x2* __restrict__ stats,
-                                                           int heads, int n_q, int64_t o_sb, int64_t o_sh, int64_t o_sn,
-                                                           int64_t do_sb, int64_t do_sh, int64_t do_sn, int64_t lse_sb,
-                                                           int64_t lse_sh, float scale, int64_t total_rows) {
-  typedef typename ElemTraits<T>::vec8 vec8;
-  constexpr int PR = D / 8;
-  const int64_t item = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  const int64_t grow = item / PR;
-  const int piece = (int)(item % PR);
-  float acc = 0.f;
-  int64_t b = 0, h = 0;
-  int row = 0;
-  if (grow < total_rows) {
-    const int64_t bh = grow / n_q;
-    row = (int)(grow - bh * n_q);
-    b = bh / heads;
-    h = bh - b * heads;
-    const vec8 o = *reinterpret_cast<const vec8*>(out + b * o_sb + h * o_sh + row * o_sn + piece * 8);
-    const vec8 g = *reinterpret_cast<const vec8*>(dout + b * do_sb + h * do_sh + row * do_sn + piece * 8);
-#pragma unroll
-    for (int e = 0; e < 8; ++e) acc += (float)o[e] * (float)g[e];
-  }
-#pragma unroll
-  for (int m = 1; m < PR; m <<= 1) acc += __shfl_xor(acc, m);
-  if (grow < total_rows && piece == 0) stats[grow] = f32x2{lse[b * lse_sb + h * lse_sh + row] * LOG2E, acc * scale};
-}
-
 __global__ __launch_bounds__(256) void ha_bwd_zero_kernel(f32x4* __restrict__ buf, int64_t n4) {
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n4) buf[i] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -808,6 +793,9 @@ int check_grads(const ha_attn_operands& t, int64_t sample_size, const ha_attn_gr
 
 void fill_bwd_params(const ha_attn_operands& t, const ha_attn_grads& g, const Workspace& w, ha_attn_bwd_params& p) {
   p.q = t.q; p.k = t.k; p.v = t.v; p.dout = g.dout;
+  p.out = t.out; p.lse = t.lse;
+  p.o_sb = t.o_stride_b; p.o_sh = t.o_stride_h; p.o_sn = t.o_stride_n;
+  p.lse_sb = t.lse_stride_b; p.lse_sh = t.lse_stride_h;
   p.stats = w.stats;
   p.dq = g.dq; p.dk = g.dk; p.dv = g.dv; p.dk32 = w.dk32; p.dv32 = w.dv32;
   p.q_sb = t.q_stride_b; p.q_sh = t.q_stride_h; p.q_sn = t.q_stride_n;
@@ -830,18 +818,6 @@ void fill_bwd_params(const ha_attn_operands& t, const ha_attn_grads& g, const Wo
   p.scale_log2 = t.scale * LOG2E;
 }
 
-// {L, D} for every query
-template <typename T, int D>
-int launch_prepare(const ha_attn_operands& t, const ha_attn_grads& g, const Workspace& w, hipStream_t stream) {
-  const int64_t rows = t.batch * t.heads * t.n_q;
-  const int64_t items = rows * (D / 8);
-  hipLaunchKernelGGL((ha_bwd_stats_kernel<T, D>), dim3((unsigned)((items + 255) / 256)), dim3(256), 0, stream,
-                     (const T*)t.out, (const T*)g.dout, t.lse, w.stats, (int)t.heads, (int)t.n_q, t.o_stride_b, t.o_stride_h,
-                     t.o_stride_n, g.do_stride_b, g.do_stride_h, g.do_stride_n, t.lse_stride_b, t.lse_stride_h, t.scale,
-                     rows);
-  return ha_launch_status("attention backward: row statistics");
-}
-
 // the sampled keys' sums onto their rows of dk, dv
 template <typename T, int D>
 int launch_add_samples(const ha_block_attn_args& a, const ha_attn_grads& g, const Workspace& w, hipStream_t stream) {
@@ -860,8 +836,7 @@ template <typename T, int D>
 int run_block_bwd(const ha_block_attn_args& a, const ha_attn_grads& g, hipStream_t stream) {
   const ha_attn_operands& t = a.t;
   const Workspace w = carve(t, a.sample_size, g.workspace);
-  int st = launch_prepare<T, D>(t, g, w, stream);
-  if (st != HA_OK) return st;
+  int st;
   ha_attn_bwd_params p;
   fill_bwd_params(t, g, w, p);
   p.q_idx = a.q_idx; p.k_idx = a.k_idx; p.sampled_idx = a.sampled_idx;
@@ -900,8 +875,7 @@ int run_block_bwd(const ha_block_attn_args& a, const ha_attn_grads& g, hipStream
 template <typename T, int D>
 int run_flash_bwd(const ha_attn_operands& t, bool causal, const ha_attn_grads& g, hipStream_t stream) {
   const Workspace w = carve(t, 0, g.workspace);
-  int st = launch_prepare<T, D>(t, g, w, stream);
-  if (st != HA_OK) return st;
+  int st;
   ha_attn_bwd_params p;
   fill_bwd_params(t, g, w, p);
   const int64_t bh = t.batch * t.heads, bhk = t.batch * (t.heads / t.kv_group);
