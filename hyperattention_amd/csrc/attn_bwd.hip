@@ -348,12 +348,14 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 || PASS == HA_BWD_DQ_BLOCK ? 2
   vec8 x1f[KSTEPS], x2f[KSTEPS];
   float st_lse2 = 0.f, st_delta = 0.f;  // dQ passes: L (log2 units) and D * scale of the lane's query
   vec8 of[KSTEPS];  // dQ passes: the lane's pieces of its query's output row
+  const unsigned char* const ob = (const unsigned char*)((const T*)p.out + b * p.o_sb + h0 * p.o_sh);
+  const uint32_t o_rb = (uint32_t)p.o_sn * 2;
   if (!KEY_ST) {
-    const unsigned char* const ob = (const unsigned char*)((const T*)p.out + b * p.o_sb + h0 * p.o_sh);
-    const uint32_t o_rb = (uint32_t)p.o_sn * 2;
+    if (!STAGE_X) {
 #pragma unroll
-    for (int ks = 0; ks < KSTEPS; ++ks)
-      of[ks] = *reinterpret_cast<const vec8*>(row_address(ob, st_row, o_rb, (ks * 16 + hi * 8) * 2));
+      for (int ks = 0; ks < KSTEPS; ++ks)
+        of[ks] = *reinterpret_cast<const vec8*>(row_address(ob, st_row, o_rb, (ks * 16 + hi * 8) * 2));
+    }
     st_lse2 = p.lse[b * p.lse_sb + h0 * p.lse_sh + st_row] * LOG2E;
   }
   if (!STAGE_X) {
@@ -385,11 +387,28 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 || PASS == HA_BWD_DQ_BLOCK ? 2
       x1f[ks] = lds_read_k<T>(lds_x1, off);
       x2f[ks] = lds_read_k<T>(lds_x2, off);
     }
+    if (!KEY_ST) {
+      // the queries' output rows (for D) follow through the first staging area, once it has been read
+      __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+      __builtin_amdgcn_wave_barrier();
+#pragma unroll
+      for (int j = 0; j < 32 / ROWS_PER_LOAD; ++j) {
+        const int r = j * ROWS_PER_LOAD + row_in_load;
+        const int row = __shfl(st_row, r);
+        const uint32_t piece = (uint32_t)((phys_piece ^ bwd_swizzle<D>(r)) << 4);
+        global_to_lds_16(row_address(ob, row, o_rb, piece), lds_x1 + (wave_s * 32 + j * ROWS_PER_LOAD) * D * 2);
+      }
+    }
   }
 
   load_tile(0);
   fetch_rows(1);
 
+  if (!KEY_ST && STAGE_X) {
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the output rows (and the first tile) have landed
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) of[ks] = lds_read_k<T>(lds_x1, bwd_tile_offset<D>(wave_s * 32 + col, ks * 2 + hi));
+  }
   if (!KEY_ST) {
     // D = sum_c dO * O of the lane's query: the two lanes of a column hold complementary pieces of the row.
     // The dK/dV passes of the call read both statistics from the workspace.
