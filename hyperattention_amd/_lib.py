@@ -28,13 +28,14 @@ HIPCC_FLAGS = [
 # exported symbols, in the order of include/hyperattn.h
 SYMBOLS = [
     "ha_abi_version", "ha_last_error", "ha_lsh_hash", "ha_bucket_argsort_workspace_bytes",
-    "ha_bucket_argsort", "ha_gather_rows", "ha_block_attn_fwd", "ha_flash_attn_fwd",
+    "ha_bucket_argsort", "ha_bucket_argsort_static", "ha_gather_rows", "ha_block_attn_fwd", "ha_flash_attn_fwd",
     "ha_attn_bwd_workspace_bytes", "ha_block_attn_bwd", "ha_flash_attn_bwd", "ha_lse_merge",
     "ha_lse_merge_segments",
     "ha_forward_workspace_bytes", "ha_forward",
 ]
 
 HA_F16, HA_BF16 = 0, 1
+ABI_VERSION = 4
 HA_IDX_I32, HA_IDX_I64 = 0, 1
 
 
@@ -142,6 +143,8 @@ def _declare(lib):
     lib.ha_bucket_argsort_workspace_bytes.argtypes = [i64, i64, i64]
     lib.ha_bucket_argsort.restype = ci
     lib.ha_bucket_argsort.argtypes = [vp, vp, ci, i64, i64, i64, i64, i64, vp, i64, vp]
+    lib.ha_bucket_argsort_static.restype = ci
+    lib.ha_bucket_argsort_static.argtypes = [vp, vp, ci, i64, i64, i64, i64, i64, vp]
     lib.ha_gather_rows.restype = ci
     lib.ha_gather_rows.argtypes = [vp, vp, ci, vp] + [i64] * 9 + [ci, vp]
     lib.ha_block_attn_fwd.restype = ci
@@ -174,7 +177,7 @@ def lib():
                 "(hipcc, gfx950). There is no fallback path.")
         loaded = ctypes.CDLL(LIB_PATH)
         _declare(loaded)
-        if loaded.ha_abi_version() != 3:
+        if loaded.ha_abi_version() != ABI_VERSION:
             raise RuntimeError("libhyperattn.so: ABI version mismatch")
         _lib = loaded
     return _lib

@@ -13,6 +13,8 @@
 #include "ha_common.h"
 #include "bucket_sort.h"
 
+#include <mutex>
+
 namespace {
 
 constexpr int SORT_THREADS = 256;
@@ -242,9 +244,9 @@ extern "C" int64_t ha_bucket_argsort_workspace_bytes(int64_t num_segments, int64
   return bytes;
 }
 
-extern "C" int ha_bucket_argsort(const int32_t* keys, void* idx_out, int idx_type, int64_t num_segments,
-                                 int64_t seg_len, int64_t seg_stride, int64_t seg_offset, int64_t num_keys,
-                                 void* workspace, int64_t workspace_bytes, void* stream) {
+static int bucket_argsort(const int32_t* keys, void* idx_out, int idx_type, int64_t num_segments, int64_t seg_len,
+                          int64_t seg_stride, int64_t seg_offset, int64_t num_keys, void* workspace,
+                          int64_t workspace_bytes, void* stream) {
   HA_REQUIRE(keys && idx_out, HA_ERR_NULL, "ha_bucket_argsort: null pointer");
   HA_REQUIRE(idx_type == HA_IDX_I32 || idx_type == HA_IDX_I64, HA_ERR_DTYPE, "ha_bucket_argsort: bad idx_type");
   HA_REQUIRE(num_segments > 0 && seg_len > 0, HA_ERR_SHAPE, "ha_bucket_argsort: sizes must be positive");
@@ -287,4 +289,66 @@ extern "C" int ha_bucket_argsort(const int32_t* keys, void* idx_out, int idx_typ
     prev = tmp[p & 1];
   }
   return HA_OK;
+}
+
+extern "C" int ha_bucket_argsort(const int32_t* keys, void* idx_out, int idx_type, int64_t num_segments,
+                                 int64_t seg_len, int64_t seg_stride, int64_t seg_offset, int64_t num_keys,
+                                 void* workspace, int64_t workspace_bytes, void* stream) {
+  return bucket_argsort(keys, idx_out, idx_type, num_segments, seg_len, seg_stride, seg_offset, num_keys, workspace,
+                        workspace_bytes, stream);
+}
+
+// ---- the same sort for callers that cannot allocate ------------------------------------------------
+// The histograms (and, for keys above 255, the two intermediate orders) live in a device array that is
+// part of the library's image: one copy per GPU, held until the process ends.  On the host the array's
+// name is only a handle; its device address is asked for once per device, with that device current, and
+// that address is what the kernels are given.
+static __device__ __align__(256) unsigned char scratch[HA_SORT_SCRATCH_BYTES];
+
+namespace {
+constexpr int MAX_DEVICES = 64;
+std::mutex scratch_mutex;
+void* scratch_ptr[MAX_DEVICES] = {nullptr};
+
+// device address of `scratch` on the current device (0 on failure, with the status in *st)
+void* scratch_on_current_device(int* st) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= MAX_DEVICES) {
+    *st = ha_fail(e != hipSuccess ? (int)e : HA_ERR_UNSUPPORTED, "ha_bucket_argsort_static: no usable current device");
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lock(scratch_mutex);
+  if (!scratch_ptr[dev]) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p) {
+      *st = ha_fail(e != hipSuccess ? (int)e : HA_ERR_WORKSPACE, "ha_bucket_argsort_static: hipGetSymbolAddress: %s",
+                    hipGetErrorString(e));
+      return nullptr;
+    }
+    scratch_ptr[dev] = p;
+  }
+  *st = HA_OK;
+  return scratch_ptr[dev];
+}
+}  // namespace
+
+extern "C" int ha_bucket_argsort_static(const int32_t* keys, void* idx_out, int idx_type, int64_t num_segments,
+                                        int64_t seg_len, int64_t seg_stride, int64_t seg_offset, int64_t num_keys,
+                                        void* stream) {
+  HA_REQUIRE(num_segments > 0 && seg_len > 0, HA_ERR_SHAPE, "ha_bucket_argsort_static: sizes must be positive");
+  HA_REQUIRE(num_segments < (1ll << 24) && seg_len < (1ll << 31), HA_ERR_SHAPE, "ha_bucket_argsort_static: too large");
+  const int64_t need = ha_bucket_argsort_workspace_bytes(num_segments, seg_len, num_keys);
+  HA_REQUIRE(need <= (int64_t)HA_SORT_SCRATCH_BYTES, HA_ERR_WORKSPACE,
+             "ha_bucket_argsort_static: this sort needs %lld bytes of scratch, the built-in array holds %lld; use "
+             "ha_bucket_argsort with a workspace",
+             (long long)need, (long long)HA_SORT_SCRATCH_BYTES);
+  int st = HA_OK;
+  void* ws = scratch_on_current_device(&st);
+  if (!ws) return st;
+  // every histogram entry and intermediate order that is read is written by the same call first: nothing
+  // has to start at zero
+  return bucket_argsort(keys, idx_out, idx_type, num_segments, seg_len, seg_stride, seg_offset, num_keys, ws,
+                        (int64_t)HA_SORT_SCRATCH_BYTES, stream);
 }

@@ -6,7 +6,8 @@
  * type unless stated otherwise) and a HIP stream passed as void* (hipStream_t; NULL = the
  * default stream).  The library launches asynchronously on that stream, never synchronises,
  * never allocates or frees device memory and keeps no state between calls: the caller owns
- * every buffer including workspaces.  Return value: 0 on success, a negative ha_status for an
+ * every buffer including workspaces (the one exception, ha_bucket_argsort_static, uses a device array
+ * that is part of the library's image).  Return value: 0 on success, a negative ha_status for an
  * argument error detected before any launch, or a positive hipError_t from the launch.
  * ha_last_error() returns a thread-local human readable message for the last non-zero status.
  *
@@ -22,7 +23,7 @@
 extern "C" {
 #endif
 
-#define HA_ABI_VERSION 3
+#define HA_ABI_VERSION 4
 
 typedef enum {
   HA_OK = 0,
@@ -70,6 +71,19 @@ int64_t ha_bucket_argsort_workspace_bytes(int64_t num_segments, int64_t seg_len,
 int ha_bucket_argsort(const int32_t* keys, void* idx_out, int idx_type,
                       int64_t num_segments, int64_t seg_len, int64_t seg_stride, int64_t seg_offset,
                       int64_t num_keys, void* workspace, int64_t workspace_bytes, void* stream);
+
+/* The same sort without a workspace argument and without any allocation.
+ * No counterpart in the reference: it is for callers that cannot allocate device memory (code under
+ * HIP graph capture, serving loops, harnesses that forbid hipMalloc).  The scratch memory is a device
+ * array of HA_SORT_SCRATCH_BYTES inside the library (one copy per GPU, held until the process ends); a
+ * sort whose ha_bucket_argsort_workspace_bytes() exceeds it is rejected with HA_ERR_WORKSPACE.  The
+ * device of the call is the current device.  All calls on one GPU share the array: calls that overlap
+ * on one GPU (different streams or threads) race and must be serialised by the caller.
+ */
+#define HA_SORT_SCRATCH_BYTES (8 << 20)
+int ha_bucket_argsort_static(const int32_t* keys, void* idx_out, int idx_type,
+                             int64_t num_segments, int64_t seg_len, int64_t seg_stride, int64_t seg_offset,
+                             int64_t num_keys, void* stream);
 
 /* ---------------------------------------------------------------------------------------------
  * Permuting row gather.

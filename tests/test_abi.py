@@ -32,7 +32,7 @@ def test_every_declared_symbol_is_exported(lib):
     assert declared == sorted(_lib.SYMBOLS)
     for name in declared:
         assert hasattr(lib, name), f"{name} declared in hyperattn.h but not exported"
-    assert lib.ha_abi_version() == 3
+    assert lib.ha_abi_version() == _lib.ABI_VERSION
 
 
 def test_struct_layouts_match_the_header(tmp_path):
@@ -78,6 +78,10 @@ def test_argument_errors_before_any_launch(lib):
     assert lib.ha_bucket_argsort_workspace_bytes(4, 8192, 256) == 4 * 2 * 256 * 4
     assert lib.ha_bucket_argsort(one, one, 0, 4, 8192, 8192, 0, 256, one, 16, None) == -6
     assert lib.ha_bucket_argsort(one, one, 0, 4, 8192, 8192, 0, 1 << 20, one, 1 << 30, None) == -5
+    # the sort without a workspace: more scratch than the built-in array holds
+    assert lib.ha_bucket_argsort_static(one, one, 0, 4096, 1 << 20, 1 << 20, 0, 256, None) == -6
+    assert b"scratch" in lib.ha_last_error()
+    assert lib.ha_bucket_argsort_static(one, one, 0, 0, 8, 8, 0, 256, None) == -3
     # gather: row bytes not a multiple of 16
     assert lib.ha_gather_rows(one, one, 0, one, 1, 1, 8, 8, 8, 3, 0, 0, 3, 2, None) == -4
     # merge
