@@ -138,6 +138,34 @@ def padded_head_dim(d):
     return 64 if d <= 64 else 128
 
 
+def check_sampled_idx(sampled_idx, n_k: int):
+    """An explicit sample list names key rows of the call it is used in: every entry must lie in
+    [0, n_k).  Inside the causal recursion the same list serves every level, so n_k is the key length of
+    the smallest hashed level; a larger entry would read keys of the second half there (future tokens)
+    or past the tensor.  The bounds of a list are computed once per tensor version."""
+    if sampled_idx is None:
+        return
+    cached = getattr(sampled_idx, "_ha_bounds", None)
+    if cached is None or cached[0] != sampled_idx._version:
+        lo, hi = (int(sampled_idx.min()), int(sampled_idx.max())) if sampled_idx.numel() else (0, -1)
+        cached = (sampled_idx._version, lo, hi)
+        sampled_idx._ha_bounds = cached
+    assert cached[1] >= 0 and cached[2] < n_k, \
+        f"sampled_idx must lie in [0, {n_k}) (the key length of the shortest hashed call); got [{cached[1]}, {cached[2]}]"
+
+
+def smallest_hashed_key_length(n: int, min_seq_len: int, causal: bool):
+    """Key length of the shortest call that uses the hashed kernel (hyper_attention.py:52,109), or None."""
+    if not causal:
+        return None if min_seq_len > n else n
+    smallest = None
+    while n > min_seq_len:
+        n = (n + 1) // 2
+        if not min_seq_len > n:
+            smallest = n
+    return smallest
+
+
 def _block_attn_args(q, k, v, o, lse, q_sort_idx, k_sort_idx, block_size, sample_size, softmax_scale,
                      smooth_block, sampled_idx, accumulate=False, layout_bnhd=True):
     """BlockAttnArgs for (b,n,h,d) tensors with (b,n,h) index tensors [layout_bnhd] or (b,h,n,d) tensors
@@ -157,6 +185,7 @@ def _block_attn_args(q, k, v, o, lse, q_sort_idx, k_sort_idx, block_size, sample
     keep = None
     a.sampled_stride_b = a.sampled_stride_h = 0
     if sampled_idx is not None:
+        check_sampled_idx(sampled_idx, k.shape[sn])
         keep = sampled_idx.to(device=q.device, dtype=q_sort_idx.dtype).contiguous()
         assert keep.shape in ((sample_size,), (nheads, sample_size), (batch, nheads, sample_size)), \
             "sampled_idx must be (sample_size,), (nheads, sample_size) or (batch, nheads, sample_size)"
@@ -392,6 +421,9 @@ def hyper_forward(q, k, v, proj, *, scale, causal, lsh_num_projs, block_size, sa
         keep.append(p)
         a.proj = p.data_ptr()
     if sampled_idx is not None:
+        shortest = smallest_hashed_key_length(n, min_seq_len, bool(causal))
+        if shortest is not None:
+            check_sampled_idx(sampled_idx, shortest)
         s = sampled_idx.to(device=q.device, dtype=torch.int32).contiguous()
         assert s.shape == (sample_size,)
         keep.append(s)

@@ -134,6 +134,10 @@ typedef struct {
  * idx + b*idx_stride_b + h*idx_stride_h + g*n + p*idx_stride_n (g = segment); sampled_idx: sample_size
  * key rows (local), shared by all heads when sampled_stride_h == 0 (sampled_idx == NULL means
  * 0,1,..,sample_size-1, the reference's intended set, src/hyper_attn_triton.py:576-581).
+ * PRECONDITION: every entry of sampled_idx lies in [0, n_k).  The list is device memory and is not read
+ * by the host, so the library cannot check it: an entry outside the range reads rows of another
+ * segment or head (inside a causal recursion: future tokens) or past the tensor, and the backward adds
+ * to such rows.  The Python operator layer checks the list on the host before every call.
  * n_q % 128 == 0, n_k % 128 == 0 (:695), sample_size % 128 == 0 (:911), d and dv in {64, 128}.
  * accumulate != 0: out/lse already hold a partial attention over a disjoint key set for every row;
  * the result is merged into them in place (add_self_attentions, src/attn_utils.py:6-24, fused).
@@ -239,7 +243,8 @@ int ha_lse_merge_segments(const void* attn1, const float* lse1, const void* attn
  * shapes where every recursion level has an even length (n = leaf_len * 2^levels); other shapes
  * are composed by the caller from the operators above.
  * proj: (d, r) in dtype.  sampled_idx: int32 key rows local to each un-masked call (NULL = first
- * sample_size rows), shared by all heads and levels.  out (batch,heads,n,dv) dtype, lse
+ * sample_size rows), shared by all heads and levels; PRECONDITION as for ha_block_attn_fwd, with n_k the
+ * key length of the shortest hashed level (n / 2^levels halvings down to the last length >= min_seq_len).  out (batch,heads,n,dv) dtype, lse
  * (batch,heads,n) fp32.  kv_heads divides heads (grouped-query: q head h reads kv head
  * h / (heads/kv_heads)); k and v are (batch, kv_heads, n, d).
  * q/k/v strides in elements, last dim contiguous; a tensor whose three strides are all zero is

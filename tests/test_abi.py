@@ -192,3 +192,29 @@ def test_sweep_script_command_line():
         assert sweep.get_arguments(["--mode", mode]).mode == mode
     with pytest.raises(SystemExit):  # a CUDA-only package: stops before touching the GPU
         sweep.main(["--attn_method", "flash-cuda"])
+
+
+def test_explicit_sample_lists_are_range_checked_on_the_host():
+    """A sample list is local to the keys of each call; inside the causal recursion the shortest hashed
+    level bounds it (a larger row number would name a key of the second half: a future token)."""
+    import torch
+    from hyperattention_amd import ops
+    assert ops.smallest_hashed_key_length(8192, 1024, True) == 1024      # halves 4096, 2048, 1024
+    assert ops.smallest_hashed_key_length(8192, 1025, True) == 2048      # 1024 < min_seq_len: exact there
+    assert ops.smallest_hashed_key_length(8192, 4096, False) == 8192
+    assert ops.smallest_hashed_key_length(1000, 4096, False) is None
+    ok = torch.tensor([0, 5, 1023])
+    ops.check_sampled_idx(ok, 1024)
+    with pytest.raises(AssertionError, match="sampled_idx must lie in"):
+        ops.check_sampled_idx(torch.tensor([0, 5, 1024]), 1024)
+    with pytest.raises(AssertionError, match="sampled_idx must lie in"):
+        ops.check_sampled_idx(torch.tensor([-1, 5]), 1024)
+    ok[2] = 4000  # an in-place change is seen
+    with pytest.raises(AssertionError):
+        ops.check_sampled_idx(ok, 1024)
+    # the argument block of one call checks against that call's key length
+    q = torch.zeros((1, 256, 1, 64), dtype=torch.float16)
+    idx = torch.zeros((1, 256, 1), dtype=torch.int32)
+    lse = torch.zeros((1, 1, 256))
+    with pytest.raises(AssertionError, match="sampled_idx must lie in"):
+        ops._block_attn_args(q, q, q, q, lse, idx, idx, 128, 128, 0.125, False, torch.arange(200, 328))
