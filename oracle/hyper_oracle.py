@@ -23,6 +23,8 @@ block_sampled_attention     reduces to exact_attention for block_size = n, sampl
 add_self_attentions         merging attention over two disjoint key sets == attention over union
 hyper_forward               min_seq_len >= n -> exact causal; one-level split with block = n/2
                             -> exact causal; brute-force row-by-row definition on tiny sizes
+round_dtype (reference      equals the un-rounded result exactly for float64, converges to it as the
+arithmetic mode)            type widens (bf16 > fp16 > fp32), error within the type's rounding bound
 gradients (torch autograd   central finite differences of the same functions in float64; the
 of the functions above)     closed formulas dV = P^T dO, dS = P (dP - D) scale, dQ = dS K,
                             dK = dS^T Q written out per (query, key) pair on tiny sizes
@@ -135,12 +137,32 @@ def gather_rows(x, idx, chunk_size: int = -1):
 
 
 # --------------------------------------------------------------------------- attention
-def exact_attention(q, k, v, scale=None, causal=False, dtype=torch.float64, q_chunk=1024):
+def _lse_dtype(round_dtype):
+    """The reference's kernels store their log-sum-exps in float32 (src/hyper_attn_triton.py:688,
+    src/flash_attn_triton.py:826); float64 stays float64 so that the mode can be checked against the
+    un-rounded functions."""
+    return torch.float64 if round_dtype == torch.float64 else torch.float32
+
+
+def _round_p(p, round_dtype, dtype):
+    """P as the reference's kernels hand it to the P.V product: rounded to the value type
+    (src/hyper_attn_triton.py:135,167 and src/flash_attn_triton.py:233: ``p.to(v.dtype)``)."""
+    return p if round_dtype is None else p.to(round_dtype).to(dtype)
+
+
+def exact_attention(q, k, v, scale=None, causal=False, dtype=torch.float64, q_chunk=1024, round_dtype=None):
     """Exact softmax attention and log-sum-exp.  (b,h,n,d) layout.
 
     Follows src/flash_attn_triton.py:149 (causal loop bound), :171-177 (scores, mask
     ``row >= col``), :236-241 (lse) — the same function without tiling.
     Returns out (b,h,nq,dv) and lse (b,h,nq), both in ``dtype``.
+
+    ``round_dtype`` (torch.float16 / torch.bfloat16) switches on the reference kernels' own
+    roundings: the un-normalised P = exp(s - row max) is rounded to that type before P.V (:233), the
+    row sum is taken over the un-rounded P (:222), and the output is stored in that type (:259-267);
+    out is then returned as a tensor of ``round_dtype`` and lse as float32 (:826).  The reference's
+    running maximum differs from the row maximum by a factor that is not a power of two, so its
+    roundings are these only in distribution, not value by value.
     """
     q = torch.as_tensor(q).to(dtype)
     k = torch.as_tensor(k).to(dtype)
@@ -160,7 +182,14 @@ def exact_attention(q, k, v, scale=None, causal=False, dtype=torch.float64, q_ch
             scores = scores.masked_fill(rows[:, None] < cols[None, :ke], float("-inf"))
         l = torch.logsumexp(scores, dim=-1)
         lse[:, :, s:e] = l
-        out[:, :, s:e] = torch.matmul(torch.exp(scores - l.unsqueeze(-1)), v[:, :, :ke])
+        if round_dtype is None:
+            out[:, :, s:e] = torch.matmul(torch.exp(scores - l.unsqueeze(-1)), v[:, :, :ke])
+        else:
+            m = scores.max(dim=-1, keepdim=True).values
+            p = torch.exp(scores - m)
+            out[:, :, s:e] = torch.matmul(_round_p(p, round_dtype, dtype), v[:, :, :ke]) / p.sum(-1, keepdim=True)
+    if round_dtype is not None:
+        return out.to(round_dtype), lse.to(_lse_dtype(round_dtype))
     return out, lse
 
 
@@ -194,7 +223,7 @@ def block_key_positions(n_q: int, n_k: int, block_size: int, smooth_block: bool)
 
 def block_sampled_attention(q, k, v, q_sort_idx, k_sort_idx, block_size, sample_size=0,
                             scale=None, smooth_block=False, sampled_idx=None,
-                            dtype=torch.float64):
+                            dtype=torch.float64, round_dtype=None):
     """Sorted block-diagonal + fixed-column attention, (b,h,n,d) layout.
 
     Follows src/hyper_attn_triton.py:70-192 (``_fwd_hyper_kernel``): tile ``t`` of 128 sorted
@@ -205,7 +234,9 @@ def block_sampled_attention(q, k, v, q_sort_idx, k_sort_idx, block_size, sample_
     ``arange(sample_size)`` is what the backward kernel (:576-581) and
     unit_tests/test_hyper_attention.py:65-67,200-201 use.  No n/s weighting, no removal of
     columns already in the block.
-    Returns out (b,h,nq,dv) and lse (b,h,nq) in ``dtype``.
+    Returns out (b,h,nq,dv) and lse (b,h,nq) in ``dtype``.  ``round_dtype``: the kernel's own
+    roundings as in exact_attention (P to the value type before both P.V products, :135 and :167;
+    out stored in that type, :189-192; lse float32, :688).
     """
     q = torch.as_tensor(q).to(dtype)
     k = torch.as_tensor(k).to(dtype)
@@ -248,12 +279,21 @@ def block_sampled_attention(q, k, v, q_sort_idx, k_sort_idx, block_size, sample_
             else:
                 scores = s_blk
             l = torch.logsumexp(scores, dim=-1)
-            p = torch.exp(scores - l.unsqueeze(-1))
+            if round_dtype is None:
+                p = torch.exp(scores - l.unsqueeze(-1))
+                norm = 1.0
+            else:
+                p_full = torch.exp(scores - scores.max(dim=-1, keepdim=True).values)
+                norm = p_full.sum(-1, keepdim=True)
+                p = _round_p(p_full, round_dtype, dtype)
             o = torch.matmul(p[..., :width], vg)
             if sample_size > 0:
                 o = o + torch.matmul(p[..., width:], vs)
+            o = o / norm
             out[ib, ih][qi[ib, ih]] = o.view(nq, dv)
             lse[ib, ih][qi[ib, ih]] = l.view(nq)
+    if round_dtype is not None:
+        return out.to(round_dtype), lse.to(_lse_dtype(round_dtype))
     return out, lse
 
 
@@ -271,16 +311,16 @@ def add_self_attentions(attn1, lse1, attn2, lse2):
 
 def forward_no_causal_mask(q, k, v, scale, proj, lsh_num_projs, block_size, sample_size,
                            min_seq_len, smooth_block, sampled_idx=None, dtype=torch.float64,
-                           detach_lse=False):
+                           detach_lse=False, round_dtype=None):
     """Follows hyper_attention.py:103-132.  Returns attn (b,h,n,dv), lse (b,h,n,1)."""
     n_query = q.shape[2]
     if min_seq_len > n_query:  # :109
-        attn, lse = exact_attention(q, k, v, scale, False, dtype)
+        attn, lse = exact_attention(q, k, v, scale, False, dtype, round_dtype=round_dtype)
     else:
         q_idx = stable_bucket_argsort(lsh_hash(q, proj))  # :116
         k_idx = stable_bucket_argsort(lsh_hash(k, proj))  # :117
         attn, lse = block_sampled_attention(q, k, v, q_idx, k_idx, block_size, sample_size,
-                                            scale, smooth_block, sampled_idx, dtype)
+                                            scale, smooth_block, sampled_idx, dtype, round_dtype=round_dtype)
     if detach_lse:
         lse = lse.detach()
     return attn, lse.unsqueeze(-1)
@@ -288,7 +328,7 @@ def forward_no_causal_mask(q, k, v, scale, proj, lsh_num_projs, block_size, samp
 
 def hyper_forward(q, k, v, proj, scale=None, causal=False, lsh_num_projs=8, block_size=256,
                   sample_size=256, min_seq_len=2048, smooth_block=False, sampled_idx=None,
-                  dtype=torch.float64, detach_lse=False):
+                  dtype=torch.float64, detach_lse=False, round_dtype=None):
     """HyperAttention.forward with return_lse=True, (b,h,n,d) layout.
 
     Follows hyper_attention.py:25-101: non-causal dispatch (:48-49), causal leaf (:52-57),
@@ -302,6 +342,11 @@ def hyper_forward(q, k, v, proj, scale=None, causal=False, lsh_num_projs=8, bloc
     gives the gradient the reference's autograd computes: its attention operators return no
     gradient for their log-sum-exp output (src/hyper_attn_triton.py:922-945,
     src/flash_attn_triton.py:1014-1040), so every log-sum-exp entering a merge is a constant there.
+
+    ``round_dtype`` (torch.float16 / torch.bfloat16): the reference's own arithmetic instead of
+    ``dtype`` throughout: the attention operators round P and their outputs to that type (see
+    exact_attention), their log-sum-exps are float32, and the merges then run on tensors of that type,
+    so that add_self_attentions rounds the weight c and every product and sum (src/attn_utils.py:21-23).
     """
     q = torch.as_tensor(q).to(dtype)
     k = torch.as_tensor(k).to(dtype)
@@ -312,11 +357,11 @@ def hyper_forward(q, k, v, proj, scale=None, causal=False, lsh_num_projs=8, bloc
     assert n_query == n_key  # :45
     kw = dict(proj=proj, lsh_num_projs=lsh_num_projs, block_size=block_size,
               sample_size=sample_size, min_seq_len=min_seq_len, smooth_block=smooth_block,
-              sampled_idx=sampled_idx, dtype=dtype, detach_lse=detach_lse)
+              sampled_idx=sampled_idx, dtype=dtype, detach_lse=detach_lse, round_dtype=round_dtype)
     if causal is False:
         return forward_no_causal_mask(q, k, v, scale, **kw)
     if n_key <= min_seq_len:  # :52
-        attn, lse = exact_attention(q, k, v, scale, True, dtype)
+        attn, lse = exact_attention(q, k, v, scale, True, dtype, round_dtype=round_dtype)
         if detach_lse:
             lse = lse.detach()
         return attn, lse.unsqueeze(-1)

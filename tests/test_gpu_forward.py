@@ -23,10 +23,18 @@ def _module(ha, d, dtype, seed, **kw):
     return m, m.lsh.proj_dir[0, 0].cpu()
 
 
-def _oracle(q, k, v, proj, m, causal, scale=None, sampled_idx=None):
+def _oracle(q, k, v, proj, m, causal, scale=None, sampled_idx=None, round_dtype=None):
     return O.hyper_forward(q, k, v, proj, scale=scale, causal=causal, lsh_num_projs=m.lsh_num_projs,
                            block_size=m.block_size, sample_size=m.sample_size, min_seq_len=m.min_seq_len,
-                           smooth_block=m.smooth_block, sampled_idx=sampled_idx)
+                           smooth_block=m.smooth_block, sampled_idx=sampled_idx, round_dtype=round_dtype)
+
+
+def _reference_arithmetic(dtype, *args, **kw):
+    """The oracle's output in the reference's own arithmetic for a bf16 case (None otherwise): what a bf16
+    output is measured against, see _util."""
+    if dtype != torch.bfloat16:
+        return None
+    return _oracle(*args, round_dtype=torch.bfloat16, **kw)[0]
 
 
 # --------------------------------------------------------------------------- non-causal
@@ -58,7 +66,7 @@ def test_non_causal_variants(ha, dtype, d, block, sample, smooth):
     m, proj = _module(ha, d, dtype, 113, block_size=block, sample_size=sample, smooth_block=smooth)
     attn, lse = m(q.cuda(), k.cuda(), v.cuda(), scale=0.1, return_lse=True)
     ro, rl = _oracle(q, k, v, proj, m, False, scale=0.1)
-    assert_close(attn, ro, "attn", dtype)
+    assert_close(attn, ro, "attn", dtype, _reference_arithmetic(dtype, q, k, v, proj, m, False, scale=0.1))
     assert_close(lse, rl, "lse")
 
 
@@ -84,7 +92,7 @@ def test_causal_forward(ha, dtype, d, n, msl, block, sample):
     attn, lse = m(q.cuda(), k.cuda(), v.cuda(), causal=True, return_lse=True)
     ro, rl = _oracle(q, k, v, proj, m, True)
     assert attn.shape == (1, 2, n, d)
-    assert_close(attn, ro, "attn", dtype)
+    assert_close(attn, ro, "attn", dtype, _reference_arithmetic(dtype, q, k, v, proj, m, True))
     if n <= msl:  # the reference returns the exact kernel's padded (b, h, n_rounded) lse here
         assert lse.shape == (1, 2, -(-n // 128) * 128)
         assert_close(lse[:, :, :n], rl.squeeze(-1), "lse")
@@ -221,6 +229,87 @@ def test_full_size_causal_properties(ha):
     assert_close(lse_one, rl, "lse head 5")
 
 
+def _check_sort_properties(ha, buckets):
+    """the permutation of every head is a permutation, sorts its keys, and keeps equal keys in row order"""
+    b, h, n = buckets.shape
+    perm = ha.bucket_argsort(buckets)
+    sorted_b = torch.gather(buckets.long(), 2, perm)
+    assert (sorted_b[:, :, 1:] >= sorted_b[:, :, :-1]).all()
+    ties = sorted_b[:, :, 1:] == sorted_b[:, :, :-1]
+    assert (perm[:, :, 1:][ties] > perm[:, :, :-1][ties]).all()
+    assert torch.equal(torch.sort(perm, dim=2)[0], torch.arange(n, device="cuda").expand(b, h, n))
+
+
+def test_full_size_c4_properties(ha):
+    """benchmark configuration c4 at full size (batch 2, 32 heads, seq 65536, d 128, bf16, block 512, sample
+    512, smooth_block: windows of four 128-key tiles that wrap around at 65536): permutations valid and
+    stable on every head, the fused forward equals the operator-by-operator composition bit for bit, and
+    one head matches the oracle."""
+    b, h, n, d = 2, 32, 65536, 128
+    g = torch.Generator(device="cuda").manual_seed(270)
+    q, k, v = (torch.randn((b, h, n, d), generator=g, device="cuda", dtype=torch.bfloat16) for _ in range(3))
+    m, proj = _module(ha, d, torch.bfloat16, 271, block_size=512, sample_size=512, smooth_block=True)
+    attn, lse = m(q, k, v, return_lse=True)
+    assert attn.shape == (b, h, n, d) and lse.shape == (b, h, n, 1)
+    assert torch.isfinite(attn).all() and torch.isfinite(lse).all()
+    _check_sort_properties(ha, m.lsh.hash(q))
+    _check_sort_properties(ha, m.lsh.hash(k))
+    comp, lse_c = m.forward_no_causal_mask(q, k, v, d ** -0.5)
+    assert torch.equal(comp, attn) and torch.equal(lse_c, lse)
+    del comp, lse_c
+    bi, head = 1, 7
+    sl = (slice(bi, bi + 1), slice(head, head + 1))
+    qc, kc, vc = q[sl].cpu(), k[sl].cpu(), v[sl].cpu()
+    ro, rl = _oracle(qc, kc, vc, proj, m, False)
+    assert_close(attn[sl], ro, "attn batch 1 head 7", torch.bfloat16,
+                 _reference_arithmetic(torch.bfloat16, qc, kc, vc, proj, m, False))
+    assert_close(lse[sl], rl, "lse batch 1 head 7")
+
+
+def _clustered(b, hq, hkv, n, d, seed):
+    """benchmark configuration c5 inputs: keys = 4 x one of 64 unit-norm centroids + N(0, 0.5^2) noise, queries
+    from the same centroids with their own noise, values N(0,1); bf16"""
+    g = _gen(seed)
+    cent = torch.nn.functional.normalize(torch.randn((64, d), generator=g), dim=-1)
+    kc = torch.randint(0, 64, (b, hkv, n), generator=g)
+    qc = torch.randint(0, 64, (b, hq, n), generator=g)
+    k = (4 * cent[kc] + 0.5 * torch.randn((b, hkv, n, d), generator=g)).bfloat16()
+    q = (4 * cent[qc] + 0.5 * torch.randn((b, hq, n, d), generator=g)).bfloat16()
+    v = torch.randn((b, hkv, n, d), generator=g).bfloat16()
+    return q, k, v
+
+
+def test_full_size_c5_properties(ha):
+    """benchmark configuration c5 at full size (32 query heads on 2 KV heads, seq 32768, d 128, bf16, causal,
+    min_seq_len 2048: four levels + leaves; clustered keys, so the buckets are filled unevenly):
+    the native grouped call equals the call on expanded K/V bit for bit, permutations are valid under the
+    skew, and two query heads of different groups match the oracle."""
+    from hyperattention_amd import ops
+    b, hq, hkv, n, d = 1, 32, 2, 32768, 128
+    q, k, v = _clustered(b, hq, hkv, n, d, 290)
+    m, proj = _module(ha, d, torch.bfloat16, 291)
+    qg, kg, vg = q.cuda(), k.cuda(), v.cuda()
+    native, lse_n = ops.hyper_forward(qg, kg, vg, m.lsh.proj_dir, scale=d ** -0.5, causal=True, lsh_num_projs=8,
+                                      block_size=256, sample_size=256, min_seq_len=2048, smooth_block=False)
+    group = hq // hkv
+    attn, lse = m(qg, kg.repeat_interleave(group, dim=1), vg.repeat_interleave(group, dim=1), causal=True,
+                  return_lse=True)
+    assert torch.equal(native, attn) and torch.equal(lse_n.unsqueeze(-1), lse)
+    assert torch.isfinite(attn).all() and torch.isfinite(lse).all()
+    buckets = m.lsh.hash(kg)
+    counts = torch.bincount(buckets[0, 0].long(), minlength=256)
+    assert counts.max() > 1.5 * n / 256, "clustered keys fill the buckets unevenly"
+    _check_sort_properties(ha, buckets)
+    _check_sort_properties(ha, m.lsh.hash(qg))
+    for head in (3, 20):  # query heads of KV group 0 and 1
+        sl = slice(head, head + 1)
+        kv = slice(head // group, head // group + 1)
+        ro, rl = _oracle(q[:, sl], k[:, kv], v[:, kv], proj, m, True)
+        assert_close(attn[:, sl], ro, f"attn head {head}", torch.bfloat16,
+                     _reference_arithmetic(torch.bfloat16, q[:, sl], k[:, kv], v[:, kv], proj, m, True))
+        assert_close(lse[:, sl], rl, f"lse head {head}")
+
+
 def test_grouped_query_heads(ha):
     """benchmark configuration c5 shape family (32 query heads on 2 KV heads, d 128, bf16, causal, clustered
     keys) at reduced length: the expanded-KV module call matches the oracle, and the native grouped
@@ -239,7 +328,7 @@ def test_grouped_query_heads(ha):
     m, proj = _module(ha, d, torch.bfloat16, 191, min_seq_len=1024)
     attn, lse = m(q.cuda(), k_exp.cuda(), v_exp.cuda(), causal=True, return_lse=True)
     ro, rl = _oracle(q, k_exp, v_exp, proj, m, True)
-    assert_close(attn, ro, "attn", torch.bfloat16)
+    assert_close(attn, ro, "attn", torch.bfloat16, _reference_arithmetic(torch.bfloat16, q, k_exp, v_exp, proj, m, True))
     assert_close(lse, rl, "lse")
     native, lse_n = ops.hyper_forward(q.cuda(), k.cuda(), v.cuda(), m.lsh.proj_dir, scale=d ** -0.5, causal=True,
                                       lsh_num_projs=8, block_size=256, sample_size=256, min_seq_len=1024,

@@ -415,3 +415,58 @@ def test_gradient_hyper_forward_true_and_with_constant_log_sum_exps():
     ad = _autograd_directional(detached, (q, k, v), us)
     assert abs(fd - ad) <= 1e-5 * max(1.0, abs(ad))
     assert abs(ad - _autograd_directional(true_loss, (q, k, v), us)) > 1e-6  # the two gradients do differ
+
+
+# --------------------------------------------------------------- the reference's own arithmetic
+def test_reference_arithmetic_mode_is_a_rounding_perturbation():
+    """round_dtype does the same computation with the reference kernels' roundings: float64 "rounding" gives
+    the un-rounded result back, the distance shrinks as the type widens, and stays within a small multiple
+    of the type's unit roundoff (P and the output are each rounded once; the merges add a few more)."""
+    g = torch.Generator().manual_seed(31)
+    q, k, v = (torch.randn((1, 2, 1024, 64), generator=g).bfloat16().double() for _ in range(3))
+    proj = torch.randn((64, 8), generator=g).bfloat16().double()
+    kw = dict(causal=True, min_seq_len=256, block_size=128, sample_size=128)
+    exact, lse = O.hyper_forward(q, k, v, proj, **kw)
+    same, lse_same = O.hyper_forward(q, k, v, proj, round_dtype=torch.float64, **kw)
+    assert same.dtype == torch.float64 and (same - exact).abs().max() < 1e-13 and (lse_same - lse).abs().max() < 1e-12
+    err = {}
+    for dt, eps in ((torch.bfloat16, 2.0 ** -8), (torch.float16, 2.0 ** -11), (torch.float32, 2.0 ** -24)):
+        out, l = O.hyper_forward(q, k, v, proj, round_dtype=dt, **kw)
+        assert out.dtype == dt and l.dtype == torch.float32
+        err[dt] = ((out.double() - exact).norm() / exact.norm()).item()
+        assert err[dt] <= 4 * eps + 1e-6, (dt, err[dt])
+    assert err[torch.bfloat16] > 4 * err[torch.float16] > 16 * err[torch.float32] > 0
+    for fn in (lambda **a: O.exact_attention(q, k, v, None, True, **a),
+               lambda **a: O.block_sampled_attention(q, k, v, O.stable_bucket_argsort(O.lsh_hash(q, proj)),
+                                                     O.stable_bucket_argsort(O.lsh_hash(k, proj)), 256, 128, **a)):
+        e, le = fn()
+        r, lr = fn(round_dtype=torch.float64)
+        assert (r - e).abs().max() < 1e-13 and (lr - le).abs().max() < 1e-12
+        r16, _ = fn(round_dtype=torch.float16)
+        assert 1e-5 < ((r16.double() - e).norm() / e.norm()).item() < 2.0 ** -10
+
+
+def test_bf16_arithmetic_floor():
+    """Why a bf16 output cannot be held to 2e-3: on N(0,1) data the reference kernels' arithmetic (P rounded
+    to bf16 before P.V, output stored in bf16) is more than 2e-3 from the exact result, a second faithful
+    implementation whose P is scaled by another exponent (a running maximum instead of the row maximum) is
+    further than that from the first, and the reference's PyTorch restatement (scores, soft-max and output
+    each rounded to bf16, unit_tests/test_hyper_attention.py:186-205) is further still.  fp16 has room."""
+    n, d = 2048, 64
+    q, k, v = (torch.randn((1, 2, n, d), generator=torch.Generator().manual_seed(s)).bfloat16().double() for s in (11, 12, 13))
+    s = q @ k.transpose(-1, -2) / math.sqrt(d)
+    m = s.max(-1, keepdim=True).values
+    p = torch.exp(s - m)
+    exact = (p @ v) / p.sum(-1, keepdim=True)
+    rel = lambda a, b: ((a - b).norm() / b.norm()).item()
+    for dt, lo, hi in ((torch.bfloat16, 2e-3, 4e-3), (torch.float16, 1e-4, 5e-4)):
+        rnd = lambda x: x.float().to(dt).double()
+        kernel = rnd((rnd(p) @ v) / p.sum(-1, keepdim=True))
+        p2 = torch.exp(s - m + 0.37)
+        other = rnd((rnd(p2) @ v) / p2.sum(-1, keepdim=True))
+        torch_path = rnd(rnd(torch.softmax(rnd(s), -1)) @ v)
+        assert lo < rel(kernel, exact) < hi
+        assert rel(kernel, exact) < rel(other, kernel) < 1.6 * rel(kernel, exact)
+        assert rel(torch_path, exact) > 1.5 * rel(kernel, exact)
+        out, _ = O.exact_attention(q, k, v, round_dtype=dt)
+        assert torch.equal(out.double(), kernel)
