@@ -16,13 +16,23 @@ Besides the whole-forward time the line carries
   exact_flash   our exact MFMA flash-attention forward at the same shape (the 20x comparison);
   backward      forward under autograd + backward of the module at the same shape, and of the exact
                 attention, as the reference's sweep script times them (not part of `value`);
-  cpu_baseline  the CPU oracle (float32, torch) on a bounded sample of the same workload.
+  cpu_baseline  the CPU oracle (float32, torch) on a bounded sample of the same workload;
+  cpu_baseline_c1  the CPU oracle on benchmark configuration c1 exactly (batch 1, 4 heads, seq 4096, d 64, fp32,
+                non-causal): all host threads and one thread, 3 warm-ups, 10 repetitions, median; with the
+                GPU forward on the same inputs (fp16) beside it;
+  sustained     the same forward repeated for about 1.5 s with board power and shader clock sampled from the
+                driver's sysfs files: the board's power limit, not the kernels' issue rate, is what bounds
+                them once a loop runs for longer than a few milliseconds.
 """
 import argparse
 import ctypes
+import glob
 import json
 import os
+import re
+import statistics
 import sys
+import threading
 import time
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
@@ -31,12 +41,24 @@ sys.path.insert(0, ROOT)
 METRIC = "HyperAttention fwd ms + MFMA util at seq 131k, 32 heads, d=64, fp16 causal"
 MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense fp16/bf16
 HBM_PEAK_GBS = 8000.0
-# HBM bytes per launch of the gathered attention kernel, measured with rocprofv3 --pmc (see the
-# summary of that run under profiles/); only the workload that was measured has a figure
-MEASURED_TRAFFIC_BYTES = {"c3": 1.3903e9}
+
+
+def measured_traffic(workload):
+    """HBM bytes per launch of the gathered attention kernel from the counter summary committed for this
+    workload (profiles/hbm_traffic_<workload>_pmc.md, line "traffic_bytes_per_launch = ..."), and the file's
+    name; (None, None) when the workload has no summary."""
+    path = os.path.join(ROOT, "profiles", f"hbm_traffic_{workload}_pmc.md")
+    try:
+        m = re.search(r"traffic_bytes_per_launch\s*=\s*([0-9.eE+]+)", open(path).read())
+    except OSError:
+        return None, None
+    return (float(m.group(1)), os.path.relpath(path, ROOT)) if m else (None, None)
+
 
 WORKLOADS = {
     # name: batch, q heads, kv heads, n, d, dtype, causal, block, sample, min_seq_len, smooth
+    "c1": dict(batch=1, heads=4, kv_heads=4, n=4096, d=64, dtype="fp16", causal=False, block=256, sample=256,
+               min_seq_len=2048, smooth=False),
     "c2": dict(batch=1, heads=32, kv_heads=32, n=32768, d=64, dtype="fp16", causal=False, block=256, sample=256,
                min_seq_len=2048, smooth=False),
     "c3": dict(batch=1, heads=32, kv_heads=32, n=131072, d=64, dtype="fp16", causal=True, block=256, sample=256,
@@ -90,7 +112,8 @@ def time_events(fn, reps, torch):
 
 
 def cpu_baseline(w, seed):
-    """The CPU oracle in float32 on a bounded sample: one query head (and its kv head) at full length."""
+    """The CPU oracle in float32 on a bounded sample: one query head (and its kv head) at full length, one
+    warm-up and three timed runs (median)."""
     import torch
     from oracle import hyper_oracle as O
     g = torch.Generator().manual_seed(seed)
@@ -104,17 +127,147 @@ def cpu_baseline(w, seed):
     q, k, v = (torch.randn((1, heads_sampled, n_sample, w["d"]), generator=g).to(tdt).float() for _ in range(3))
     proj = torch.randn((w["d"], 8), generator=g).to(tdt).float()
     threads = torch.get_num_threads()
-    t0 = time.perf_counter()
-    O.hyper_forward(q, k, v, proj, causal=w["causal"], block_size=w["block"], sample_size=w["sample"],
-                    min_seq_len=w["min_seq_len"], smooth_block=w["smooth"], dtype=torch.float32)
-    dt = time.perf_counter() - t0
+
+    def run():
+        t0 = time.perf_counter()
+        O.hyper_forward(q, k, v, proj, causal=w["causal"], block_size=w["block"], sample_size=w["sample"],
+                        min_seq_len=w["min_seq_len"], smooth_block=w["smooth"], dtype=torch.float32)
+        return time.perf_counter() - t0
+
+    run()
+    times = sorted(run() for _ in range(3))
+    dt = times[1]
     scale = w["batch"] * w["heads"] / heads_sampled * (n / n_sample)
     return {
         "value": round(dt * 1e3 * scale, 1), "unit": "ms", "cores": threads, "kind": "port",
         "sample": f"CPU oracle (torch float32, {threads} threads) on {heads_sampled} of {w['batch'] * w['heads']} "
-                  f"heads at seq {n_sample}: {dt:.2f} s measured, scaled x{scale:g} to the full workload",
-        "measured_s": round(dt, 3),
+                  f"heads at seq {n_sample}: median of 3 runs after a warm-up {dt:.2f} s, scaled x{scale:g} to the "
+                  f"full workload",
+        "measured_s": round(dt, 3), "runs_s": [round(x, 3) for x in times],
     }
+
+
+def cpu_baseline_c1(seed):
+    """Benchmark configuration c1 exactly (batch 1, 4 heads, seq 4096, d 64, fp32, non-causal, 8 projections, block 256,
+    sample 256, min_seq_len 2048): the CPU oracle with all host threads and with one, 3 warm-ups, 10
+    repetitions each (median, min, max), exact attention on the CPU for context, and the GPU forward on
+    the same inputs cast to fp16."""
+    import torch
+    from oracle import hyper_oracle as O
+    from hyperattention_amd import HyperAttention
+    g = torch.Generator().manual_seed(seed)
+    q, k, v = (torch.randn((1, 4, 4096, 64), generator=g) for _ in range(3))
+    proj = torch.randn((64, 8), generator=g)
+    all_threads = torch.get_num_threads()
+
+    def timed(fn, warm=3, reps=10):
+        for _ in range(warm):
+            fn()
+        ts = []
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            fn()
+            ts.append((time.perf_counter() - t0) * 1e3)
+        return {"median_ms": round(statistics.median(ts), 2), "min_ms": round(min(ts), 2), "max_ms": round(max(ts), 2)}
+
+    hyper = lambda: O.hyper_forward(q, k, v, proj, causal=False, block_size=256, sample_size=256, min_seq_len=2048,
+                                    dtype=torch.float32)
+    exact = lambda: O.exact_attention(q, k, v, dtype=torch.float32)
+    res = {"config": "c1: batch 1, 4 heads, seq 4096, d 64, fp32, non-causal, block 256, sample 256, 8 projections",
+           "kind": "port", "host_cores": os.cpu_count()}
+    res[f"threads_{all_threads}"] = timed(hyper)
+    res[f"exact_attention_threads_{all_threads}"] = timed(exact, 1, 3)
+    torch.set_num_threads(1)
+    try:
+        res["threads_1"] = timed(hyper)
+    finally:
+        torch.set_num_threads(all_threads)
+    m = HyperAttention(input_dim=64, proj_dir=proj).to(device="cuda", dtype=torch.float16)
+    qg, kg, vg = (x.half().cuda() for x in (q, k, v))
+    ms = time_events(lambda: m(qg, kg, vg), 50, torch)
+    res["gpu_fp16_ms"] = round(ms, 4)
+    return res
+
+
+class PowerSampler:
+    """Board power (W) and shader clock (MHz) read from the amdgpu sysfs files of the first card every 20 ms
+    on a background thread; empty when the files are not there or not readable."""
+
+    def __init__(self):
+        hw = sorted(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*"))
+        self.hwmon = hw[0] if hw else None
+        self.samples = []
+        self._stop = threading.Event()
+        self._thread = None
+
+    def _read(self):
+        try:
+            for name in ("power1_input", "power1_average"):
+                path = os.path.join(self.hwmon, name)
+                if os.path.exists(path):
+                    watts = int(open(path).read()) / 1e6
+                    break
+            else:
+                return None
+            sclk = None
+            for line in open(os.path.join(os.path.dirname(os.path.dirname(self.hwmon)), "pp_dpm_sclk")):
+                if "*" in line:
+                    sclk = float(re.search(r"(\d+)\s*[Mm]hz", line).group(1))
+            return watts, sclk
+        except (OSError, ValueError, AttributeError):
+            return None
+
+    def cap_watts(self):
+        try:
+            return int(open(os.path.join(self.hwmon, "power1_cap")).read()) / 1e6
+        except (OSError, ValueError, TypeError):
+            return None
+
+    def __enter__(self):
+        if self.hwmon:
+            def loop():
+                while not self._stop.is_set():
+                    r = self._read()
+                    if r:
+                        self.samples.append(r)
+                    time.sleep(0.02)
+            self._thread = threading.Thread(target=loop, daemon=True)
+            self._thread.start()
+        return self
+
+    def __exit__(self, *exc):
+        self._stop.set()
+        if self._thread:
+            self._thread.join()
+
+    def summary(self, skip_s=0.3):
+        rows = self.samples[int(skip_s / 0.02):]  # the first samples still see the clock ramping
+        if not rows:
+            return {"power_W": None, "sclk_MHz": None, "samples": 0}
+        clocks = [c for _, c in rows if c]
+        return {"power_W": round(statistics.mean(p for p, _ in rows), 1),
+                "sclk_MHz": round(statistics.mean(clocks), 0) if clocks else None, "samples": len(rows)}
+
+
+def sustained(fn, seconds, torch):
+    """fn repeated for about `seconds`: ms per call over the whole loop, average board power and clock"""
+    fn()
+    torch.cuda.synchronize()
+    n = 0
+    with PowerSampler() as ps:
+        t0 = time.perf_counter()
+        while time.perf_counter() - t0 < seconds:
+            for _ in range(20):
+                fn()
+            torch.cuda.synchronize()
+            n += 20
+        dt = time.perf_counter() - t0
+    out = {"ms": round(dt * 1e3 / n, 4), "calls": n, "seconds": round(dt, 2)}
+    out.update(ps.summary())
+    out["power_cap_W"] = ps.cap_watts()
+    if out["power_W"]:
+        out["energy_J_per_call"] = round(out["power_W"] * dt / n, 4)
+    return out
 
 
 def main():
@@ -124,6 +277,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-sustained", action="store_true", help="skip the 2.5 s of sustained loops with power sampling")
     ap.add_argument("--no-exact", action="store_true", help="skip timing the exact flash kernel at the same shape")
     ap.add_argument("--no-backward", action="store_true", help="skip timing forward + backward under autograd")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -237,7 +391,8 @@ def main():
         a.block_size, a.sample_size = w["block"], w["sample"]
         a.smooth_block, a.accumulate = int(w["smooth"]), int(w["causal"])
         st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
-        blk_ms.append(time_events(lambda: _lib.check(L.ha_block_attn_fwd(ctypes.byref(a), st)), reps, torch))
+        blk_launch = lambda a=a, st=st: _lib.check(L.ha_block_attn_fwd(ctypes.byref(a), st))
+        blk_ms.append(time_events(blk_launch, reps, torch))
 
     blk_avg = sum(blk_ms) / len(blk_ms)
     blk_flops = per_level[0]
@@ -245,18 +400,29 @@ def main():
     # lse, the sorted index arrays, and (causal: resumed partial result) the previous rows and lse; the
     # sampled rows are shared by all query blocks of a head
     lvl_q = b * h * (n // 2 if w["causal"] else n)
-    lvl_k = lvl_q  # one key block per query block
+    lvl_k = lvl_q * hk // h  # one key block per query block; the query heads of a KV group share its rows
     row_b = d * 2
     blk_bytes = lvl_q * row_b + 2 * lvl_k * row_b + lvl_q * (row_b + 4) + (lvl_q + lvl_k) * 4
     if w["causal"]:
         blk_bytes += lvl_q * (row_b + 4)
     achieved = blk_flops / blk_avg / 1e9  # TFLOP/s
-    roofline = {"kernel": "attn_fwd_kernel<gather> (block-diagonal + sampled attention)", "bound": "mfma",
-                "achieved": round(achieved, 1), "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
-                "frac": round(achieved / MFMA_PEAK_TFLOPS, 4),
-                # HBM bytes per launch from the FETCH_SIZE / WRITE_SIZE counter runs of this workload
-                # (fetch counter x 2.000, write counter x 1.000, factors from a plain copy of known size)
-                "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+    achieved_gbs = blk_bytes / blk_avg / 1e6
+    intensity = blk_flops / blk_bytes
+    ridge = MFMA_PEAK_TFLOPS * 1e12 / (HBM_PEAK_GBS * 1e9)
+    bound = "hbm" if intensity < ridge else "mfma"
+    traffic, traffic_source = measured_traffic(args.workload)
+    roofline = {"kernel": "attn_fwd_kernel<gather> (block-diagonal + sampled attention)",
+                # which peak the kernel's algorithmic intensity puts it under (ridge = MFMA peak / HBM peak)
+                "bound": bound, "intensity_flop_per_byte": round(intensity, 1), "ridge_flop_per_byte": round(ridge, 1),
+                "achieved": round(achieved_gbs if bound == "hbm" else achieved, 1),
+                "peak": HBM_PEAK_GBS if bound == "hbm" else MFMA_PEAK_TFLOPS,
+                "unit": "GB/s" if bound == "hbm" else "TFLOP/s",
+                "frac": round(achieved_gbs / HBM_PEAK_GBS if bound == "hbm" else achieved / MFMA_PEAK_TFLOPS, 4),
+                "frac_mfma": round(achieved / MFMA_PEAK_TFLOPS, 4), "achieved_TFLOPs": round(achieved, 1),
+                "frac_hbm": round(achieved_gbs / HBM_PEAK_GBS, 4), "achieved_GBs": round(achieved_gbs, 1),
+                # HBM bytes per launch from the FETCH_SIZE / WRITE_SIZE counter runs of this workload (fetch
+                # counter x 2.000, write counter x 1.000, factors from a plain copy of known size)
+                "traffic": traffic, "traffic_source": traffic_source,
                 "algorithmic_bytes": blk_bytes,
                 "flops_per_launch": blk_flops, "avg_launch_ms": round(blk_avg, 4),
                 "launch_ms_by_level": [round(x, 4) for x in blk_ms]}
@@ -283,6 +449,22 @@ def main():
         kernels["flash leaves (exact causal)"] = {"ms": round(ms, 4), "bound": "mfma", "flops": leaf_flops,
                                                   "achieved_TFLOPs": round(leaf_flops / ms / 1e9, 1),
                                                   "frac": round(leaf_flops / ms / 1e9 / MFMA_PEAK_TFLOPS, 4)}
+
+    # the operator-level kernels that the one-call forward does not launch (row gather of the reference's
+    # `indexing`, merge of two partial attentions), at this workload's tensor size
+    perm = torch.argsort(bq.view(b, h, n), dim=2)
+    ms = time_events(lambda: ops.indexing(q, perm), reps, torch)
+    g_bytes = rows_q * (2 * d * 2 + 8)
+    kernels["gather_rows (indexing, bucket-sorted order)"] = {
+        "ms": round(ms, 4), "bound": "hbm", "bytes": g_bytes, "achieved_GBs": round(g_bytes / ms / 1e6, 1),
+        "frac": round(g_bytes / ms / 1e6 / HBM_PEAK_GBS, 4)}
+    lse4 = lse.unsqueeze(-1)
+    ms = time_events(lambda: ops.add_self_attentions(q, lse4, out, lse4), reps, torch)
+    m_bytes = rows_q * (3 * d * 2 + 12)
+    kernels["lse_merge (add_self_attentions)"] = {
+        "ms": round(ms, 4), "bound": "hbm", "bytes": m_bytes, "achieved_GBs": round(m_bytes / ms / 1e6, 1),
+        "frac": round(m_bytes / ms / 1e6 / HBM_PEAK_GBS, 4)}
+    del perm
 
     exact = None
     if not args.no_exact and hk == h:
@@ -327,8 +509,23 @@ def main():
         "exact_equivalent_TFLOPs": round(exact_flops / ms_per_step / 1e9, 1),
         "roofline": roofline, "kernels": kernels, "exact_flash": exact, "backward": backward,
     }
+    if not args.no_sustained:
+        # every kernel of the path (and a plain copy, and the exact kernel) on its own for about a second: the
+        # board draws its power limit under each of them, at a clock that depends on what the kernel does
+        sus = {"forward": sustained(step, 1.5, torch), "roofline_kernel": sustained(blk_launch, 1.0, torch)}
+        sus["lsh_hash"] = sustained(lambda: ops.lsh_hash(q, proj2), 0.7, torch)
+        if leaf is not None:
+            sus["leaves"] = sustained(leaves, 0.7, torch)
+        dst = torch.empty_like(q)
+        sus["copy_of_q"] = sustained(lambda: dst.copy_(q), 0.7, torch)
+        sus["copy_of_q"]["bytes_moved"] = 2 * q.numel() * q.element_size()
+        del dst
+        if not args.no_exact and hk == h:
+            sus["exact_flash"] = sustained(lambda: ops.flash_attn_func(qt, kt, vt, None, w["causal"], scale), 1.0, torch)
+        result["sustained"] = sus
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(w, seed)
+        result["cpu_baseline_c1"] = cpu_baseline_c1(seed)
     print(json.dumps(result))
 
 
