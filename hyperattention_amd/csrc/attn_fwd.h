@@ -36,7 +36,7 @@ struct ha_attn_kernel_params {
   float scale_log2;   // softmax scale * log2(e)
   // the divisors of the workgroup -> (head, segment, tile) decomposition as multiply-and-shift
   // constants (filled by ha_attn_launch): the kernel never divides
-  ha_divisor div_qtiles, div_segs, div_heads, div_kv_group, div_block_tiles;
+  ha_divisor div_qtiles, div_segs, div_heads, div_kv_heads, div_kv_group, div_block_tiles;
 };
 
 int ha_attn_launch(const ha_attn_kernel_params& p, int d, int dtype, bool gather, bool causal, hipStream_t stream);

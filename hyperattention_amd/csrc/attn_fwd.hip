@@ -250,16 +250,21 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
   const int hi = lane >> 5, col = lane & 31;
 
   // ---- which (virtual) head and query tile -----------------------------------------------------
+  // Workgroup number = (((batch, kv head), segment), tile, query head inside the kv group), the last one
+  // fastest: the query heads that share a kv head work on the same tile side by side, on one XCD, so that the
+  // K and V rows of the tile (the same for all of them) come from HBM once and from L2 after that.
   const int wg = xcd_contiguous_id(blockIdx.x, gridDim.x);
   const int qtiles = (p.n_q + WG_QUERIES - 1) / WG_QUERIES;
-  const int vhead = fast_div(wg, p.div_qtiles);
+  const int wg_tile = fast_div(wg, p.div_kv_group);
+  const int hg = wg - wg_tile * p.kv_group;
+  const int vseq = fast_div(wg_tile, p.div_qtiles);
   // causal: the tiles with the most keys go first, so that the last workgroups of the grid are short
-  const int qt_fwd = wg - vhead * qtiles;
+  const int qt_fwd = wg_tile - vseq * qtiles;
   const int qt = CAUSAL ? qtiles - 1 - qt_fwd : qt_fwd;
-  const int bh = fast_div(vhead, p.div_segs);
-  const int seg = vhead - bh * p.segs;
-  const int b = fast_div(bh, p.div_heads), h = bh - b * p.heads;
-  const int hk = fast_div(h, p.div_kv_group);
+  const int bhk = fast_div(vseq, p.div_segs);
+  const int seg = vseq - bhk * p.segs;
+  const int b = fast_div(bhk, p.div_kv_heads), hk = bhk - b * fast_div(p.heads, p.div_kv_group);
+  const int h = hk * p.kv_group + hg;
 
   // ---- row numbers of the queries: the first thing the workgroup has to wait for, so they are asked
   // for before the rest of the set-up (sorted query positions of this head: entries of 4 or 8 bytes,
@@ -736,6 +741,7 @@ int ha_attn_launch(const ha_attn_kernel_params& params, int d, int dtype, bool g
   p.div_qtiles = make_divisor(qtiles);
   p.div_segs = make_divisor(p.segs);
   p.div_heads = make_divisor(p.heads);
+  p.div_kv_heads = make_divisor(p.heads / p.kv_group);
   p.div_kv_group = make_divisor(p.kv_group);
   p.div_block_tiles = make_divisor(p.block_tiles);
   const int64_t grid = qtiles * p.batch * p.heads * p.segs;
