@@ -431,6 +431,14 @@ def main():
     kernels["bucket_argsort(one launch per level and side)"] = {"ms": round(sort_total, 4), "bound": "hbm", "bytes": sort_elems * 8,
                                              "achieved_GBs": round(sort_elems * 8 / sort_total / 1e6, 1),
                                              "frac": round(sort_elems * 8 / sort_total / 1e6 / HBM_PEAK_GBS, 4)}
+    # the first stage of the one-call forward: bucket ids of q and k in one launch, one ranking of the rows,
+    # one placement launch for all levels.  Algorithmic bytes: q and k read once, the orders written once.
+    ms = time_events(lambda: ops.forward_sort(q, k, proj2, causal=w["causal"], lsh_num_projs=8,
+                                              min_seq_len=w["min_seq_len"]), reps, torch)
+    stage_bytes = (rows_q + rows_k) * d * 2 + sort_elems * 4
+    kernels["ha_forward_sort (hash q+k, rank, place: all levels)"] = {
+        "ms": round(ms, 4), "bound": "hbm", "bytes": stage_bytes, "achieved_GBs": round(stage_bytes / ms / 1e6, 1),
+        "frac": round(stage_bytes / ms / 1e6 / HBM_PEAK_GBS, 4)}
     if leaf is not None:
         def leaves():
             t = _lib.AttnOperands()

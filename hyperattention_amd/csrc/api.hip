@@ -6,6 +6,8 @@
 #include "bucket_sort.h"
 
 #include <math.h>
+#include <string.h>
+#include <algorithm>
 
 char* ha_error_buffer() {
   static thread_local char buf[512] = {0};
@@ -164,30 +166,62 @@ int make_plan(const ha_forward_args& a, Plan& pl) {
 }
 
 struct Workspace {
-  int64_t buckets_q, buckets_k;        // byte offsets
+  bool units;                          // one ranking for all levels (byte-sized ids), else a sort per level
+  ha_unit_grid grid;
+  int64_t buckets_q, buckets_k;        // byte offsets; one byte per id with `units`, else int32
+  int64_t sorted_q, sorted_k;          // with `units`: per-unit orders
+  int64_t unit_hist_q, unit_hist_k;    // with `units`: per-unit bucket counts
   int64_t qidx[48], kidx[48];          // per hyper level (index 0 for the non-causal case)
-  int64_t hist_q[48], hist_k[48];
+  int64_t hist_q[48], hist_k[48];      // without `units`: per-level chunk histograms
+  int64_t tmp_q[48][2], tmp_k[48][2];  // without `units`, more than 256 buckets: orders between the two passes
   int64_t total;
 };
 
+// A placement workgroup adds up the bucket counts of all units of its segment and moves one unit's rows: the
+// longest hashed segment may span this many units before the per-level sort is the better choice.
+inline int64_t max_units_per_segment(int unit) { return std::max<int64_t>(64, unit / 4); }
+
 void layout_workspace(const ha_forward_args& a, const Plan& pl, Workspace& w) {
   int64_t off = 0;
-  w.buckets_q = w.buckets_k = 0;
-  if (pl.any_hyper) {
-    w.buckets_q = off; off += align256(a.batch * a.heads * a.n * 4);
-    w.buckets_k = off; off += align256(a.batch * a.kv_heads * a.n * 4);
-  }
+  memset(&w, 0, sizeof(w));
   const int nlev = a.causal ? pl.levels : 1;
+  if (pl.any_hyper) {
+    ha_unit_grid& g = w.grid;
+    g.n = a.n;
+    g.granule = a.causal ? pl.len[pl.levels] : a.n;
+    g.units_per_granule = (int)((g.granule + HA_SORT_CHUNK - 1) / HA_SORT_CHUNK);
+    g.unit = (int)std::min<int64_t>(g.granule, HA_SORT_CHUNK);
+    g.units_per_seq = (int)(a.n / g.granule) * g.units_per_granule;
+    int64_t longest = 0;
+    for (int j = 0; j < nlev; ++j)
+      if (pl.level_hyper[j]) longest = std::max<int64_t>(longest, a.causal ? pl.len[j] / 2 : a.n);
+    w.units = a.lsh_num_projs <= 8 && longest / g.granule * g.units_per_granule <= max_units_per_segment(g.unit) &&
+              a.n % g.granule == 0;
+    const int64_t id_bytes = w.units ? 1 : 4;
+    w.buckets_q = off; off += align256(a.batch * a.heads * a.n * id_bytes);
+    w.buckets_k = off; off += align256(a.batch * a.kv_heads * a.n * id_bytes);
+    if (w.units) {
+      w.sorted_q = off; off += align256(a.batch * a.heads * a.n * 4);
+      w.sorted_k = off; off += align256(a.batch * a.kv_heads * a.n * 4);
+      w.unit_hist_q = off; off += align256(a.batch * a.heads * g.units_per_seq * 256 * 4);
+      w.unit_hist_k = off; off += align256(a.batch * a.kv_heads * g.units_per_seq * 256 * 4);
+    }
+  }
   for (int j = 0; j < nlev; ++j) {
-    w.qidx[j] = w.kidx[j] = w.hist_q[j] = w.hist_k[j] = 0;
     if (!pl.level_hyper[j]) continue;
     const int64_t seg_len = a.causal ? pl.len[j] / 2 : a.n;
     const int64_t segs = a.causal ? (1ll << j) : 1;
     const int64_t chunks = (seg_len + HA_SORT_CHUNK - 1) / HA_SORT_CHUNK;
     w.qidx[j] = off; off += align256(a.batch * a.heads * segs * seg_len * 4);
     w.kidx[j] = off; off += align256(a.batch * a.kv_heads * segs * seg_len * 4);
+    if (w.units) continue;
     w.hist_q[j] = off; off += align256(a.batch * a.heads * segs * chunks * 256 * 4);
     w.hist_k[j] = off; off += align256(a.batch * a.kv_heads * segs * chunks * 256 * 4);
+    if (a.lsh_num_projs > 8)
+      for (int t = 0; t < 2; ++t) {
+        w.tmp_q[j][t] = off; off += align256(a.batch * a.heads * segs * seg_len * 4);
+        w.tmp_k[j][t] = off; off += align256(a.batch * a.kv_heads * segs * seg_len * 4);
+      }
   }
   w.total = off > 0 ? off : 256;
 }
@@ -205,6 +239,136 @@ int check_forward(const ha_forward_args& a) {
   HA_REQUIRE(a.scale > 0.f && isfinite(a.scale), HA_ERR_SHAPE, "ha_forward: softmax scale must be positive and finite");
   HA_REQUIRE(a.block_size > 0 && a.sample_size >= 0 && a.sample_size % 128 == 0 && a.min_seq_len >= 0, HA_ERR_SHAPE,
              "ha_forward: block_size > 0 and sample_size a non-negative multiple of 128 required");
+  return HA_OK;
+}
+
+// (batch, heads, n, d) operands of the whole forward pass: contiguous unless strides are given
+void forward_operands(const ha_forward_args& a, ha_attn_operands& t) {
+  t.q = a.q; t.k = a.k; t.v = a.v; t.out = a.out; t.lse = a.lse;
+  t.batch = a.batch; t.heads = a.heads; t.d = a.d; t.dv = a.dv;
+  t.q_stride_b = a.heads * a.n * a.d; t.q_stride_h = a.n * a.d; t.q_stride_n = a.d;
+  t.k_stride_b = a.kv_heads * a.n * a.d; t.k_stride_h = a.n * a.d; t.k_stride_n = a.d;
+  t.v_stride_b = a.kv_heads * a.n * a.dv; t.v_stride_h = a.n * a.dv; t.v_stride_n = a.dv;
+  t.o_stride_b = a.heads * a.n * a.dv; t.o_stride_h = a.n * a.dv; t.o_stride_n = a.dv;
+  if (a.q_stride_b || a.q_stride_h || a.q_stride_n) {
+    t.q_stride_b = a.q_stride_b; t.q_stride_h = a.q_stride_h; t.q_stride_n = a.q_stride_n;
+  }
+  if (a.k_stride_b || a.k_stride_h || a.k_stride_n) {
+    t.k_stride_b = a.k_stride_b; t.k_stride_h = a.k_stride_h; t.k_stride_n = a.k_stride_n;
+  }
+  if (a.v_stride_b || a.v_stride_h || a.v_stride_n) {
+    t.v_stride_b = a.v_stride_b; t.v_stride_h = a.v_stride_h; t.v_stride_n = a.v_stride_n;
+  }
+  t.lse_stride_b = a.heads * a.n; t.lse_stride_h = a.n;
+  t.kv_group = a.heads / a.kv_heads;
+  t.scale = a.scale;
+  t.dtype = a.dtype;
+}
+
+// Bucket ids of q and k, then the stable bucket order of the query and key segment of every hashed level
+// (hyper_attention.py:112-117 at every level of the recursion), as int32 rows local to the segment.
+int hash_and_sort(const ha_forward_args& a, const Plan& pl, const Workspace& w, const ha_attn_operands& t,
+                  hipStream_t stream) {
+  unsigned char* ws = (unsigned char*)a.workspace;
+  const int nlev = a.causal ? pl.levels : 1;
+  int st;
+  if (w.units) {
+    const int64_t qs[3] = {t.q_stride_b, t.q_stride_h, t.q_stride_n}, ks[3] = {t.k_stride_b, t.k_stride_h, t.k_stride_n};
+    st = ha_hash_pair_u8(a.q, a.k, a.proj, ws + w.buckets_q, ws + w.buckets_k, a.batch, a.heads, a.kv_heads, a.n, a.d,
+                         a.lsh_num_projs, qs, ks, a.dtype, stream);
+    if (st != HA_OK) return st;
+    const uint8_t* ids[2] = {ws + w.buckets_q, ws + w.buckets_k};
+    uint32_t* sorted[2] = {(uint32_t*)(ws + w.sorted_q), (uint32_t*)(ws + w.sorted_k)};
+    uint32_t* hist[2] = {(uint32_t*)(ws + w.unit_hist_q), (uint32_t*)(ws + w.unit_hist_k)};
+    const int64_t seqs[2] = {a.batch * a.heads, a.batch * a.kv_heads};
+    st = ha_rank_units(ids, sorted, hist, seqs, w.grid, stream);
+    if (st != HA_OK) return st;
+    ha_place_jobs jobs;
+    jobs.num_jobs = 0;
+    jobs.grid = w.grid;
+    int64_t blocks = 0;
+    for (int j = 0; j < nlev; ++j) {
+      if (!pl.level_hyper[j]) continue;
+      const int64_t seg_len = a.causal ? pl.len[j] / 2 : a.n;
+      const int64_t segs = a.causal ? (1ll << j) : 1;
+      for (int side = 0; side < 2; ++side) {
+        HA_REQUIRE(jobs.num_jobs < HA_SORT_MAX_JOBS, HA_ERR_SHAPE, "ha_forward: too many sort jobs");
+        ha_place_job& job = jobs.job[jobs.num_jobs++];
+        job.sorted = sorted[side];
+        job.hist = hist[side];
+        job.out = (int32_t*)(ws + (side == 0 ? w.qidx[j] : w.kidx[j]));
+        job.seg_stride = a.causal ? pl.len[j] : a.n;
+        job.seg_offset = (a.causal && side == 0) ? seg_len : 0;  // queries: second halves, keys: first halves
+        job.seg_len = (int)seg_len;
+        job.segs_per_seq = (int)segs;
+        job.units_per_seg = (int)(seg_len / w.grid.granule) * w.grid.units_per_granule;
+        job.first_block = (int)blocks;
+        blocks += seqs[side] * segs * job.units_per_seg;
+        HA_REQUIRE(blocks < (1ll << 30), HA_ERR_SHAPE, "ha_forward: too many sort units");
+      }
+    }
+    return ha_place_units(jobs, (int)blocks, stream);
+  }
+
+  int32_t* bq = (int32_t*)(ws + w.buckets_q);
+  int32_t* bk = (int32_t*)(ws + w.buckets_k);
+  st = ha_lsh_hash(a.q, a.proj, bq, a.batch, a.heads, a.n, a.d, a.lsh_num_projs, t.q_stride_b, t.q_stride_h,
+                   t.q_stride_n, 0, 0, a.dtype, stream);
+  if (st != HA_OK) return st;
+  st = ha_lsh_hash(a.k, a.proj, bk, a.batch, a.kv_heads, a.n, a.d, a.lsh_num_projs, t.k_stride_b, t.k_stride_h,
+                   t.k_stride_n, 0, 0, a.dtype, stream);
+  if (st != HA_OK) return st;
+  // all segmented sorts of all levels in one batch of launches per 8-bit digit
+  const int passes = a.lsh_num_projs > 8 ? 2 : 1;
+  for (int pass = 0; pass < passes; ++pass) {
+    const bool last = pass == passes - 1;
+    ha_sort_jobs jobs;
+    jobs.num_jobs = 0;
+    jobs.shift = 8 * pass;
+    jobs.idx64 = 0;
+    int blocks = 0, segments = 0;
+    bool multi = false;
+    for (int j = 0; j < nlev; ++j) {
+      if (!pl.level_hyper[j]) continue;
+      const int64_t seg_len = a.causal ? pl.len[j] / 2 : a.n;
+      const int64_t segs = a.causal ? (1ll << j) : 1;
+      const int64_t stride = a.causal ? pl.len[j] : a.n;
+      const int64_t chunks = (seg_len + HA_SORT_CHUNK - 1) / HA_SORT_CHUNK;
+      for (int side = 0; side < 2; ++side) {
+        HA_REQUIRE(jobs.num_jobs < HA_SORT_MAX_JOBS, HA_ERR_SHAPE, "ha_forward: too many sort jobs");
+        ha_sort_job& job = jobs.job[jobs.num_jobs++];
+        const int64_t nseg = a.batch * (side == 0 ? a.heads : a.kv_heads) * segs;
+        const int64_t* tmp = side == 0 ? w.tmp_q[j] : w.tmp_k[j];
+        job.keys = side == 0 ? bq : bk;
+        job.prev = pass == 0 ? nullptr : (const int32_t*)(ws + tmp[(pass - 1) & 1]);
+        job.out = last ? ws + (side == 0 ? w.qidx[j] : w.kidx[j]) : ws + tmp[pass & 1];
+        job.hist = (uint32_t*)(ws + (side == 0 ? w.hist_q[j] : w.hist_k[j]));
+        job.seg_stride = stride;
+        job.seg_offset = (a.causal && side == 0) ? seg_len : 0;  // queries: second halves, keys: first halves
+        job.seg_len = (int)seg_len;
+        job.num_segments = (int)nseg;
+        job.chunks_per_seg = (int)chunks;
+        job.first_block = blocks;
+        job.first_segment = segments;
+        HA_REQUIRE(nseg * chunks + blocks < (1ll << 30), HA_ERR_SHAPE, "ha_forward: too many sort chunks");
+        blocks += (int)(nseg * chunks);
+        segments += (int)nseg;
+        multi = multi || chunks > 1;
+      }
+    }
+    st = ha_sort_launch(jobs, blocks, segments, multi, stream);
+    if (st != HA_OK) return st;
+  }
+  return HA_OK;
+}
+
+// checks shared by ha_forward and ha_forward_sort once the plan and the workspace layout are known
+int check_hashing(const ha_forward_args& a, const Workspace& w, const char* who) {
+  HA_REQUIRE(a.proj, HA_ERR_NULL, "%s: null projection matrix", who);
+  HA_REQUIRE(a.lsh_num_projs >= 1, HA_ERR_SHAPE, "%s: Invalid value for num_projs", who);
+  HA_REQUIRE(a.lsh_num_projs <= 16, HA_ERR_UNSUPPORTED, "%s: lsh_num_projs above 16 is not built", who);
+  HA_REQUIRE(a.workspace && a.workspace_bytes >= w.total, HA_ERR_WORKSPACE, "%s: workspace of %lld bytes needed", who,
+             (long long)w.total);
   return HA_OK;
 }
 
@@ -234,6 +398,38 @@ extern "C" int64_t ha_forward_workspace_bytes(const ha_forward_args* args) {
   return w.total;
 }
 
+extern "C" int ha_forward_sort(const ha_forward_args* args, int64_t* q_idx_offset, int64_t* k_idx_offset,
+                               int* num_levels, void* stream) {
+  HA_REQUIRE(args && q_idx_offset && k_idx_offset && num_levels, HA_ERR_NULL, "ha_forward_sort: null argument");
+  const ha_forward_args& a = *args;
+  HA_REQUIRE(a.q && a.k, HA_ERR_NULL, "ha_forward_sort: null tensor pointer");
+  HA_REQUIRE(a.dtype == HA_F16 || a.dtype == HA_BF16, HA_ERR_DTYPE, "ha_forward_sort: Only support fp16 and bf16");
+  HA_REQUIRE(a.batch > 0 && a.heads > 0 && a.kv_heads > 0 && a.n > 0 && a.min_seq_len >= 0 && a.heads % a.kv_heads == 0,
+             HA_ERR_SHAPE, "ha_forward_sort: sizes must be positive and kv_heads must divide heads");
+  HA_REQUIRE(a.n < (1ll << 30), HA_ERR_SHAPE, "ha_forward_sort: sequence too long");
+  HA_REQUIRE(a.d == 64 || a.d == 128, HA_ERR_UNSUPPORTED, "ha_forward_sort: head dim %lld not built (64 and 128 are)",
+             (long long)a.d);
+  Plan pl;
+  int st = make_plan(a, pl);
+  if (st != HA_OK) return st;
+  Workspace w;
+  layout_workspace(a, pl, w);
+  const int nlev = a.causal ? pl.levels : 1;
+  *num_levels = nlev;
+  for (int j = 0; j < nlev; ++j) {
+    q_idx_offset[j] = pl.level_hyper[j] ? w.qidx[j] : -1;
+    k_idx_offset[j] = pl.level_hyper[j] ? w.kidx[j] : -1;
+  }
+  if (!pl.any_hyper) return HA_OK;
+  st = check_hashing(a, w, "ha_forward_sort");
+  if (st != HA_OK) return st;
+  ha_attn_operands t;
+  ha_forward_args b = a;
+  b.dv = a.d;
+  forward_operands(b, t);
+  return hash_and_sort(a, pl, w, t, (hipStream_t)stream);
+}
+
 extern "C" int ha_forward(const ha_forward_args* args, void* stream_) {
   HA_REQUIRE(args, HA_ERR_NULL, "ha_forward: null argument block");
   const ha_forward_args& a = *args;
@@ -246,86 +442,18 @@ extern "C" int ha_forward(const ha_forward_args* args, void* stream_) {
   Workspace w;
   layout_workspace(a, pl, w);
   if (pl.any_hyper) {
-    HA_REQUIRE(a.proj, HA_ERR_NULL, "ha_forward: null projection matrix");
-    HA_REQUIRE(a.lsh_num_projs >= 1, HA_ERR_SHAPE, "ha_forward: Invalid value for num_projs");
-    HA_REQUIRE(a.lsh_num_projs <= 8, HA_ERR_UNSUPPORTED, "ha_forward: lsh_num_projs > 8; compose from the operators");
-    HA_REQUIRE(a.workspace && a.workspace_bytes >= w.total, HA_ERR_WORKSPACE, "ha_forward: workspace of %lld bytes needed",
-               (long long)w.total);
+    st = check_hashing(a, w, "ha_forward");
+    if (st != HA_OK) return st;
   }
   unsigned char* ws = (unsigned char*)a.workspace;
-  const int64_t group = a.heads / a.kv_heads;
 
-  // operands shared by every launch: (batch, heads, n, d) tensors, contiguous unless strides are given
   ha_attn_operands t;
-  t.q = a.q; t.k = a.k; t.v = a.v; t.out = a.out; t.lse = a.lse;
-  t.batch = a.batch; t.heads = a.heads; t.d = a.d; t.dv = a.dv;
-  t.q_stride_b = a.heads * a.n * a.d; t.q_stride_h = a.n * a.d; t.q_stride_n = a.d;
-  t.k_stride_b = a.kv_heads * a.n * a.d; t.k_stride_h = a.n * a.d; t.k_stride_n = a.d;
-  t.v_stride_b = a.kv_heads * a.n * a.dv; t.v_stride_h = a.n * a.dv; t.v_stride_n = a.dv;
-  t.o_stride_b = a.heads * a.n * a.dv; t.o_stride_h = a.n * a.dv; t.o_stride_n = a.dv;
-  if (a.q_stride_b || a.q_stride_h || a.q_stride_n) {
-    t.q_stride_b = a.q_stride_b; t.q_stride_h = a.q_stride_h; t.q_stride_n = a.q_stride_n;
-  }
-  if (a.k_stride_b || a.k_stride_h || a.k_stride_n) {
-    t.k_stride_b = a.k_stride_b; t.k_stride_h = a.k_stride_h; t.k_stride_n = a.k_stride_n;
-  }
-  if (a.v_stride_b || a.v_stride_h || a.v_stride_n) {
-    t.v_stride_b = a.v_stride_b; t.v_stride_h = a.v_stride_h; t.v_stride_n = a.v_stride_n;
-  }
-  t.lse_stride_b = a.heads * a.n; t.lse_stride_h = a.n;
-  t.kv_group = group;
-  t.scale = a.scale;
-  t.dtype = a.dtype;
+  forward_operands(a, t);
 
-  // 1. bucket ids, once for the whole tensors (the projection does not depend on the level)
-  int32_t* bq = nullptr;
-  int32_t* bk = nullptr;
+  // 1. bucket ids, once for the whole tensors (the projection does not depend on the level), and
+  // 2. the bucket order of every segment of every hashed level
   if (pl.any_hyper) {
-    bq = (int32_t*)(ws + w.buckets_q);
-    bk = (int32_t*)(ws + w.buckets_k);
-    st = ha_lsh_hash(a.q, a.proj, bq, a.batch, a.heads, a.n, a.d, a.lsh_num_projs, t.q_stride_b, t.q_stride_h,
-                     t.q_stride_n, 0, 0, a.dtype, stream);
-    if (st != HA_OK) return st;
-    st = ha_lsh_hash(a.k, a.proj, bk, a.batch, a.kv_heads, a.n, a.d, a.lsh_num_projs, t.k_stride_b, t.k_stride_h,
-                     t.k_stride_n, 0, 0, a.dtype, stream);
-    if (st != HA_OK) return st;
-
-    // 2. all segmented sorts of all levels in one batch of launches
-    ha_sort_jobs jobs;
-    jobs.num_jobs = 0;
-    jobs.shift = 0;
-    jobs.idx64 = 0;
-    int blocks = 0, segments = 0;
-    bool multi = false;
-    const int nlev = a.causal ? pl.levels : 1;
-    for (int j = 0; j < nlev; ++j) {
-      if (!pl.level_hyper[j]) continue;
-      const int64_t seg_len = a.causal ? pl.len[j] / 2 : a.n;
-      const int64_t segs = a.causal ? (1ll << j) : 1;
-      const int64_t stride = a.causal ? pl.len[j] : a.n;
-      const int64_t chunks = (seg_len + HA_SORT_CHUNK - 1) / HA_SORT_CHUNK;
-      for (int side = 0; side < 2; ++side) {
-        HA_REQUIRE(jobs.num_jobs < HA_SORT_MAX_JOBS, HA_ERR_SHAPE, "ha_forward: too many sort jobs");
-        ha_sort_job& job = jobs.job[jobs.num_jobs++];
-        const int64_t nseg = a.batch * (side == 0 ? a.heads : a.kv_heads) * segs;
-        job.keys = side == 0 ? bq : bk;
-        job.prev = nullptr;
-        job.out = ws + (side == 0 ? w.qidx[j] : w.kidx[j]);
-        job.hist = (uint32_t*)(ws + (side == 0 ? w.hist_q[j] : w.hist_k[j]));
-        job.seg_stride = stride;
-        job.seg_offset = (a.causal && side == 0) ? seg_len : 0;  // queries: second halves, keys: first halves
-        job.seg_len = (int)seg_len;
-        job.num_segments = (int)nseg;
-        job.chunks_per_seg = (int)chunks;
-        job.first_block = blocks;
-        job.first_segment = segments;
-        HA_REQUIRE(nseg * chunks + blocks < (1ll << 30), HA_ERR_SHAPE, "ha_forward: too many sort chunks");
-        blocks += (int)(nseg * chunks);
-        segments += (int)nseg;
-        multi = multi || chunks > 1;
-      }
-    }
-    st = ha_sort_launch(jobs, blocks, segments, multi, stream);
+    st = hash_and_sort(a, pl, w, t, stream);
     if (st != HA_OK) return st;
   }
 

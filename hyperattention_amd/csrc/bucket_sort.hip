@@ -222,7 +222,135 @@ __global__ __launch_bounds__(SORT_THREADS) void sort_scatter_kernel(ha_sort_jobs
   }
 }
 
+
+// ---- one ranking for all levels ---------------------------------------------------------------------
+struct RankArgs {
+  const uint8_t* ids[2];
+  uint32_t* sorted[2];
+  uint32_t* hist[2];
+  int units0;   // units of the first tensor (seqs * units_per_seq)
+  ha_unit_grid grid;
+};
+
+// One workgroup per unit: bucket order of the unit's rows and its bucket counts.  Same ranking as the
+// scatter kernel above (a wave owns a contiguous run, ballot matching inside 64-row steps).
+__global__ __launch_bounds__(SORT_THREADS) void rank_units_kernel(RankArgs a) {
+  __shared__ uint32_t wave_hist[SORT_WAVES][256];
+  __shared__ uint32_t wave_totals[SORT_WAVES];
+  __shared__ uint32_t staged[HA_SORT_CHUNK];
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int which = (int)blockIdx.x >= a.units0 ? 1 : 0;
+  const int unit_id = (int)blockIdx.x - (which ? a.units0 : 0);
+  const ha_unit_grid& g = a.grid;
+  const int seq = unit_id / g.units_per_seq, u = unit_id % g.units_per_seq;
+  const int gran = u / g.units_per_granule, w = u % g.units_per_granule;
+  const int64_t row0 = (int64_t)seq * g.n + (int64_t)gran * g.granule + (int64_t)w * g.unit;
+  const int len = (int)min((int64_t)g.unit, g.granule - (int64_t)w * g.unit);
+  const uint8_t* ids = a.ids[which] + row0;
+#pragma unroll
+  for (int k = 0; k < SORT_WAVES; ++k) wave_hist[k][tid] = 0;
+  __syncthreads();
+
+  const int per_wave = ((len + SORT_THREADS - 1) / SORT_THREADS) * HA_WAVE;  // rows per wave, whole steps
+  const int wave_start = wave * per_wave;
+  int digit_all[SORT_STEPS];
+#pragma unroll
+  for (int s = 0; s < SORT_STEPS; ++s) digit_all[s] = ids[min(wave_start + s * HA_WAVE + lane, len - 1)];
+#pragma unroll
+  for (int s = 0; s < SORT_STEPS; ++s)
+    if (s * HA_WAVE < per_wave && wave_start + s * HA_WAVE + lane < len) atomicAdd(&wave_hist[wave][digit_all[s]], 1u);
+  __syncthreads();
+  uint32_t total = 0;
+#pragma unroll
+  for (int k = 0; k < SORT_WAVES; ++k) total += wave_hist[k][tid];
+  a.hist[which][(int64_t)unit_id * 256 + tid] = total;
+  uint32_t run = block_exclusive_scan(total, wave_totals);
+#pragma unroll
+  for (int k = 0; k < SORT_WAVES; ++k) {
+    const uint32_t c = wave_hist[k][tid];
+    wave_hist[k][tid] = run;
+    run += c;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int s = 0; s < SORT_STEPS; ++s) {
+    if (s * HA_WAVE >= per_wave) break;  // the same for every lane of the workgroup
+    const int i = wave_start + s * HA_WAVE + lane;
+    const bool valid = i < len;
+    const int digit = digit_all[s];
+    const uint64_t m = match_digit(digit, valid);
+    const uint32_t below = rank_below(m);
+    if (valid) staged[wave_hist[wave][digit] + below] = ((uint32_t)digit << 16) | (uint32_t)i;
+    __builtin_amdgcn_wave_barrier();
+    if (valid && below == 0) wave_hist[wave][digit] += (uint32_t)__popcll(m);
+    __builtin_amdgcn_wave_barrier();
+  }
+  __syncthreads();
+  uint32_t* out = a.sorted[which] + row0;
+  for (int pos = tid; pos < len; pos += SORT_THREADS) out[pos] = staged[pos];
+}
+
+// One workgroup per (job, segment, unit): where the unit's rows of every bucket start in the segment's
+// order, then a copy of the unit's order to those places.
+__global__ __launch_bounds__(SORT_THREADS) void place_units_kernel(ha_place_jobs jobs) {
+  __shared__ uint32_t wave_totals[SORT_WAVES];
+  __shared__ int32_t delta[256];   // segment slot minus unit slot, per bucket
+  int j = 0;
+  while (j + 1 < jobs.num_jobs && (int)blockIdx.x >= jobs.job[j + 1].first_block) ++j;
+  const ha_place_job& job = jobs.job[j];
+  const ha_unit_grid& g = jobs.grid;
+  const int tid = threadIdx.x;
+  const int local = (int)blockIdx.x - job.first_block;
+  const int seg = local / job.units_per_seg, u = local % job.units_per_seg;
+  const int seq = seg / job.segs_per_seq, sis = seg % job.segs_per_seq;
+  const int64_t first_row = job.seg_offset + (int64_t)sis * job.seg_stride;   // of the segment, in its sequence
+  const int64_t first_unit = (int64_t)seq * g.units_per_seq + (first_row / g.granule) * g.units_per_granule;
+  const uint32_t* h = job.hist + first_unit * 256 + tid;
+  uint32_t tot = 0, before = 0, mine = 0;
+  for (int k = 0; k < job.units_per_seg; ++k) {
+    const uint32_t c = h[(int64_t)k * 256];
+    before += k < u ? c : 0u;
+    mine = k == u ? c : mine;
+    tot += c;
+  }
+  const uint32_t seg_first = block_exclusive_scan(tot, wave_totals);
+  const uint32_t unit_first = block_exclusive_scan(mine, wave_totals);
+  delta[tid] = (int32_t)(seg_first + before) - (int32_t)unit_first;
+  __syncthreads();
+  const int gran = u / g.units_per_granule, w = u % g.units_per_granule;
+  const int64_t row0 = (int64_t)gran * g.granule + (int64_t)w * g.unit;   // of the unit, in its segment
+  const int len = (int)min((int64_t)g.unit, g.granule - (int64_t)w * g.unit);
+  const uint32_t* src = job.sorted + (int64_t)seq * g.n + first_row + row0;
+  int32_t* out = job.out + (int64_t)seg * job.seg_len;
+  for (int pos = tid; pos < len; pos += SORT_THREADS) {
+    const uint32_t v = src[pos];
+    out[pos + delta[v >> 16]] = (int32_t)row0 + (int32_t)(v & 0xFFFFu);
+  }
+}
+
 }  // namespace
+
+int ha_rank_units(const uint8_t* const ids[2], uint32_t* const sorted[2], uint32_t* const hist[2], const int64_t seqs[2],
+                  const ha_unit_grid& grid, hipStream_t stream) {
+  RankArgs a;
+  for (int i = 0; i < 2; ++i) {
+    a.ids[i] = ids[i];
+    a.sorted[i] = sorted[i];
+    a.hist[i] = hist[i];
+  }
+  a.grid = grid;
+  const int64_t units = (seqs[0] + seqs[1]) * grid.units_per_seq;
+  HA_REQUIRE(units < (1ll << 31) && grid.unit >= 1 && grid.unit <= HA_SORT_CHUNK, HA_ERR_SHAPE,
+             "ha_forward: too many sort units");
+  a.units0 = (int)(seqs[0] * grid.units_per_seq);
+  hipLaunchKernelGGL(rank_units_kernel, dim3((unsigned)units), dim3(SORT_THREADS), 0, stream, a);
+  return ha_launch_status("ha_forward (rank)");
+}
+
+int ha_place_units(const ha_place_jobs& jobs, int total_blocks, hipStream_t stream) {
+  hipLaunchKernelGGL(place_units_kernel, dim3(total_blocks), dim3(SORT_THREADS), 0, stream, jobs);
+  return ha_launch_status("ha_forward (place)");
+}
 
 int ha_sort_launch(const ha_sort_jobs& jobs, int total_blocks, int total_segments, bool any_multi_chunk,
                    hipStream_t stream) {

@@ -16,6 +16,7 @@
 // lsh_hash_kernel (any head dim that is a multiple of 8): one thread per row, rows staged through
 // LDS with coalesced 16-byte loads, all projections accumulated in fp64.
 #include "ha_common.h"
+#include "bucket_sort.h"
 
 namespace {
 
@@ -100,21 +101,33 @@ constexpr int HASH_UNROLL = 8;           // tiles in flight per wave
 // MFMA row m = (data row)*PARTS + part; lane (m = lane%16, kg = lane/16) holds elements
 // part*32 + 8*kg .. +7 of its data row.  The C registers i = 0..3 of a lane are MFMA rows 4*kg + i
 // of projection slot lane%16; the partial projections of one data row are summed afterwards.
-template <typename T, int D>
-__global__ __launch_bounds__(256) void lsh_hash_mfma_kernel(const T* __restrict__ x, const T* __restrict__ proj,
-                                                            int32_t* __restrict__ buckets, int heads, int64_t n, int r,
-                                                            int64_t sb, int64_t sh, int64_t sn, int64_t psb,
-                                                            int64_t psh) {
+// Up to two tensors per launch (queries and keys of one forward): blockIdx.y counts the (batch, head)
+// sequences of the first tensor, then those of the second.
+struct HashTensors {
+  const void* x[2];
+  void* out[2];        // bucket ids, (batch, heads, n) contiguous, int32 or (OUT8) one byte each
+  int64_t sb[2], sh[2], sn[2];
+  int heads[2];
+  int seqs0;           // batch * heads of the first tensor
+};
+
+template <typename T, int D, bool OUT8>
+__global__ __launch_bounds__(256) void lsh_hash_mfma_kernel(const HashTensors ten, const T* __restrict__ proj, int64_t n,
+                                                            int r, int64_t psb, int64_t psh) {
   typedef typename ElemTraits<T>::vec8 vec8;
   constexpr int PARTS = D / 32;
   constexpr int ROWS = 16 / PARTS;            // data rows per tile
   constexpr int NS = PARTS >= 4 ? 1 : 4 / PARTS;  // data rows per lane (sums of C registers)
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int bh = blockIdx.y;
+  const int which = (int)blockIdx.y >= ten.seqs0 ? 1 : 0;
+  const int bh = (int)blockIdx.y - (which ? ten.seqs0 : 0);
+  const int heads = ten.heads[which];
   const int b = bh / heads, h = bh % heads;
-  const T* xbase = x + b * sb + h * sh;
+  const T* xbase = (const T*)ten.x[which] + b * ten.sb[which] + h * ten.sh[which];
+  const int64_t sn = ten.sn[which];
   const T* pbase = proj + b * psb + h * psh;
-  int32_t* obase = buckets + (int64_t)bh * n;
+  int32_t* obase = OUT8 ? nullptr : (int32_t*)ten.out[which] + (int64_t)bh * n;
+  uint8_t* obase8 = OUT8 ? (uint8_t*)ten.out[which] + (int64_t)bh * n : nullptr;
   const int m = lane & 15, kg = lane >> 4;
   const int my_row = m / PARTS, my_part = m % PARTS;  // data row inside a tile, 32-element part of it
   const int j = m;                                    // projection slot of this lane's C registers
@@ -220,18 +233,22 @@ __global__ __launch_bounds__(256) void lsh_hash_mfma_kernel(const T* __restrict_
         for (int qq = 1; qq < NS; ++qq) sel = q == qq ? pos[qq] : sel;
         bin = (int)((sel >> (16 * g)) & ((1u << r) - 1u));
       }
-      if (lane < ROWS && tile_row0 + lane < n) obase[tile_row0 + lane] = bin ^ (bin >> 1);
+      if (lane < ROWS && tile_row0 + lane < n) {
+        if (OUT8)
+          obase8[tile_row0 + lane] = (uint8_t)(bin ^ (bin >> 1));
+        else
+          obase[tile_row0 + lane] = bin ^ (bin >> 1);
+      }
     }
   }
 }
 
-template <typename T, int D>
-int launch_hash_mfma(const void* x, const void* proj, int32_t* buckets, int64_t batch, int64_t heads, int64_t n,
-                     int64_t r, int64_t sb, int64_t sh, int64_t sn, int64_t psb, int64_t psh, hipStream_t stream) {
+template <typename T, int D, bool OUT8>
+int launch_hash_mfma(const HashTensors& ten, int64_t seqs, const void* proj, int64_t n, int64_t r, int64_t psb, int64_t psh,
+                     hipStream_t stream) {
   const int64_t rows_per_block = 4 * HASH_TILES_PER_WAVE * (16 / (D / 32));
-  dim3 grid((unsigned)((n + rows_per_block - 1) / rows_per_block), (unsigned)(batch * heads));
-  hipLaunchKernelGGL((lsh_hash_mfma_kernel<T, D>), grid, dim3(256), 0, stream, (const T*)x, (const T*)proj, buckets,
-                     (int)heads, n, (int)r, sb, sh, sn, psb, psh);
+  dim3 grid((unsigned)((n + rows_per_block - 1) / rows_per_block), (unsigned)seqs);
+  hipLaunchKernelGGL((lsh_hash_mfma_kernel<T, D, OUT8>), grid, dim3(256), 0, stream, ten, (const T*)proj, n, (int)r, psb, psh);
   return ha_launch_status("ha_lsh_hash");
 }
 
@@ -268,13 +285,16 @@ extern "C" int ha_lsh_hash(const void* x, const void* proj, int32_t* buckets, in
   HA_REQUIRE(x_stride_n % 8 == 0 && x_stride_h % 8 == 0 && x_stride_b % 8 == 0 && ((uintptr_t)x % 16) == 0,
              HA_ERR_SHAPE, "ha_lsh_hash: rows must be 16-byte aligned");
   hipStream_t s = (hipStream_t)stream;
-#define HA_HASH_MFMA(DD)                                                                                             \
-  if (d == DD) {                                                                                                     \
-    if (dtype == HA_F16)                                                                                             \
-      return launch_hash_mfma<f16_t, DD>(x, proj, buckets, batch, heads, n, r, x_stride_b, x_stride_h, x_stride_n,   \
-                                         proj_stride_b, proj_stride_h, s);                                           \
-    return launch_hash_mfma<bf16_t, DD>(x, proj, buckets, batch, heads, n, r, x_stride_b, x_stride_h, x_stride_n,    \
-                                        proj_stride_b, proj_stride_h, s);                                            \
+  HashTensors ten = {};
+  ten.x[0] = x; ten.out[0] = buckets;
+  ten.sb[0] = x_stride_b; ten.sh[0] = x_stride_h; ten.sn[0] = x_stride_n;
+  ten.heads[0] = ten.heads[1] = (int)heads;
+  ten.seqs0 = (int)(batch * heads);
+#define HA_HASH_MFMA(DD)                                                                                              \
+  if (d == DD) {                                                                                                      \
+    if (dtype == HA_F16)                                                                                              \
+      return launch_hash_mfma<f16_t, DD, false>(ten, batch * heads, proj, n, r, proj_stride_b, proj_stride_h, s);     \
+    return launch_hash_mfma<bf16_t, DD, false>(ten, batch * heads, proj, n, r, proj_stride_b, proj_stride_h, s);      \
   }
   HA_HASH_MFMA(32) HA_HASH_MFMA(64) HA_HASH_MFMA(128) HA_HASH_MFMA(256)
 #undef HA_HASH_MFMA
@@ -283,4 +303,29 @@ extern "C" int ha_lsh_hash(const void* x, const void* proj, int32_t* buckets, in
                               proj_stride_b, proj_stride_h, s);
   return launch_hash<bf16_t>(x, proj, buckets, batch, heads, n, d, r, x_stride_b, x_stride_h, x_stride_n,
                              proj_stride_b, proj_stride_h, s);
+}
+
+// Bucket ids of the queries and keys of one forward pass as one byte each (r <= 8 projections, one shared
+// projection matrix), in one launch.  q: (batch, heads, n, d), k: (batch, kv_heads, n, d), d in {64, 128}.
+int ha_hash_pair_u8(const void* q, const void* k, const void* proj, uint8_t* ids_q, uint8_t* ids_k, int64_t batch,
+                    int64_t heads, int64_t kv_heads, int64_t n, int64_t d, int64_t r, const int64_t (&q_strides)[3],
+                    const int64_t (&k_strides)[3], int dtype, hipStream_t stream) {
+  HA_REQUIRE(r >= 1 && r <= 8, HA_ERR_UNSUPPORTED, "ha_forward: byte-sized bucket ids need at most 8 projections");
+  HA_REQUIRE(batch * (heads + kv_heads) <= 65535, HA_ERR_SHAPE, "ha_forward: batch*(heads + kv_heads) must be <= 65535");
+  HashTensors ten = {};
+  ten.x[0] = q; ten.x[1] = k; ten.out[0] = ids_q; ten.out[1] = ids_k;
+  ten.sb[0] = q_strides[0]; ten.sh[0] = q_strides[1]; ten.sn[0] = q_strides[2];
+  ten.sb[1] = k_strides[0]; ten.sh[1] = k_strides[1]; ten.sn[1] = k_strides[2];
+  ten.heads[0] = (int)heads; ten.heads[1] = (int)kv_heads;
+  ten.seqs0 = (int)(batch * heads);
+  const int64_t seqs = batch * (heads + kv_heads);
+  if (d == 64) {
+    if (dtype == HA_F16) return launch_hash_mfma<f16_t, 64, true>(ten, seqs, proj, n, r, 0, 0, stream);
+    return launch_hash_mfma<bf16_t, 64, true>(ten, seqs, proj, n, r, 0, 0, stream);
+  }
+  if (d == 128) {
+    if (dtype == HA_F16) return launch_hash_mfma<f16_t, 128, true>(ten, seqs, proj, n, r, 0, 0, stream);
+    return launch_hash_mfma<bf16_t, 128, true>(ten, seqs, proj, n, r, 0, 0, stream);
+  }
+  return ha_fail(HA_ERR_UNSUPPORTED, "ha_forward: head dim %lld not built (64 and 128 are)", (long long)d);
 }

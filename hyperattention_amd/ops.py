@@ -390,7 +390,7 @@ class FlashAttnFunc(torch.autograd.Function):
 # ------------------------------------------------------------------------- whole forward pass
 def forward_plan_supported(n: int, min_seq_len: int, causal: bool, lsh_num_projs: int) -> bool:
     """True when ha_forward covers this shape: every causal recursion level has an even length."""
-    if lsh_num_projs > 8:
+    if lsh_num_projs > 16:
         return False
     if not causal:
         return True
@@ -401,19 +401,19 @@ def forward_plan_supported(n: int, min_seq_len: int, causal: bool, lsh_num_projs
     return True
 
 
-def hyper_forward(q, k, v, proj, *, scale, causal, lsh_num_projs, block_size, sample_size, min_seq_len,
+def _forward_args(q, k, v, out, lse, proj, *, scale, causal, lsh_num_projs, block_size, sample_size, min_seq_len,
                   smooth_block, sampled_idx=None):
-    """One-call forward for (b,h,n,d) q and (b,h_kv,n,d) k, v of any strides with a contiguous last
-    dimension (permuted views are read in place).  Returns contiguous out (b,h,n,dv) and lse (b,h,n) fp32."""
-    assert q.is_cuda and k.is_cuda and v.is_cuda
-    assert q.stride(-1) == 1 and k.stride(-1) == 1 and v.stride(-1) == 1
-    assert q.dtype == k.dtype == v.dtype, "All tensors must have the same type"
+    """ForwardArgs for (b,h,n,d) q and (b,h_kv,n,d) k, v with its workspace attached; the second result keeps
+    the tensors alive that the struct only points to."""
+    assert q.is_cuda and k.is_cuda
+    assert q.stride(-1) == 1 and k.stride(-1) == 1 and (v is None or v.stride(-1) == 1)
+    assert q.dtype == k.dtype and (v is None or v.dtype == q.dtype), "All tensors must have the same type"
     b, h, n, d = q.shape
     hk = k.shape[1]
     a = ForwardArgs()
-    out = torch.empty((b, h, n, v.shape[-1]), device=q.device, dtype=q.dtype)
-    lse = torch.empty((b, h, n), device=q.device, dtype=torch.float32)
-    a.q, a.k, a.v, a.out, a.lse = q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr()
+    a.q, a.k = q.data_ptr(), k.data_ptr()
+    if v is not None:
+        a.v, a.out, a.lse = v.data_ptr(), out.data_ptr(), lse.data_ptr()
     keep = []
     if proj is not None:
         assert proj.dtype == q.dtype, "All three tensors must have the same type"
@@ -428,20 +428,65 @@ def hyper_forward(q, k, v, proj, *, scale, causal, lsh_num_projs, block_size, sa
         assert s.shape == (sample_size,)
         keep.append(s)
         a.sampled_idx = s.data_ptr()
-    a.batch, a.heads, a.kv_heads, a.n, a.d, a.dv = b, h, hk, n, d, v.shape[-1]
+    a.batch, a.heads, a.kv_heads, a.n, a.d = b, h, hk, n, d
+    a.dv = v.shape[-1] if v is not None else d
     a.lsh_num_projs, a.block_size, a.sample_size, a.min_seq_len = lsh_num_projs, block_size, sample_size, min_seq_len
     a.smooth_block, a.causal = int(bool(smooth_block)), int(bool(causal))
     a.scale = scale
     a.dtype = _dtype_code(q)
     a.q_stride_b, a.q_stride_h, a.q_stride_n = q.stride(0), q.stride(1), q.stride(2)
     a.k_stride_b, a.k_stride_h, a.k_stride_n = k.stride(0), k.stride(1), k.stride(2)
-    a.v_stride_b, a.v_stride_h, a.v_stride_n = v.stride(0), v.stride(1), v.stride(2)
-    L = _lib.lib()
-    ws_bytes = L.ha_forward_workspace_bytes(ctypes.byref(a))
+    if v is not None:
+        a.v_stride_b, a.v_stride_h, a.v_stride_n = v.stride(0), v.stride(1), v.stride(2)
+    ws_bytes = _lib.lib().ha_forward_workspace_bytes(ctypes.byref(a))
     if ws_bytes < 0:
         _lib.check(int(ws_bytes))
     ws = torch.empty(int(ws_bytes), device=q.device, dtype=torch.uint8)
     a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
+    keep.append(ws)
+    return a, keep
+
+
+def hyper_forward(q, k, v, proj, *, scale, causal, lsh_num_projs, block_size, sample_size, min_seq_len,
+                  smooth_block, sampled_idx=None):
+    """One-call forward for (b,h,n,d) q and (b,h_kv,n,d) k, v of any strides with a contiguous last
+    dimension (permuted views are read in place).  Returns contiguous out (b,h,n,dv) and lse (b,h,n) fp32."""
+    assert v.is_cuda
+    b, h, n, d = q.shape
+    out = torch.empty((b, h, n, v.shape[-1]), device=q.device, dtype=q.dtype)
+    lse = torch.empty((b, h, n), device=q.device, dtype=torch.float32)
+    a, keep = _forward_args(q, k, v, out, lse, proj, scale=scale, causal=causal, lsh_num_projs=lsh_num_projs,
+                            block_size=block_size, sample_size=sample_size, min_seq_len=min_seq_len,
+                            smooth_block=smooth_block, sampled_idx=sampled_idx)
     with torch.cuda.device(q.device):
-        _lib.check(L.ha_forward(ctypes.byref(a), _stream(q)))
+        _lib.check(_lib.lib().ha_forward(ctypes.byref(a), _stream(q)))
     return out, lse
+
+
+def forward_sort(q, k, proj, *, causal, lsh_num_projs, min_seq_len):
+    """Bucket orders of every hashed level of the forward pass (ha_forward_sort): one hash launch for q and
+    k, one ranking, one placement.  Returns (q_idx, k_idx): per level (0 = whole sequence) an int32 tensor
+    (b, h * 2^level, half) / (b, h_kv * 2^level, half) of rows local to the level's query segment (second
+    halves) / key segment (first halves), or None where the level is exact.  The tensors are views of one
+    workspace."""
+    b, h, n, d = q.shape
+    hk = k.shape[1]
+    a, keep = _forward_args(q, k, None, None, None, proj, scale=1.0, causal=causal, lsh_num_projs=lsh_num_projs,
+                            block_size=128, sample_size=0, min_seq_len=min_seq_len, smooth_block=False)
+    ws = keep[-1]
+    q_off = (ctypes.c_int64 * 48)()
+    k_off = (ctypes.c_int64 * 48)()
+    levels = ctypes.c_int(0)
+    with torch.cuda.device(q.device):
+        _lib.check(_lib.lib().ha_forward_sort(ctypes.byref(a), q_off, k_off, ctypes.byref(levels), _stream(q)))
+    q_idx, k_idx = [], []
+    for j in range(levels.value):
+        if q_off[j] < 0:
+            q_idx.append(None)
+            k_idx.append(None)
+            continue
+        segs = (1 << j) if causal else 1
+        half = (n >> (j + 1)) if causal else n
+        q_idx.append(ws[q_off[j]:q_off[j] + 4 * b * h * segs * half].view(torch.int32).view(b, h * segs, half))
+        k_idx.append(ws[k_off[j]:k_off[j] + 4 * b * hk * segs * half].view(torch.int32).view(b, hk * segs, half))
+    return q_idx, k_idx

@@ -23,7 +23,7 @@
 extern "C" {
 #endif
 
-#define HA_ABI_VERSION 4
+#define HA_ABI_VERSION 5
 
 typedef enum {
   HA_OK = 0,
@@ -274,6 +274,21 @@ typedef struct {
 
 int64_t ha_forward_workspace_bytes(const ha_forward_args* args);
 int ha_forward(const ha_forward_args* args, void* stream);
+
+/* The first stage of ha_forward alone: bucket ids of q and k (one launch) and the stable bucket order of the
+ * query and key segment of every hashed level (one ranking of the rows, one placement launch for all
+ * levels), written into the workspace.
+ * replaces: the lsh.hash + torch.sort pairs of every level of the recursion (hyper_attention.py:112-117
+ * under :51-96) for a caller that runs the levels itself, e.g. to keep what a backward pass needs.
+ * For level j (0 = whole sequence; the only one without a causal mask) q_idx_offset[j] / k_idx_offset[j]
+ * receive the byte offsets into the workspace of int32 arrays (batch, heads * 2^j, half) and
+ * (batch, kv_heads * 2^j, half) of rows local to the level's query segment (second halves) and key segment
+ * (first halves), or -1 where the level is exact (its half is shorter than min_seq_len).  Both arrays must
+ * hold 48 entries; *num_levels receives the number of levels.  Only q, k, proj, the sizes, dtype, causal,
+ * min_seq_len, lsh_num_projs, the strides and the workspace of `args` are read.
+ */
+int ha_forward_sort(const ha_forward_args* args, int64_t* q_idx_offset, int64_t* k_idx_offset, int* num_levels,
+                    void* stream);
 
 #ifdef __cplusplus
 }

@@ -229,6 +229,44 @@ def test_full_size_causal_properties(ha):
     assert_close(lse_one, rl, "lse head 5")
 
 
+@pytest.mark.parametrize("b,h,hk,n,d,msl,causal,r,dtype", [
+    (1, 4, 4, 8192, 64, 1024, True, 8, torch.float16),      # leaves of 1024 rows: a unit per leaf
+    (2, 4, 2, 16384, 128, 2048, True, 7, torch.bfloat16),   # grouped-query, 7 projections
+    (1, 2, 2, 40960, 64, 6000, True, 8, torch.float16),     # leaves of 5120 rows: units of 4096 and 1024
+    (1, 2, 1, 12800, 64, 2048, False, 8, torch.float16),    # one segment of units 4096, 4096, 4096, 512
+    (1, 2, 2, 8192, 64, 1024, True, 12, torch.float16),     # 4096 buckets: two-digit sort per level
+    (1, 1, 1, 262144, 64, 128, True, 4, torch.float16),     # more units per segment than one ranking serves
+    (1, 2, 2, 8192, 64, 128, True, 8, torch.float16),       # 32 units of 128 rows in the longest segment
+    (1, 2, 2, 16384, 64, 9000, True, 8, torch.float16),     # top level exact, none hashed
+])
+def test_forward_sort_is_the_stable_sort_of_every_level(ha, b, h, hk, n, d, msl, causal, r, dtype):
+    """The orders that the one-call forward works with are, bit for bit, the stable sorts of the bucket ids of
+    every level's query and key segment (hyper_attention.py:112-117 inside :51-96)."""
+    from hyperattention_amd import ops
+    q = _randn((b, h, n, d), 300, dtype).cuda()
+    k = _randn((b, hk, n, d), 301, dtype).cuda()
+    proj = _randn((1, 1, d, r), 302, dtype).cuda()
+    q_idx, k_idx = ops.forward_sort(q, k, proj, causal=causal, lsh_num_projs=r, min_seq_len=msl)
+    bq, bk = ops.lsh_hash(q, proj), ops.lsh_hash(k, proj)
+    assert len(q_idx) == len(k_idx) and len(q_idx) >= 1
+    for level in range(len(q_idx)):
+        half = (n >> (level + 1)) if causal else n
+        hashed = not (msl > half)
+        assert (q_idx[level] is not None) == hashed and (k_idx[level] is not None) == hashed
+        if not hashed:
+            continue
+        if causal:
+            want_q = bq.view(b, h << level, 2, half)[:, :, 1].sort(dim=-1, stable=True).indices
+            want_k = bk.view(b, hk << level, 2, half)[:, :, 0].sort(dim=-1, stable=True).indices
+        else:
+            want_q = bq.sort(dim=-1, stable=True).indices
+            want_k = bk.sort(dim=-1, stable=True).indices
+        assert torch.equal(q_idx[level].long(), want_q), f"query order of level {level}"
+        assert torch.equal(k_idx[level].long(), want_k), f"key order of level {level}"
+    if causal:
+        assert (n >> len(q_idx)) <= msl < (n >> (len(q_idx) - 1))
+
+
 def _check_sort_properties(ha, buckets):
     """the permutation of every head is a permutation, sorts its keys, and keeps equal keys in row order"""
     b, h, n = buckets.shape
