@@ -31,7 +31,7 @@ SYMBOLS = [
     "ha_bucket_argsort", "ha_bucket_argsort_static", "ha_gather_rows", "ha_block_attn_fwd", "ha_flash_attn_fwd",
     "ha_attn_bwd_workspace_bytes", "ha_block_attn_bwd", "ha_flash_attn_bwd", "ha_lse_merge",
     "ha_lse_merge_segments",
-    "ha_forward_workspace_bytes", "ha_forward", "ha_forward_sort",
+    "ha_forward_workspace_bytes", "ha_forward", "ha_forward_sort", "ha_lse_merge_levels",
 ]
 
 HA_F16, HA_BF16 = 0, 1
@@ -165,6 +165,9 @@ def _declare(lib):
     lib.ha_forward_workspace_bytes.argtypes = [ctypes.POINTER(ForwardArgs)]
     lib.ha_forward.restype = ci
     lib.ha_forward.argtypes = [ctypes.POINTER(ForwardArgs), vp]
+    lib.ha_lse_merge_levels.restype = ci
+    lib.ha_lse_merge_levels.argtypes = [vp, vp, ctypes.POINTER(vp), ctypes.POINTER(vp), ctypes.POINTER(vp), vp, vp, vp,
+                                        ci, i64, i64, i64, ci, vp]
     lib.ha_forward_sort.restype = ci
     lib.ha_forward_sort.argtypes = [ctypes.POINTER(ForwardArgs), ctypes.POINTER(i64), ctypes.POINTER(i64),
                                     ctypes.POINTER(ci), vp]

@@ -33,9 +33,11 @@ class AngularLSH(torch.nn.Module):
         i = torch.arange(1 << size_n, dtype=torch.int32)
         return i ^ (i >> 1)
 
-    def hash(self, mat):
-        """Bucket ids from the HIP kernel; mat is (b, h, n, d) fp16/bf16 on the GPU."""
-        proj = self.proj_dir
+    def hash(self, mat, proj=None):
+        """Bucket ids from the HIP kernel; mat is (b, h, n, d) fp16/bf16 on the GPU.  proj (not in the
+        reference): a projection to use instead of the module's own, e.g. one with zero rows added for
+        zero-padded inputs."""
+        proj = self.proj_dir if proj is None else proj
         if proj.dim() == 3:
             proj = proj.unsqueeze(0)
         return ops.lsh_hash(mat, proj)

@@ -39,6 +39,8 @@ struct ha_attn_bwd_params {
   int64_t ki_sb, ki_sh, ki_sn;
   int64_t si_sb, si_sh;
   int batch, heads, kv_group;
+  int segs;                                // segments per head, as in the forward
+  int64_t seg_stride, q_seg_off, k_seg_off;  // rows
   int n_q, n_k;
   int block_tiles;  // ceil(block_size / 128)
   int sample_size;

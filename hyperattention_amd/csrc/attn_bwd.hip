@@ -115,7 +115,9 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 || PASS == HA_BWD_DQ_BLOCK ? 2
   // (the dk/dv tiles are in that order as they come: the first key tile streams the most queries)
   if (PASS == HA_BWD_DQ_EXACT && CAUSAL) tile = st_tiles - 1 - tile;
   const int split = rest % splits;
-  const int bh = rest / splits;
+  const int vseq = rest / splits;   // (batch, head, segment)
+  const int seg = vseq % p.segs;
+  const int bh = vseq / p.segs;
   // The dK/dV passes that see every query of a key (exact attention, the blocks) take one workgroup per
   // KEY head and stream the queries of all the query heads of its group, one head after the other, so
   // that the sums are complete in registers; the other passes take one workgroup per query head.
@@ -132,22 +134,25 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 || PASS == HA_BWD_DQ_BLOCK ? 2
     hk = h0 / p.kv_group;
   }
   const int n_group = GROUP_LOOP ? p.kv_group : 1;
+  // first row of this segment in the query-side and in the key-side tensors
+  const int64_t q_row0 = p.q_seg_off + (int64_t)seg * p.seg_stride;
+  const int64_t k_row0 = p.k_seg_off + (int64_t)seg * p.seg_stride;
 
   // query-side tensors of query head h0 + gi
-  auto q_head = [&](int gi) { return (const unsigned char*)((const T*)p.q + b * p.q_sb + (h0 + gi) * p.q_sh); };
-  auto do_head = [&](int gi) { return (const unsigned char*)((const T*)p.dout + b * p.do_sb + (h0 + gi) * p.do_sh); };
+  auto q_head = [&](int gi) { return (const unsigned char*)((const T*)p.q + b * p.q_sb + (h0 + gi) * p.q_sh + q_row0 * p.q_sn); };
+  auto do_head = [&](int gi) { return (const unsigned char*)((const T*)p.dout + b * p.do_sb + (h0 + gi) * p.do_sh + q_row0 * p.do_sn); };
   // per query: {L in log2 units, D * scale} with D_i = sum_c dO_ic O_ic (src/hyper_attn_triton.py:195-226),
   // written by the dq pass of the call
-  auto stats_head = [&](int gi) { return p.stats + (int64_t)(b * p.heads + h0 + gi) * p.n_q; };
+  auto stats_head = [&](int gi) { return p.stats + ((int64_t)(b * p.heads + h0 + gi) * p.segs + seg) * p.n_q; };
   const int idx_shift = p.idx64 ? 3 : 2;
   auto q_idx_head = [&](int gi) {
-    return (const unsigned char*)p.q_idx + ((b * p.qi_sb + (h0 + gi) * p.qi_sh) << idx_shift);
+    return (const unsigned char*)p.q_idx + ((b * p.qi_sb + (h0 + gi) * p.qi_sh + (int64_t)seg * p.n_q * p.qi_sn) << idx_shift);
   };
-  const unsigned char* const kb = (const unsigned char*)((const T*)p.k + b * p.k_sb + hk * p.k_sh);
-  const unsigned char* const vb = (const unsigned char*)((const T*)p.v + b * p.v_sb + hk * p.v_sh);
+  const unsigned char* const kb = (const unsigned char*)((const T*)p.k + b * p.k_sb + hk * p.k_sh + k_row0 * p.k_sn);
+  const unsigned char* const vb = (const unsigned char*)((const T*)p.v + b * p.v_sb + hk * p.v_sh + k_row0 * p.v_sn);
   const uint32_t q_rb = (uint32_t)p.q_sn * 2, k_rb = (uint32_t)p.k_sn * 2, v_rb = (uint32_t)p.v_sn * 2,
                  do_rb = (uint32_t)p.do_sn * 2;
-  const unsigned char* const k_idx = (const unsigned char*)p.k_idx + ((b * p.ki_sb + hk * p.ki_sh) << idx_shift);
+  const unsigned char* const k_idx = (const unsigned char*)p.k_idx + ((b * p.ki_sb + hk * p.ki_sh + (int64_t)seg * p.n_k * p.ki_sn) << idx_shift);
   const unsigned char* const s_idx =
       p.sampled_idx ? (const unsigned char*)p.sampled_idx + ((b * p.si_sb + hk * p.si_sh) << idx_shift) : nullptr;
   const uint32_t qi_rb = (uint32_t)p.qi_sn << idx_shift, ki_rb = (uint32_t)p.ki_sn << idx_shift;
@@ -290,9 +295,9 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 || PASS == HA_BWD_DQ_BLOCK ? 2
     // nothing attends (or is attended by) this tile: its gradient is zero
     if (PASS != HA_BWD_DKV_SAMPLED && st_valid) {
       const vec4 zero = {(T)0.f, (T)0.f, (T)0.f, (T)0.f};
-      unsigned char* const dqb = (unsigned char*)((T*)p.dq + b * p.dq_sb + h0 * p.dq_sh) + (int64_t)st_row * p.dq_sn * 2;
-      unsigned char* const dkb = (unsigned char*)((T*)p.dk + b * p.dk_sb + hk * p.dk_sh) + (int64_t)st_row * p.dk_sn * 2;
-      unsigned char* const dvb = (unsigned char*)((T*)p.dv + b * p.dv_sb + hk * p.dv_sh) + (int64_t)st_row * p.dv_sn * 2;
+      unsigned char* const dqb = (unsigned char*)((T*)p.dq + b * p.dq_sb + h0 * p.dq_sh + q_row0 * p.dq_sn) + (int64_t)st_row * p.dq_sn * 2;
+      unsigned char* const dkb = (unsigned char*)((T*)p.dk + b * p.dk_sb + hk * p.dk_sh + k_row0 * p.dk_sn) + (int64_t)st_row * p.dk_sn * 2;
+      unsigned char* const dvb = (unsigned char*)((T*)p.dv + b * p.dv_sb + hk * p.dv_sh + k_row0 * p.dv_sn) + (int64_t)st_row * p.dv_sn * 2;
 #pragma unroll
       for (int db = 0; db < DB; ++db)
 #pragma unroll
@@ -348,7 +353,7 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 || PASS == HA_BWD_DQ_BLOCK ? 2
   vec8 x1f[KSTEPS], x2f[KSTEPS];
   float st_lse2 = 0.f, st_delta = 0.f;  // dQ passes: L (log2 units) and D * scale of the lane's query
   vec8 of[KSTEPS];  // dQ passes: the lane's pieces of its query's output row
-  const unsigned char* const ob = (const unsigned char*)((const T*)p.out + b * p.o_sb + h0 * p.o_sh);
+  const unsigned char* const ob = (const unsigned char*)((const T*)p.out + b * p.o_sb + h0 * p.o_sh + q_row0 * p.o_sn);
   const uint32_t o_rb = (uint32_t)p.o_sn * 2;
   if (!KEY_ST) {
     if (!STAGE_X) {
@@ -356,7 +361,7 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 || PASS == HA_BWD_DQ_BLOCK ? 2
       for (int ks = 0; ks < KSTEPS; ++ks)
         of[ks] = *reinterpret_cast<const vec8*>(row_address(ob, st_row, o_rb, (ks * 16 + hi * 8) * 2));
     }
-    st_lse2 = p.lse[b * p.lse_sb + h0 * p.lse_sh + st_row] * LOG2E;
+    st_lse2 = p.lse[b * p.lse_sb + h0 * p.lse_sh + q_row0 + st_row] * LOG2E;
   }
   if (!STAGE_X) {
 #pragma unroll
@@ -418,7 +423,7 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 || PASS == HA_BWD_DQ_BLOCK ? 2
 #pragma unroll
       for (int e = 0; e < 8; ++e) part = __builtin_fmaf((float)of[ks][e], (float)x2f[ks][e], part);
     st_delta = (part + __shfl_xor(part, 32)) * p.scale;
-    if (hi == 0 && st_valid) p.stats[(int64_t)(b * p.heads + h0) * p.n_q + st_row] = f32x2{st_lse2, st_delta};
+    if (hi == 0 && st_valid) p.stats[((int64_t)(b * p.heads + h0) * p.segs + seg) * p.n_q + st_row] = f32x2{st_lse2, st_delta};
   }
 
   // per-lane LDS offsets of the operand reads
@@ -609,14 +614,14 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 || PASS == HA_BWD_DQ_BLOCK ? 2
       }
     };
     if (!KEY_ST) {
-      store_rows(acc1, (unsigned char*)((T*)p.dq + b * p.dq_sb + h0 * p.dq_sh), p.dq_sn * 2);
+      store_rows(acc1, (unsigned char*)((T*)p.dq + b * p.dq_sb + h0 * p.dq_sh + q_row0 * p.dq_sn), p.dq_sn * 2);
     } else {
-      store_rows(acc1, (unsigned char*)((T*)p.dk + b * p.dk_sb + hk * p.dk_sh), p.dk_sn * 2);
-      store_rows(acc2, (unsigned char*)((T*)p.dv + b * p.dv_sb + hk * p.dv_sh), p.dv_sn * 2);
+      store_rows(acc1, (unsigned char*)((T*)p.dk + b * p.dk_sb + hk * p.dk_sh + k_row0 * p.dk_sn), p.dk_sn * 2);
+      store_rows(acc2, (unsigned char*)((T*)p.dv + b * p.dv_sb + hk * p.dv_sh + k_row0 * p.dv_sn), p.dv_sn * 2);
     }
   }
   if (!TURN_RESULTS && !KEY_ST && st_valid) {
-    unsigned char* const dqb = (unsigned char*)((T*)p.dq + b * p.dq_sb + h0 * p.dq_sh) + (int64_t)st_row * p.dq_sn * 2;
+    unsigned char* const dqb = (unsigned char*)((T*)p.dq + b * p.dq_sb + h0 * p.dq_sh + q_row0 * p.dq_sn) + (int64_t)st_row * p.dq_sn * 2;
 #pragma unroll
     for (int db = 0; db < DB; ++db)
 #pragma unroll
@@ -635,8 +640,8 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 || PASS == HA_BWD_DQ_BLOCK ? 2
       }
   } else if (!TURN_RESULTS && (PASS == HA_BWD_DKV_EXACT || PASS == HA_BWD_DKV_BLOCK) && st_valid) {
     // complete sums (of the blocks: every key is in exactly one tile of the sorted order): straight to dk, dv
-    unsigned char* const dkb = (unsigned char*)((T*)p.dk + b * p.dk_sb + hk * p.dk_sh) + (int64_t)st_row * p.dk_sn * 2;
-    unsigned char* const dvb = (unsigned char*)((T*)p.dv + b * p.dv_sb + hk * p.dv_sh) + (int64_t)st_row * p.dv_sn * 2;
+    unsigned char* const dkb = (unsigned char*)((T*)p.dk + b * p.dk_sb + hk * p.dk_sh + k_row0 * p.dk_sn) + (int64_t)st_row * p.dk_sn * 2;
+    unsigned char* const dvb = (unsigned char*)((T*)p.dv + b * p.dv_sb + hk * p.dv_sh + k_row0 * p.dv_sn) + (int64_t)st_row * p.dv_sn * 2;
 #pragma unroll
     for (int db = 0; db < DB; ++db)
 #pragma unroll
@@ -670,7 +675,7 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 || PASS == HA_BWD_DQ_BLOCK ? 2
     // each of 64 rows.
     __syncthreads();
     float* const turn = reinterpret_cast<float*>(wave_s < 2 ? lds_y1[wave_s] : lds_y2[wave_s - 2]);
-    const int64_t head_base = (int64_t)(b * kv_heads + hk) * p.sample_size * D;
+    const int64_t head_base = ((int64_t)(b * kv_heads + hk) * p.segs + seg) * p.sample_size * D;
 #pragma unroll
     for (int which = 0; which < 2; ++which) {
       float* const dst = (which == 0 ? p.dk32 : p.dv32) + head_base;
@@ -710,20 +715,23 @@ __global__ __launch_bounds__(256) void ha_bwd_add_samples_kernel(const float* __
                                                                  const void* __restrict__ sampled_idx, int idx64,
                                                                  int64_t si_sb, int64_t si_sh, int kv_heads, int sample_size,
                                                                  int64_t dk_sb, int64_t dk_sh, int64_t dk_sn, int64_t dv_sb,
-                                                                 int64_t dv_sh, int64_t dv_sn, int64_t total_slots) {
+                                                                 int64_t dv_sh, int64_t dv_sn, int64_t total_slots,
+                                                                 int segs, int64_t seg_stride, int64_t k_seg_off) {
   typedef typename ElemTraits<T>::vec8 vec8;
   constexpr int PR = D / 8;
   const int64_t item = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   const int64_t gslot = item / PR;
   const int piece = (int)(item % PR);
   if (gslot >= total_slots) return;
-  const int64_t bh = gslot / sample_size;
-  const int slot = (int)(gslot - bh * sample_size);
+  const int64_t bhs = gslot / sample_size;   // (batch, kv head, segment)
+  const int slot = (int)(gslot - bhs * sample_size);
+  const int64_t bh = bhs / segs, seg = bhs - bh * segs;
   const int64_t b = bh / kv_heads, h = bh - b * kv_heads;
+  const int64_t row0 = k_seg_off + seg * seg_stride;
   int row = slot;
   float sum_k[8], sum_v[8];
-  const float* const bk = sk32 + (bh * sample_size) * D + piece * 8;
-  const float* const bv = sv32 + (bh * sample_size) * D + piece * 8;
+  const float* const bk = sk32 + (bhs * sample_size) * D + piece * 8;
+  const float* const bv = sv32 + (bhs * sample_size) * D + piece * 8;
   auto add_slot = [&](int s2) {
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
@@ -744,8 +752,8 @@ __global__ __launch_bounds__(256) void ha_bwd_add_samples_kernel(const float* __
   } else {
     add_slot(slot);
   }
-  vec8* const dst_k = reinterpret_cast<vec8*>(dk + b * dk_sb + h * dk_sh + row * dk_sn + piece * 8);
-  vec8* const dst_v = reinterpret_cast<vec8*>(dv + b * dv_sb + h * dv_sh + row * dv_sn + piece * 8);
+  vec8* const dst_k = reinterpret_cast<vec8*>(dk + b * dk_sb + h * dk_sh + (row0 + row) * dk_sn + piece * 8);
+  vec8* const dst_v = reinterpret_cast<vec8*>(dv + b * dv_sb + h * dv_sh + (row0 + row) * dv_sn + piece * 8);
   vec8 ok = *dst_k, ov = *dst_v;
 #pragma unroll
   for (int e = 0; e < 8; ++e) {
@@ -776,8 +784,8 @@ struct Workspace {
 
 Workspace carve(const ha_attn_operands& t, int64_t sample_size, void* base) {
   Workspace w;
-  const int64_t delta_bytes = align256(t.batch * t.heads * t.n_q * 8);
-  w.acc_floats = t.batch * (t.heads / t.kv_group) * sample_size * t.d;
+  const int64_t delta_bytes = align256(t.batch * t.heads * t.segs * t.n_q * 8);
+  w.acc_floats = t.batch * (t.heads / t.kv_group) * t.segs * sample_size * t.d;
   const int64_t acc_bytes = align256(w.acc_floats * 4);
   w.stats = (f32x2*)base;
   w.dk32 = (float*)((char*)base + delta_bytes);
@@ -788,8 +796,6 @@ Workspace carve(const ha_attn_operands& t, int64_t sample_size, void* base) {
 
 int check_grads(const ha_attn_operands& t, int64_t sample_size, const ha_attn_grads& g, const char* who) {
   HA_REQUIRE(g.dout && g.dq && g.dk && g.dv, HA_ERR_NULL, "%s: null gradient pointer", who);
-  HA_REQUIRE(t.segs == 1 && t.q_seg_offset == 0 && t.k_seg_offset == 0, HA_ERR_UNSUPPORTED,
-             "%s: the backward takes whole heads (segs == 1, no segment offsets)", who);
   const int64_t strides[] = {g.do_stride_b, g.do_stride_h, g.do_stride_n, g.dq_stride_b, g.dq_stride_h, g.dq_stride_n,
                              g.dk_stride_b, g.dk_stride_h, g.dk_stride_n, g.dv_stride_b, g.dv_stride_h, g.dv_stride_n};
   for (int64_t s : strides) HA_REQUIRE(s % 8 == 0, HA_ERR_SHAPE, "%s: gradient rows must be 16-byte aligned", who);
@@ -829,6 +835,7 @@ void fill_bwd_params(const ha_attn_operands& t, const ha_attn_grads& g, const Wo
   p.ki_sb = p.ki_sh = p.ki_sn = 0;
   p.si_sb = p.si_sh = 0;
   p.batch = (int)t.batch; p.heads = (int)t.heads; p.kv_group = (int)t.kv_group;
+  p.segs = (int)t.segs; p.seg_stride = t.seg_stride_rows; p.q_seg_off = t.q_seg_offset; p.k_seg_off = t.k_seg_offset;
   p.n_q = (int)t.n_q; p.n_k = (int)t.n_k;
   p.block_tiles = 1; p.sample_size = 0; p.smooth = 0; p.idx64 = 0;
   p.accumulate = g.accumulate != 0;
@@ -842,12 +849,13 @@ template <typename T, int D>
 int launch_add_samples(const ha_block_attn_args& a, const ha_attn_grads& g, const Workspace& w, hipStream_t stream) {
   const ha_attn_operands& t = a.t;
   const int64_t kv_heads = t.heads / t.kv_group;
-  const int64_t slots = t.batch * kv_heads * a.sample_size;
+  const int64_t slots = t.batch * kv_heads * t.segs * a.sample_size;
   const int64_t items = slots * (D / 8);
   hipLaunchKernelGGL((ha_bwd_add_samples_kernel<T, D>), dim3((unsigned)((items + 255) / 256)), dim3(256), 0, stream,
                      w.dk32, w.dv32, (T*)g.dk, (T*)g.dv, a.sampled_idx, (int)(a.idx_type == HA_IDX_I64),
                      a.sampled_stride_b, a.sampled_stride_h, (int)kv_heads, (int)a.sample_size, g.dk_stride_b,
-                     g.dk_stride_h, g.dk_stride_n, g.dv_stride_b, g.dv_stride_h, g.dv_stride_n, slots);
+                     g.dk_stride_h, g.dk_stride_n, g.dv_stride_b, g.dv_stride_h, g.dv_stride_n, slots, (int)t.segs,
+                     t.seg_stride_rows, t.k_seg_offset);
   return ha_launch_status("attention backward: sampled keys");
 }
 
@@ -866,7 +874,7 @@ int run_block_bwd(const ha_block_attn_args& a, const ha_attn_grads& g, hipStream
   p.sample_size = (int)a.sample_size;
   p.smooth = a.smooth_block != 0;
   p.idx64 = a.idx_type == HA_IDX_I64;
-  const int64_t bh = t.batch * t.heads, bhk = t.batch * (t.heads / t.kv_group);
+  const int64_t bh = t.batch * t.heads * t.segs, bhk = t.batch * (t.heads / t.kv_group) * t.segs;
   st = launch_pass<T, D, HA_BWD_DQ_BLOCK, false>(p, bh * (t.n_q / ST_ROWS), stream, "ha_block_attn_bwd: dq");
   if (st != HA_OK) return st;
   st = launch_pass<T, D, HA_BWD_DKV_BLOCK, false>(p, bhk * (t.n_k / ST_ROWS), stream, "ha_block_attn_bwd: dk, dv of the blocks");
@@ -897,7 +905,7 @@ int run_flash_bwd(const ha_attn_operands& t, bool causal, const ha_attn_grads& g
   int st;
   ha_attn_bwd_params p;
   fill_bwd_params(t, g, w, p);
-  const int64_t bh = t.batch * t.heads, bhk = t.batch * (t.heads / t.kv_group);
+  const int64_t bh = t.batch * t.heads * t.segs, bhk = t.batch * (t.heads / t.kv_group) * t.segs;
   const int64_t q_tiles = (t.n_q + ST_ROWS - 1) / ST_ROWS, k_tiles = (t.n_k + ST_ROWS - 1) / ST_ROWS;
   if (causal) {
     st = launch_pass<T, D, HA_BWD_DQ_EXACT, true>(p, bh * q_tiles, stream, "ha_flash_attn_bwd: dq");
@@ -915,8 +923,8 @@ int run_flash_bwd(const ha_attn_operands& t, bool causal, const ha_attn_grads& g
 
 extern "C" int64_t ha_attn_bwd_workspace_bytes(const ha_attn_operands* t, int64_t sample_size) {
   if (!t || t->batch <= 0 || t->heads <= 0 || t->n_q <= 0 || t->n_k <= 0 || t->d <= 0 || t->kv_group <= 0 ||
-      t->heads % t->kv_group != 0 || sample_size < 0)
-    return ha_fail(HA_ERR_SHAPE, "ha_attn_bwd_workspace_bytes: sizes must be positive, kv_group dividing heads");
+      t->heads % t->kv_group != 0 || sample_size < 0 || t->segs < 1)
+    return ha_fail(HA_ERR_SHAPE, "ha_attn_bwd_workspace_bytes: sizes must be positive, kv_group dividing heads, segs >= 1");
   return carve(*t, sample_size, nullptr).bytes;
 }
 

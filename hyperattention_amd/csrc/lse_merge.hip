@@ -1,8 +1,8 @@
 // Merge of two partial attentions computed over disjoint key sets.
 // Stands in for add_self_attentions (src/attn_utils.py:6-24 of the reference):
 //   c = 1 / (1 + exp(lse2 - lse1)); attn = c*attn1 + (1-c)*attn2; lse = lse1 - log(c + eps).
-// The arithmetic here is fp32 throughout (the reference rounds c to fp16/bf16 first), with the
-// same eps = 2^-23 inside the log.  One 8-element piece (16 bytes) per lane.
+// c is rounded to the attention's type before it is used, as the reference does (src/attn_utils.py:21);
+// the rest is fp32, with the same eps = 2^-23 inside the log.  One 8-element piece (16 bytes) per lane.
 #include "ha_common.h"
 
 namespace {
@@ -18,7 +18,7 @@ __global__ __launch_bounds__(256) void lse_merge_kernel(const T* a1, const float
   const int piece = (int)(item % pieces);
   if (row >= rows) return;
   const float x1 = l1[row * ls1], x2 = l2[row * ls2];
-  const float c = 1.0f / (1.0f + __expf(x2 - x1));
+  const float c = (float)(T)(1.0f / (1.0f + __expf(x2 - x1)));
   const vec8 v1 = *reinterpret_cast<const vec8*>(a1 + row * s1 + piece * 8);
   const vec8 v2 = *reinterpret_cast<const vec8*>(a2 + row * s2 + piece * 8);
   vec8 r;
@@ -131,4 +131,122 @@ extern "C" int ha_lse_merge_segments(const void* attn1, const float* lse1, const
                        attn1_seg_stride, attn1_row_stride, attn2_seg_stride, attn2_row_stride, out_seg_stride,
                        out_row_stride, lse1_seg_stride, lse2_seg_stride, lse_out_seg_stride, weight_seg_stride);
   return ha_launch_status("ha_lse_merge_segments");
+}
+
+// All merges of the causal recursion in one pass over the rows.
+// A row of a (batch, heads, n, d) tensor takes part in the un-masked call of level j (segments of n / 2^j
+// rows) iff it lies in the second half of its segment.  Deepest level first, as the recursion returns
+// (hyper_attention.py:86-89), its leaf result is merged with the results of those calls, each merge with the
+// arithmetic of lse_merge_segments_kernel (weight rounded to the attention's type, merged rows rounded
+// after every level).  All per-level arrays have the layout of the whole tensors; rows outside a level's
+// second halves are neither read nor written.
+//
+// For a backward pass the row's weights are turned into shifted log-sum-exps on the way: the gradient of the
+// output reaches the call of level j scaled by w_j = (1 - c_j) * prod of c_i over the shallower levels i the
+// row takes part in, and the leaf by the product of all its c_i.  A call's gradients depend on its output
+// gradient only through P = exp(s - lse) times that gradient, so scaling the gradient by w equals handing the
+// call lse - log(w): those are written to shifted[j] and leaf_shifted (w = 0 gives +inf: P = 0).
+namespace {
+
+constexpr int MERGE_MAX_LEVELS = 24;
+
+struct MergeLevels {
+  const void* o_un[MERGE_MAX_LEVELS];
+  const float* lse_un[MERGE_MAX_LEVELS];
+  float* shifted[MERGE_MAX_LEVELS];
+  int levels;
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void lse_merge_levels_kernel(const T* __restrict__ o_leaf, const float* __restrict__ lse_leaf,
+                                                               T* __restrict__ out, float* __restrict__ lse_out,
+                                                               float* __restrict__ leaf_shifted, MergeLevels lv,
+                                                               int64_t rows, int64_t n, int pieces) {
+  typedef typename ElemTraits<T>::vec8 vec8;
+  const int64_t item = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t row = item / pieces;
+  const int piece = (int)(item % pieces);
+  if (row >= rows) return;
+  // leaf number of the row inside its sequence: its bit (levels - 1 - j) says which half of its level-j
+  // segment the row is in (such a half is 2^(levels - 1 - j) leaves long)
+  const uint32_t leaf_no = (uint32_t)(row % n) / (uint32_t)(n >> lv.levels);
+  const int64_t at = row * pieces * 8 + piece * 8;
+  float x = lse_leaf[row];
+  const float x_leaf = x;
+  vec8 r = *reinterpret_cast<const vec8*>(o_leaf + at);
+  float c_of[MERGE_MAX_LEVELS], x_of[MERGE_MAX_LEVELS];
+#pragma unroll
+  for (int j = MERGE_MAX_LEVELS - 1; j >= 0; --j) {
+    c_of[j] = 1.0f;
+    x_of[j] = 0.0f;
+    if (j < lv.levels && ((leaf_no >> (lv.levels - 1 - j)) & 1u)) {
+      const float x2 = lv.lse_un[j][row];
+      const float c = (float)(T)(1.0f / (1.0f + __expf(x2 - x)));
+      const vec8 v2 = *reinterpret_cast<const vec8*>((const T*)lv.o_un[j] + at);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) r[e] = (T)(c * (float)r[e] + (1.0f - c) * (float)v2[e]);
+      x = x - __logf(c + 1.1920929e-07f);
+      c_of[j] = c;
+      x_of[j] = x2;
+    }
+  }
+  *reinterpret_cast<vec8*>(out + at) = r;
+  if (piece != 0) return;
+  lse_out[row] = x;
+  if (!leaf_shifted) return;
+  float log_w = 0.0f;  // log of the product of the weights c of the shallower levels
+#pragma unroll
+  for (int j = 0; j < MERGE_MAX_LEVELS; ++j) {
+    if (j < lv.levels && ((leaf_no >> (lv.levels - 1 - j)) & 1u)) {
+      lv.shifted[j][row] = x_of[j] - log1pf(-c_of[j]) - log_w;
+      log_w += logf(c_of[j]);
+    }
+  }
+  leaf_shifted[row] = x_leaf - log_w;
+}
+
+}  // namespace
+
+extern "C" int ha_lse_merge_levels(const void* o_leaf, const float* lse_leaf, const void* const* o_un,
+                                   const float* const* lse_un, float* const* lse_shifted, float* leaf_shifted,
+                                   void* out, float* lse_out, int levels, int64_t batch_heads, int64_t n, int64_t d,
+                                   int dtype, void* stream) {
+  HA_REQUIRE(o_leaf && lse_leaf && out && lse_out && (levels == 0 || (o_un && lse_un)), HA_ERR_NULL,
+             "ha_lse_merge_levels: null pointer");
+  HA_REQUIRE(dtype == HA_F16 || dtype == HA_BF16, HA_ERR_DTYPE, "ha_lse_merge_levels: Only support fp16 and bf16");
+  HA_REQUIRE(levels >= 0 && levels <= MERGE_MAX_LEVELS, HA_ERR_UNSUPPORTED, "ha_lse_merge_levels: at most %d levels",
+             MERGE_MAX_LEVELS);
+  HA_REQUIRE(batch_heads > 0 && n > 0 && d > 0 && d % 8 == 0, HA_ERR_SHAPE,
+             "ha_lse_merge_levels: sizes must be positive and d % 8 == 0");
+  HA_REQUIRE((n >> levels) << levels == n, HA_ERR_SHAPE, "ha_lse_merge_levels: n must be divisible by 2^levels");
+  HA_REQUIRE((leaf_shifted != nullptr) == (lse_shifted != nullptr) || levels == 0, HA_ERR_NULL,
+             "ha_lse_merge_levels: leaf_shifted and lse_shifted go together");
+  HA_REQUIRE(((uintptr_t)o_leaf % 16) == 0 && ((uintptr_t)out % 16) == 0, HA_ERR_SHAPE,
+             "ha_lse_merge_levels: tensors must be 16-byte aligned");
+  HA_REQUIRE(out != o_leaf && lse_out != lse_leaf, HA_ERR_UNSUPPORTED, "ha_lse_merge_levels: not in place");
+  MergeLevels lv;
+  lv.levels = levels;
+  for (int j = 0; j < MERGE_MAX_LEVELS; ++j) {
+    lv.o_un[j] = nullptr; lv.lse_un[j] = nullptr; lv.shifted[j] = nullptr;
+  }
+  for (int j = 0; j < levels; ++j) {
+    HA_REQUIRE(o_un[j] && lse_un[j] && (!leaf_shifted || lse_shifted[j]), HA_ERR_NULL,
+               "ha_lse_merge_levels: null pointer for level %d", j);
+    HA_REQUIRE(((uintptr_t)o_un[j] % 16) == 0, HA_ERR_SHAPE, "ha_lse_merge_levels: tensors must be 16-byte aligned");
+    lv.o_un[j] = o_un[j];
+    lv.lse_un[j] = lse_un[j];
+    lv.shifted[j] = leaf_shifted ? lse_shifted[j] : nullptr;
+  }
+  const int pieces = (int)(d / 8);
+  const int64_t rows = batch_heads * n, items = rows * pieces;
+  HA_REQUIRE((items + 255) / 256 < (1ll << 31), HA_ERR_SHAPE, "ha_lse_merge_levels: too many rows");
+  dim3 grid((unsigned)((items + 255) / 256));
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == HA_F16)
+    hipLaunchKernelGGL((lse_merge_levels_kernel<f16_t>), grid, dim3(256), 0, s, (const f16_t*)o_leaf, lse_leaf,
+                       (f16_t*)out, lse_out, leaf_shifted, lv, rows, n, pieces);
+  else
+    hipLaunchKernelGGL((lse_merge_levels_kernel<bf16_t>), grid, dim3(256), 0, s, (const bf16_t*)o_leaf, lse_leaf,
+                       (bf16_t*)out, lse_out, leaf_shifted, lv, rows, n, pieces);
+  return ha_launch_status("ha_lse_merge_levels");
 }

@@ -1,15 +1,15 @@
 """HyperAttention module: same constructor and forward signature as the reference
 (hyper_attention.py:9-132), computed by the HIP library.
 
-Contiguous inputs whose causal recursion only meets even lengths take one library call
-(ha_forward: hash once, all sorts in one batch, leaves, then each level merged in place).  Other
-shapes (an odd length somewhere in the recursion, more than 8 projections) are composed here from
-the same HIP operators, following the reference's recursion step by step.
+Inputs whose causal recursion only meets even lengths take one library call (ha_forward: q and k
+hashed in one launch, the rows ranked once for all levels, leaves, then each level merged in place).
+Other shapes (an odd length somewhere in the recursion) are composed here from the same HIP operators,
+following the reference's recursion step by step.
 
 With inputs that require grad the forward keeps what the backward needs: the non-causal case is one
-differentiable operator call, the causal recursion with even lengths runs on views of the tensors
-with the calls' gradients accumulated by the kernels (_CausalRecursionFunc), anything else operator
-by operator under torch autograd.
+differentiable operator call, the causal recursion with even lengths runs on segments of the whole
+tensors with the calls' gradients accumulated by the kernels (_CausalRecursionFunc), anything else
+operator by operator under torch autograd.
 """
 from __future__ import annotations
 
@@ -23,78 +23,113 @@ from .angular_lsh import AngularLSH
 
 class _CausalRecursionFunc(torch.autograd.Function):
     """The causal divide-and-conquer (hyper_attention.py:51-96) with its gradient, for lengths that stay
-    even down to the leaves.
+    even down to the leaves; key and value may have fewer heads than the query (grouped queries).
 
     Same arithmetic as the reference's recursion under autograd: exact causal attention on the leaves,
     one un-masked call per level on (second-half queries, first-half keys/values), merges with the
     weight rounded to the attention's type (src/attn_utils.py:21-23), and log-sum-exps that carry no
-    gradient (src/hyper_attn_triton.py:922-945).  What differs is the bookkeeping: every call reads and
-    writes strided views of the (batch, heads, n, d) tensors through the C entry points, the merges
-    run in place, and in the backward the gradients of the calls are accumulated by the kernels
-    (`accumulate`), so there are no concatenations, zero-padded slice gradients or gradient additions.
+    gradient (src/hyper_attn_triton.py:922-945).  What differs is the bookkeeping.  All rows are hashed
+    in one launch and ranked once for all levels (ha_forward_sort).  Every call reads and writes its
+    segments of the whole (batch, heads, n, d) tensors through the C entry points; the result of level j
+    is kept in o_un[j] at the rows of the output it belongs to.  One pass merges the leaf and level
+    results of every row (ha_lse_merge_levels) and, on the way, turns the merge weights into the shifted
+    log-sum-exps that the backward hands to each call in place of a weighted copy of the output gradient.
+    In the backward the gradients of the calls are accumulated by the kernels (`accumulate`), so there
+    are no concatenations, zero-padded slice gradients or gradient additions.
     """
 
     @staticmethod
-    def forward(ctx, module, scale, query, key, value):
+    def _segments(t, lens, j, leaves=False):
+        """Point the operands at the segments of level j: the un-masked call on (second-half queries,
+        first-half keys) of every segment of lens[j] rows, or the leaves."""
+        if leaves:
+            t.n_q = t.n_k = lens[j]
+            t.segs, t.seg_stride_rows, t.q_seg_offset, t.k_seg_offset = 1 << j, lens[j], 0, 0
+        else:
+            half = lens[j + 1]
+            t.n_q = t.n_k = half
+            t.segs, t.seg_stride_rows, t.q_seg_offset, t.k_seg_offset = 1 << j, lens[j], half, 0
+        return t
+
+    @staticmethod
+    def _level_args(module, query, key, value, out, lse, scale, lens, j, q_idx, k_idx, sampled):
+        """BlockAttnArgs of the hashed un-masked call of level j on the whole tensors."""
+        b, h, n, d = query.shape
+        hk, half, segs = key.shape[1], lens[j + 1], 1 << j
+        a = _lib.BlockAttnArgs()
+        a.t = _CausalRecursionFunc._segments(
+            ops._operands(query, key, value, out, lse, scale, layout_bnhd=False, lse_row_stride=n), lens, j)
+        a.q_idx, a.k_idx, a.idx_type = q_idx.data_ptr(), k_idx.data_ptr(), ops._idx_code(q_idx)
+        a.q_idx_stride_b, a.q_idx_stride_h, a.q_idx_stride_n = h * segs * half, segs * half, 1
+        a.k_idx_stride_b, a.k_idx_stride_h, a.k_idx_stride_n = hk * segs * half, segs * half, 1
+        a.sampled_stride_b = a.sampled_stride_h = 0
+        if sampled is not None:
+            a.sampled_idx = sampled.data_ptr()
+        a.block_size, a.sample_size = module.block_size, module.sample_size
+        a.smooth_block, a.accumulate = int(bool(module.smooth_block)), 0
+        return a
+
+    @staticmethod
+    def _sampled(module, query, lens, hashed):
+        """The module's explicit sample list as an int32 device tensor, checked against the shortest hashed
+        level (the list serves every level)."""
+        if module.sampled_idx is None or not any(hashed):
+            return None
+        ops.check_sampled_idx(module.sampled_idx, min(lens[j + 1] for j in range(len(hashed)) if hashed[j]))
+        sampled = module.sampled_idx.to(device=query.device, dtype=torch.int32).contiguous()
+        assert sampled.shape == (module.sample_size,), "inside the causal recursion sampled_idx is one (sample_size,) list"
+        return sampled
+
+    @staticmethod
+    def forward(ctx, module, scale, query, key, value, proj):
         b, h, n, d = query.shape
         lens = [n]
         while lens[-1] > module.min_seq_len:
             lens.append(lens[-1] // 2)
         levels = len(lens) - 1
         lib, stream = _lib.lib(), ops._stream(query)
-        f32 = dict(device=query.device, dtype=torch.float32)
-        heads = lambda x, j: x.view(b, h << j, lens[j], x.shape[-1])
+        dev = query.device
+        f32 = dict(device=dev, dtype=torch.float32)
+        hashed = [not module.min_seq_len > lens[j + 1] for j in range(levels)]  # hyper_attention.py:109
+        segments = _CausalRecursionFunc._segments
+        operands = lambda out, lse: ops._operands(query, key, value, out, lse, scale, layout_bnhd=False, lse_row_stride=n)
 
-        with torch.cuda.device(query.device):
+        q_idx = k_idx = [None] * levels
+        if any(hashed):
+            q_idx, k_idx = ops.forward_sort(query, key, proj, causal=True,
+                                            lsh_num_projs=module.lsh_num_projs, min_seq_len=module.min_seq_len)
+        sampled = _CausalRecursionFunc._sampled(module, query, lens, hashed)
+        o_leaf, lse_leaf = torch.empty_like(query), torch.empty((b, h, n), **f32)
+        o_un = torch.empty((levels, b, h, n, d), device=dev, dtype=query.dtype)
+        lse_un = torch.empty((levels, b, h, n), **f32)
+        lse_shifted, leaf_shifted = torch.empty((levels, b, h, n), **f32), torch.empty((b, h, n), **f32)
+        out, lse = torch.empty_like(query), torch.empty((b, h, n), **f32)
+        with torch.cuda.device(dev):
             # leaves: exact causal attention on every segment of lens[levels] rows
-            o_leaf, lse_leaf = torch.empty_like(query), torch.empty((b, h, n), **f32)
-            t = ops._operands(heads(query, levels), heads(key, levels), heads(value, levels), heads(o_leaf, levels),
-                              lse_leaf.view(b, h << levels, lens[levels]), scale, layout_bnhd=False,
-                              lse_row_stride=lens[levels])
+            t = segments(operands(o_leaf, lse_leaf), lens, levels, leaves=True)
             _lib.check(lib.ha_flash_attn_fwd(ctypes.byref(t), 1, stream))
-            out, lse = o_leaf.clone(), lse_leaf.clone()
-
-            # a row's bucket does not depend on the level: hash once, sort per level
-            hashed = [j for j in range(levels) if not module.min_seq_len > lens[j + 1]]
-            if hashed:
-                buckets_q, buckets_k = module.lsh.hash(query), module.lsh.hash(key)
-            per_level = []
-            for j in reversed(range(levels)):  # deepest level first, as the recursion returns
-                H, half = h << j, lens[j + 1]
-                q2 = query.view(b, H, 2, half, d)[:, :, 1]
-                k1 = key.view(b, H, 2, half, d)[:, :, 0]
-                v1 = value.view(b, H, 2, half, d)[:, :, 0]
-                o_un, lse_un = torch.empty((b, H, half, d), device=query.device, dtype=query.dtype), torch.empty((b, H, half), **f32)
-                if module.min_seq_len > half:  # hyper_attention.py:109
-                    q_idx = k_idx = None
-                    t = ops._operands(q2, k1, v1, o_un, lse_un, scale, layout_bnhd=False, lse_row_stride=half)
-                    _lib.check(lib.ha_flash_attn_fwd(ctypes.byref(t), 0, stream))
-                else:
-                    num_keys = 1 << module.lsh_num_projs
-                    q_idx = ops.bucket_argsort(buckets_q.view(b, H, 2, half)[:, :, 1], num_keys, torch.int32)
-                    k_idx = ops.bucket_argsort(buckets_k.view(b, H, 2, half)[:, :, 0], num_keys, torch.int32)
-                    a, keep = ops._block_attn_args(q2, k1, v1, o_un, lse_un, q_idx, k_idx, module.block_size,
-                                                   module.sample_size, scale, module.smooth_block, module.sampled_idx,
-                                                   layout_bnhd=False)
+            for j in range(levels):
+                if hashed[j]:
+                    a = _CausalRecursionFunc._level_args(module, query, key, value, o_un[j], lse_un[j], scale, lens, j,
+                                                         q_idx[j], k_idx[j], sampled)
                     _lib.check(lib.ha_block_attn_fwd(ctypes.byref(a), stream))
-                # merge into the second halves, in place; c: the weight of what was there (fp32 copy of the
-                # weight rounded to the attention's type)
-                out2 = out.view(b, H, 2, half, d)[:, :, 1]
-                lse2 = lse.view(b, H, 2, half)[:, :, 1]
-                c = torch.empty((b, H, half), **f32)
-                _lib.check(lib.ha_lse_merge_segments(
-                    out2.data_ptr(), lse2.data_ptr(), o_un.data_ptr(), lse_un.data_ptr(), out2.data_ptr(),
-                    lse2.data_ptr(), c.data_ptr(), b * H, half, d, 2 * half * d, d, half * d, d, 2 * half * d, d,
-                    2 * half, half, 2 * half, half, ops._dtype_code(query), stream))
-                per_level.append((j, o_un, lse_un, c, q_idx, k_idx))
+                else:
+                    t = segments(operands(o_un[j], lse_un[j]), lens, j)
+                    _lib.check(lib.ha_flash_attn_fwd(ctypes.byref(t), 0, stream))
+            ptrs = lambda x: (ctypes.c_void_p * max(levels, 1))(*[x[j].data_ptr() for j in range(levels)])
+            _lib.check(lib.ha_lse_merge_levels(
+                o_leaf.data_ptr(), lse_leaf.data_ptr(), ptrs(o_un), ptrs(lse_un), ptrs(lse_shifted),
+                leaf_shifted.data_ptr(), out.data_ptr(), lse.data_ptr(), levels, b * h, n, d, ops._dtype_code(query),
+                stream))
 
-        tensors = [query, key, value, o_leaf, lse_leaf]
-        layout = []
-        for j, o_un, lse_un, c, q_idx, k_idx in per_level:
-            layout.append((j, q_idx is not None))
-            tensors += [o_un, lse_un, c] + ([q_idx, k_idx] if q_idx is not None else [])
+        tensors = [query, key, value, o_leaf, leaf_shifted, o_un, lse_shifted]
+        if sampled is not None:
+            tensors.append(sampled)
+        for j in range(levels):
+            if hashed[j]:
+                tensors += [q_idx[j], k_idx[j]]
         ctx.save_for_backward(*tensors)
-        ctx.layout, ctx.lens, ctx.module, ctx.scale = layout, lens, module, scale
+        ctx.hashed, ctx.lens, ctx.module, ctx.scale, ctx.has_sampled = hashed, lens, module, scale, sampled is not None
         lse = lse.unsqueeze(-1)
         ctx.mark_non_differentiable(lse)
         return out, lse
@@ -102,70 +137,43 @@ class _CausalRecursionFunc(torch.autograd.Function):
     @staticmethod
     def backward(ctx, dout, dlse=None):
         saved = list(ctx.saved_tensors)
-        query, key, value, o_leaf, lse_leaf = saved[:5]
-        rest = saved[5:]
-        module, scale, lens = ctx.module, ctx.scale, ctx.lens
+        query, key, value, o_leaf, leaf_shifted, o_un, lse_shifted = saved[:7]
+        rest = saved[7:]
+        sampled = rest.pop(0) if ctx.has_sampled else None
+        module, scale, lens, hashed = ctx.module, ctx.scale, ctx.lens, ctx.hashed
         b, h, n, d = query.shape
         levels = len(lens) - 1
         lib, stream = _lib.lib(), ops._stream(query)
-        heads = lambda x, j: x.view(b, h << j, lens[j], x.shape[-1])
-
-        per_level = {}
-        for j, hashed in ctx.layout:
-            o_un, lse_un, c = rest[:3]
-            q_idx, k_idx = (rest[3], rest[4]) if hashed else (None, None)
-            rest = rest[5:] if hashed else rest[3:]
-            per_level[j] = (o_un, lse_un, c, q_idx, k_idx)
+        segments = _CausalRecursionFunc._segments
 
         with torch.cuda.device(query.device):
             # The gradient of the output splits at every merge, from the top level down: (1 - c) of it goes
             # to the un-masked call of the level, c of it further down.  A call's gradients are linear in
             # the output gradient it is given, and that enters only through P = exp(s - lse): weighting a
             # row's output gradient by w equals giving the call the log-sum-exp lse - log(w) for that row
-            # (w = 0: lse = +inf, P = 0).  So every call gets the output gradient as it is and a shifted
-            # copy of its small log-sum-exp array, and no weighted copy of the gradient is ever made.
+            # (w = 0: lse = +inf, P = 0).  So every call gets the output gradient as it is and the shifted
+            # log-sum-exps that the forward's merge pass wrote, and no weighted copy of the gradient is made.
             dout = dout.contiguous()
-            log_w = torch.zeros((b, h, n), device=query.device, dtype=torch.float32)
-            lse_shifted = {}
-            for j in range(levels):
-                H, half = h << j, lens[j + 1]
-                lse_un, c = per_level[j][1], per_level[j][2]
-                log_w2 = log_w.view(b, H, 2, half)[:, :, 1]
-                lse_shifted[j] = lse_un - torch.log1p(-c) - log_w2
-                log_w2.add_(torch.log(c))
-            lse_leaf = lse_leaf - log_w
-
             dq, dk, dv = torch.empty_like(query), torch.empty_like(key), torch.empty_like(value)
-            # leaves first: they write every row of dq, dk, dv; the levels then add to their views
-            t = ops._operands(heads(query, levels), heads(key, levels), heads(value, levels), heads(o_leaf, levels),
-                              lse_leaf.view(b, h << levels, lens[levels]), scale, layout_bnhd=False,
-                              lse_row_stride=lens[levels])
-            g, ws = ops._attn_grads(t, heads(dout, levels), heads(dq, levels), heads(dk, levels), heads(dv, levels),
-                                    layout_bnhd=False)
+            # leaves first: they write every row of dq, dk, dv; the levels then add to their segments
+            t = segments(ops._operands(query, key, value, o_leaf, leaf_shifted, scale, layout_bnhd=False,
+                                       lse_row_stride=n), lens, levels, leaves=True)
+            g, ws = ops._attn_grads(t, dout, dq, dk, dv, layout_bnhd=False)
             _lib.check(lib.ha_flash_attn_bwd(ctypes.byref(t), 1, ctypes.byref(g), stream))
             for j in range(levels):
-                H, half = h << j, lens[j + 1]
-                o_un, _, _, q_idx, k_idx = per_level[j]
-                lse_un = lse_shifted[j]
-                do2 = dout.view(b, H, 2, half, d)[:, :, 1]
-                q2 = query.view(b, H, 2, half, d)[:, :, 1]
-                k1 = key.view(b, H, 2, half, d)[:, :, 0]
-                v1 = value.view(b, H, 2, half, d)[:, :, 0]
-                dq2 = dq.view(b, H, 2, half, d)[:, :, 1]
-                dk1 = dk.view(b, H, 2, half, d)[:, :, 0]
-                dv1 = dv.view(b, H, 2, half, d)[:, :, 0]
-                if q_idx is None:
-                    t = ops._operands(q2, k1, v1, o_un, lse_un, scale, layout_bnhd=False, lse_row_stride=half)
-                    g, ws = ops._attn_grads(t, do2, dq2, dk1, dv1, layout_bnhd=False, accumulate=True)
-                    _lib.check(lib.ha_flash_attn_bwd(ctypes.byref(t), 0, ctypes.byref(g), stream))
-                else:
-                    a, keep = ops._block_attn_args(q2, k1, v1, o_un, lse_un, q_idx, k_idx, module.block_size,
-                                                   module.sample_size, scale, module.smooth_block, module.sampled_idx,
-                                                   layout_bnhd=False)
-                    g, ws = ops._attn_grads(a.t, do2, dq2, dk1, dv1, layout_bnhd=False, accumulate=True,
+                if hashed[j]:
+                    q_idx, k_idx = rest.pop(0), rest.pop(0)
+                    a = _CausalRecursionFunc._level_args(module, query, key, value, o_un[j], lse_shifted[j], scale,
+                                                         lens, j, q_idx, k_idx, sampled)
+                    g, ws = ops._attn_grads(a.t, dout, dq, dk, dv, layout_bnhd=False, accumulate=True,
                                             sample_size=module.sample_size)
                     _lib.check(lib.ha_block_attn_bwd(ctypes.byref(a), ctypes.byref(g), stream))
-        return None, None, dq, dk, dv
+                else:
+                    t = segments(ops._operands(query, key, value, o_un[j], lse_shifted[j], scale, layout_bnhd=False,
+                                               lse_row_stride=n), lens, j)
+                    g, ws = ops._attn_grads(t, dout, dq, dk, dv, layout_bnhd=False, accumulate=True)
+                    _lib.check(lib.ha_flash_attn_bwd(ctypes.byref(t), 0, ctypes.byref(g), stream))
+        return None, None, dq, dk, dv, None
 
 
 class HyperAttention(torch.nn.Module):
@@ -210,27 +218,30 @@ class HyperAttention(torch.nn.Module):
         assert n_query == n_key
 
         dim_v = value.shape[-1]
+        proj = self.lsh.proj_dir
         if dim not in ops.KERNEL_HEAD_DIMS or dim_v != dim:
             # head dims the kernels are not built for (and a value dim different from the q/k dim) run
             # zero-padded: zero columns change neither the projections, nor q.k, nor the wanted outputs
             assert dim <= 128 and dim_v <= 128, "FlashAttention only support head dimensions up to 128"
             wide = ops.padded_head_dim(max(dim, dim_v))
             pad = lambda x: torch.nn.functional.pad(x, (0, wide - x.shape[-1]))
-            proj = self.lsh.proj_dir
-            self.lsh.proj_dir = torch.nn.functional.pad(proj, (0, 0, 0, wide - dim))
-            try:
-                res = self.forward(pad(query), pad(key), pad(value), scale, causal, True)
-            finally:
-                self.lsh.proj_dir = proj
-            attn, lse = res[0][..., :dim_v], res[1]
-            return (attn, lse) if return_lse else attn
+            attn, lse = self._forward_built(pad(query), pad(key), pad(value), scale, causal,
+                                            torch.nn.functional.pad(proj, (0, 0, 0, wide - dim)))
+            attn = attn[..., :dim_v]
+        else:
+            attn, lse = self._forward_built(query, key, value, scale, causal, proj)
+        return (attn, lse) if return_lse else attn
 
+    def _forward_built(self, query, key, value, scale, causal, proj):
+        """forward() for a head dim the kernels are built for, value dim equal to it; proj: the
+        (1, 1, dim, lsh_num_projs) projection to hash with.  Returns (attn, lse)."""
+        n_key = key.shape[2]
         # gradients are taken operator by operator, as in the reference (each attention operator has its own
         # backward and the merges are differentiable tensor arithmetic); the one-call forward has none
         if (ops.forward_plan_supported(n_key, self.min_seq_len, causal is not False, self.lsh_num_projs)
                 and not ops._wants_grad(query, key, value)):
             attn, lse = ops.hyper_forward(
-                query, key, value, self.lsh.proj_dir, scale=scale, causal=causal is not False,
+                query, key, value, proj, scale=scale, causal=causal is not False,
                 lsh_num_projs=self.lsh_num_projs, block_size=self.block_size, sample_size=self.sample_size,
                 min_seq_len=self.min_seq_len, smooth_block=self.smooth_block, sampled_idx=self.sampled_idx)
             if causal is not False and n_key <= self.min_seq_len:
@@ -239,6 +250,12 @@ class HyperAttention(torch.nn.Module):
                 lse = torch.nn.functional.pad(lse, (0, n_rounded - n_key))
             else:
                 lse = lse.unsqueeze(-1)
+        elif (causal is not False and n_key > self.min_seq_len
+              and ops.forward_plan_supported(n_key, self.min_seq_len, True, self.lsh_num_projs)):
+            # gradients wanted and every level has an even length: the recursion and its gradient on
+            # segments of the whole tensors, grouped-query heads as they are
+            attn, lse = _CausalRecursionFunc.apply(self, scale, query.contiguous(), key.contiguous(), value.contiguous(),
+                                                   proj)
         else:
             if key.shape[1] != query.shape[1]:
                 # grouped-query inputs on the operator-by-operator path: it follows the reference, which
@@ -246,24 +263,20 @@ class HyperAttention(torch.nn.Module):
                 group = query.shape[1] // key.shape[1]
                 key, value = key.repeat_interleave(group, dim=1), value.repeat_interleave(group, dim=1)
             query, key, value = query.contiguous(), key.contiguous(), value.contiguous()
-            if (causal is not False and n_key > self.min_seq_len and ops._wants_grad(query, key, value)
-                    and ops.forward_plan_supported(n_key, self.min_seq_len, True, 8)):
-                # every level has an even length: the recursion and its gradient on views, in place
-                attn, lse = _CausalRecursionFunc.apply(self, scale, query, key, value)
-            else:
-                attn, lse = self._forward_composed(query, key, value, scale, causal)
+            attn, lse = self._forward_composed(query, key, value, scale, causal, proj)
 
-        if not return_lse:
-            return attn
-        else:
-            return attn, lse
+        if causal is not False and n_key <= self.min_seq_len and lse.dim() == 4:
+            # a top-level leaf: the exact kernel's padded 3-d lse, whichever path computed it
+            n_rounded = -(-n_key // 128) * 128
+            lse = torch.nn.functional.pad(lse.squeeze(-1), (0, n_rounded - n_key))
+        return attn, lse
 
     # ---- the reference's recursion, operator by operator (shapes ha_forward does not take) --------
-    def _forward_composed(self, query, key, value, scale, causal):
+    def _forward_composed(self, query, key, value, scale, causal, proj=None):
         batch_size, n_heads, n_key, dim = key.shape
         n_query = query.shape[2]
         if causal is False:
-            return self.forward_no_causal_mask(query, key, value, scale)
+            return self.forward_no_causal_mask(query, key, value, scale, proj)
         if n_key <= self.min_seq_len:
             attn, lse = ops.flash_attn_func(query.transpose(1, 2), key.transpose(1, 2), value.transpose(1, 2),
                                             None, True, scale)
@@ -276,11 +289,11 @@ class HyperAttention(torch.nn.Module):
         q_bd = query.view(batch_size, 2 * n_heads, half, query.shape[-1])
         k_bd = key.view(batch_size, 2 * n_heads, half, key.shape[-1])
         v_bd = value.view(batch_size, 2 * n_heads, half, value.shape[-1])
-        attn_bd, lse_bd = self._forward_composed(q_bd, k_bd, v_bd, scale, True)
+        attn_bd, lse_bd = self._forward_composed(q_bd, k_bd, v_bd, scale, True, proj)
         attn_bd = attn_bd.contiguous().view(batch_size, n_heads, -1, value.shape[-1])
         lse_bd = lse_bd.contiguous().view(batch_size, n_heads, -1, 1)
         attn_unmasked, lse_unmasked = self.forward_no_causal_mask(
-            query[:, :, half:, :], key[:, :, :half, :], value[:, :, :half, :], scale)
+            query[:, :, half:, :], key[:, :, :half, :], value[:, :, :half, :], scale, proj)
         attn_down, lse_down = ops.add_self_attentions(attn_bd[:, :, half:, :], lse_bd[:, :, half:, :],
                                                       attn_unmasked, lse_unmasked)
         attn = torch.cat((attn_bd[:, :, :half, :], attn_down), dim=-2)
@@ -290,9 +303,10 @@ class HyperAttention(torch.nn.Module):
             lse = lse[:, :, :-1, :]
         return attn, lse
 
-    def forward_no_causal_mask(self, query, key, value, scale):
+    def forward_no_causal_mask(self, query, key, value, scale, proj=None):
         """
             - sequence lengths must be divisible by block_size
+            - proj (not in the reference): projection to hash with instead of the module's own
         """
         batch_size, head_size, n_query, dim = query.shape
 
@@ -302,8 +316,8 @@ class HyperAttention(torch.nn.Module):
             lse = lse[:, :, :n_query]
         else:
             num_keys = 1 << self.lsh_num_projs
-            query_sort_idx = ops.bucket_argsort(self.lsh.hash(query), num_keys)
-            key_sort_idx = ops.bucket_argsort(self.lsh.hash(key), num_keys)
+            query_sort_idx = ops.bucket_argsort(self.lsh.hash(query, proj), num_keys)
+            key_sort_idx = ops.bucket_argsort(self.lsh.hash(key, proj), num_keys)
             attn, lse = ops.hyper_attn_func(query.transpose(1, 2), key.transpose(1, 2), value.transpose(1, 2),
                                             query_sort_idx.transpose(1, 2), key_sort_idx.transpose(1, 2),
                                             self.block_size, self.sample_size, scale, self.smooth_block,

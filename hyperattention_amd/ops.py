@@ -294,8 +294,9 @@ def add_self_attentions(attn1, lse1, attn2, lse2):
     if _wants_grad(attn1, attn2, lse1, lse2):
         # differentiable form, in the reference's own arithmetic (src/attn_utils.py:21-23): the weight is
         # rounded to the attention's type before it is used
+        # (the logarithm is taken in fp32, as the kernel does; the reference takes it in the attention's type)
         c = torch.sigmoid(lse1 - lse2).to(attn1.dtype)
-        return c * attn1 + (1 - c) * attn2, lse1 - (c + torch.finfo(lse1.dtype).eps).log()
+        return c * attn1 + (1 - c) * attn2, lse1 - (c.float() + torch.finfo(lse1.dtype).eps).log()
     b, h, n, d = attn1.shape
     a1 = attn1.contiguous()
     a2 = attn2.contiguous()

@@ -174,7 +174,8 @@ int ha_flash_attn_fwd(const ha_attn_operands* t, int causal, void* stream);
  * query head of a group adds into its key head.  All in dtype, last dim contiguous, written in full
  * (or, with accumulate, added to in full: a caller that differentiates several attention calls on
  * views of the same tensors, like the causal recursion, sums their gradients without extra passes).
- * Only whole heads: segs == 1 and zero segment offsets.
+ * Segments (segs, seg_stride_rows and the offsets) as in the forward; dout, dq follow q's segment
+ * layout, dk, dv that of k, v.
  * workspace: ha_attn_bwd_workspace_bytes(t, sample_size) bytes (sample_size = 0 for exact attention),
  * 256-byte aligned: two floats per query, and fp32 sums of the sampled keys, cleared by the call.
  */
@@ -235,6 +236,23 @@ int ha_lse_merge_segments(const void* attn1, const float* lse1, const void* attn
                           int64_t out_seg_stride, int64_t out_row_stride,
                           int64_t lse1_seg_stride, int64_t lse2_seg_stride, int64_t lse_out_seg_stride,
                           int64_t weight_seg_stride, int dtype, void* stream);
+
+/* All merges of the causal recursion in one pass (hyper_attention.py:86-89 at every level, i.e. the chain
+ * of add_self_attentions calls a row goes through, deepest level first), for a caller that runs the
+ * levels itself and keeps their results, as a backward pass needs them.
+ * o_leaf, lse_leaf: exact causal attention of the leaves; o_un[j], lse_un[j] (j < levels, 0 = whole
+ * sequence): result of the un-masked call of level j.  Every tensor has the layout of the whole
+ * (batch_heads, n, d) / (batch_heads, n) contiguous tensors; level j only uses the rows in the second half
+ * of each segment of n / 2^j rows.  out, lse_out: the merged result (not in place).
+ * If leaf_shifted is not NULL, lse_shifted[j] (second halves) and leaf_shifted (all rows) receive
+ * lse - log(w), w the total weight the merges give that call's result in `out`: handing a call's backward
+ * this log-sum-exp together with the gradient of `out` equals handing it its own log-sum-exp and w times
+ * the gradient (weights carry no gradient, src/hyper_attn_triton.py:922-945).
+ */
+int ha_lse_merge_levels(const void* o_leaf, const float* lse_leaf, const void* const* o_un,
+                        const float* const* lse_un, float* const* lse_shifted, float* leaf_shifted,
+                        void* out, float* lse_out, int levels, int64_t batch_heads, int64_t n, int64_t d,
+                        int dtype, void* stream);
 
 /* ---------------------------------------------------------------------------------------------
  * Whole forward pass of the module for (batch, heads, n, d) tensors, one call, no host

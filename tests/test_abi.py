@@ -169,6 +169,11 @@ def test_backward_argument_errors_before_any_launch(lib):
     assert lib.ha_flash_attn_bwd(ctypes.byref(t), 0, ctypes.byref(g), None) == -1  # null tensors
     assert lib.ha_attn_bwd_workspace_bytes(ctypes.byref(t), 0) == -3                # zero sizes
     t.batch, t.heads, t.n_q, t.n_k, t.d, t.dv, t.kv_group = 2, 4, 300, 200, 64, 64, 2
+    assert lib.ha_attn_bwd_workspace_bytes(ctypes.byref(t), 0) == -3                # segs must be >= 1
+    t.segs = 3   # three segments per head: three times the per-query and per-sample scratch
+    assert lib.ha_attn_bwd_workspace_bytes(ctypes.byref(t), 0) == 3 * 19200
+    assert lib.ha_attn_bwd_workspace_bytes(ctypes.byref(t), 128) == 3 * 19200 + 2 * 3 * 2 * 2 * 128 * 64 * 4
+    t.segs = 1
     # two floats per query (256-byte aligned) + two fp32 (batch, kv_heads, sample_size, d) arrays
     assert lib.ha_attn_bwd_workspace_bytes(ctypes.byref(t), 0) == 19200
     assert lib.ha_attn_bwd_workspace_bytes(ctypes.byref(t), 128) == 19200 + 2 * (2 * 2 * 128 * 64 * 4)

@@ -163,6 +163,39 @@ def test_grouped_query_on_the_composed_path(ha):
     assert_close(lse, rl, "lse")
 
 
+def test_top_level_leaf_returns_the_same_lse_shape_with_and_without_grad(ha):
+    """n <= min_seq_len under a causal mask: one exact call whose padded 3-d log-sum-exp the reference returns as
+    it is (hyper_attention.py:52-58); the shape must not depend on whether gradients are wanted."""
+    q, k, v = (_randn((1, 2, 1000, 64), s, torch.float16).cuda() for s in (150, 151, 152))
+    m, _ = _module(ha, 64, torch.float16, 153)
+    attn, lse = m(q, k, v, causal=True, return_lse=True)
+    attn_g, lse_g = m(q.clone().requires_grad_(), k, v, causal=True, return_lse=True)
+    assert lse.shape == lse_g.shape == (1, 2, 1024)
+    assert torch.equal(attn, attn_g.detach()) and torch.equal(lse[..., :1000], lse_g.detach()[..., :1000])
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_more_than_eight_projections_in_one_call(ha, causal):
+    """4096 buckets: the one-call forward sorts in two digit passes; against the oracle and the composed path."""
+    dtype, n = torch.float16, 4096
+    q, k, v = (_randn((1, 2, n, 64), s, dtype) for s in (160, 161, 162))
+    m, proj = _module(ha, 64, dtype, 163, lsh_num_projs=12, block_size=128, sample_size=128, min_seq_len=1024)
+    attn, lse = m(q.cuda(), k.cuda(), v.cuda(), causal=causal, return_lse=True)
+    ro, rl = _oracle(q, k, v, proj, m, causal)
+    assert_close(attn, ro, "attn", dtype)
+    assert_close(lse, rl, "lse")
+    co, cl = m._forward_composed(q.cuda(), k.cuda(), v.cuda(), 64 ** -0.5, causal)
+    assert_close(attn, co.double().cpu(), "one call vs composed", dtype)
+
+
+def test_other_head_dims_leave_the_module_as_it_is(ha):
+    q, k, v = (_randn((1, 2, 2048, 32), s, torch.float16).cuda() for s in (170, 171, 172))
+    m, _ = _module(ha, 32, torch.float16, 173, min_seq_len=512)
+    before = m.lsh.proj_dir.clone()
+    m(q, k, v, causal=True)
+    assert m.lsh.proj_dir.shape == before.shape and torch.equal(m.lsh.proj_dir, before)
+
+
 def test_module_argument_errors(ha):
     m, _ = _module(ha, 64, torch.float16, 160)
     q = torch.zeros((1, 1, 256, 64), dtype=torch.float16, device="cuda")

@@ -366,6 +366,88 @@ def test_add_self_attentions(ha, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_add_self_attentions_is_the_same_with_and_without_grad(ha, dtype):
+    """The weight is rounded to the attention's type on both routes (src/attn_utils.py:21): the kernel and
+    the differentiable tensor arithmetic give the same merge up to the last rounding of the output."""
+    b, h, n, d = 1, 2, 200, 64
+    a1, a2 = (_randn((b, h, n, d), s, dtype).cuda() for s in (70, 71))
+    l1, l2 = (_randn((b, h, n, 1), s, torch.float32).cuda() * 3 for s in (72, 73))
+    plain, plain_lse = ha.add_self_attentions(a1, l1, a2, l2)
+    g1 = a1.clone().requires_grad_()
+    grad, grad_lse = ha.add_self_attentions(g1, l1, a2, l2)
+    # torch rounds c*a1 and (1-c)*a2 to the type before adding them, the kernel rounds once: one ulp apart
+    ulp = 2.0 ** (-10 if dtype == torch.float16 else -7)
+    assert float((plain.float() - grad.detach().float()).abs().max()) <= 2 * ulp * float(plain.float().abs().max())
+    assert torch.allclose(plain_lse, grad_lse.detach(), rtol=0, atol=1e-5)
+    # the weight itself: with a1 = 1, a2 = 0 the merged rows ARE the rounded weight
+    ones, zeros = torch.ones_like(a1), torch.zeros_like(a2)
+    c_kernel, _ = ha.add_self_attentions(ones, l1, zeros, l2)
+    c_ref = torch.sigmoid(l1 - l2).to(dtype)
+    assert torch.equal(c_kernel, c_ref.expand_as(c_kernel))
+
+
+@pytest.mark.parametrize("dtype,levels", [(torch.float16, 3), (torch.bfloat16, 2), (torch.float16, 0)])
+def test_merge_levels_equals_the_chain_of_segment_merges(ha, dtype, levels):
+    """ha_lse_merge_levels against the per-level in-place merges it stands for (bit for bit), and its shifted
+    log-sum-exps against lse - log(weight) from the weights those merges write."""
+    import ctypes
+    from hyperattention_amd import _lib
+    b, h, d, leaf = 2, 3, 64, 40
+    n = leaf << levels
+    dev = dict(device="cuda")
+    o_leaf = _randn((b, h, n, d), 80, dtype).cuda()
+    lse_leaf = _randn((b, h, n), 81, torch.float32).cuda() * 4
+    o_un = _randn((max(levels, 1), b, h, n, d), 82, dtype).cuda()
+    lse_un = _randn((max(levels, 1), b, h, n), 83, torch.float32).cuda() * 4
+    if levels:
+        lse_un[0, :, :, -5:] += 200.0   # weight of what was there rounds to 0
+        lse_un[levels - 1, :, :, n - leaf:n - leaf + 5] -= 200.0   # weight of the level's call is 0
+    lib, code = _lib.lib(), 0 if dtype == torch.float16 else 1
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    # the chain, deepest level first
+    out, lse = o_leaf.clone(), lse_leaf.clone()
+    cs = {}
+    for j in reversed(range(levels)):
+        H, half = (b * h) << j, n >> (j + 1)
+        out2, lse2 = out.view(H, 2, half, d)[:, 1], lse.view(H, 2, half)[:, 1]
+        o2 = o_un[j].view(H, 2, half, d)[:, 1].contiguous()
+        l2 = lse_un[j].view(H, 2, half)[:, 1].contiguous()
+        c = torch.empty((H, half), dtype=torch.float32, **dev)
+        _lib.check(lib.ha_lse_merge_segments(
+            out2.data_ptr(), lse2.data_ptr(), o2.data_ptr(), l2.data_ptr(), out2.data_ptr(), lse2.data_ptr(),
+            c.data_ptr(), H, half, d, 2 * half * d, d, half * d, d, 2 * half * d, d, 2 * half, half, 2 * half, half,
+            code, stream))
+        cs[j] = c
+    got, got_lse = torch.empty_like(o_leaf), torch.empty_like(lse_leaf)
+    shifted = torch.full((max(levels, 1), b, h, n), float("nan"), dtype=torch.float32, **dev)
+    leaf_shifted = torch.empty_like(lse_leaf)
+    ptrs = lambda x: (ctypes.c_void_p * max(levels, 1))(*[x[j].data_ptr() for j in range(levels)])
+    _lib.check(lib.ha_lse_merge_levels(o_leaf.data_ptr(), lse_leaf.data_ptr(), ptrs(o_un), ptrs(lse_un), ptrs(shifted),
+                                       leaf_shifted.data_ptr(), got.data_ptr(), got_lse.data_ptr(), levels, b * h, n, d,
+                                       code, stream))
+    torch.cuda.synchronize()
+    assert torch.equal(got, out) and torch.equal(got_lse, lse)
+    log_w = torch.zeros((b, h, n), dtype=torch.float64, **dev)
+    for j in range(levels):
+        H, half = (b * h) << j, n >> (j + 1)
+        c = cs[j].double()
+        log_w2 = log_w.view(H, 2, half)[:, 1]
+        want = lse_un[j].view(H, 2, half)[:, 1].double() - torch.log1p(-c) - log_w2
+        have = shifted[j].view(H, 2, half)
+        assert torch.isnan(have[:, 0]).all(), "first halves are not written"
+        have = have[:, 1].double()
+        both_inf = torch.isinf(want) & torch.isinf(have) & (want > 0) & (have > 0)
+        assert (both_inf | ((want - have).abs() <= 1e-4 * (1 + want.abs()))).all(), f"shifted lse of level {j}"
+        log_w2 += torch.log(c)
+    want = lse_leaf.double() - log_w
+    have = leaf_shifted.double()
+    both_inf = torch.isinf(want) & torch.isinf(have) & (want > 0) & (have > 0)
+    assert (both_inf | ((want - have).abs() <= 1e-4 * (1 + want.abs()))).all(), "shifted lse of the leaves"
+    if levels:
+        assert torch.isinf(leaf_shifted).any() and torch.isinf(shifted[levels - 1][~torch.isnan(shifted[levels - 1])]).any()
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_merge_segments_in_place(ha, dtype):
     """ha_lse_merge_segments on the second halves of every head, in place, with the weight written out:
     the merge of one level of the causal recursion (hyper_attention.py:86-89)."""
