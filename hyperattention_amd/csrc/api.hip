@@ -29,10 +29,9 @@ int ha_check_operands(const ha_attn_operands& t, const char* who) {
   HA_REQUIRE(t.batch > 0 && t.heads > 0 && t.n_q > 0 && t.n_k > 0, HA_ERR_SHAPE, "%s: sizes must be positive", who);
   // the kernels address a row as a per-head base plus a 32-bit byte offset computed with a 24-bit multiply
   HA_REQUIRE(t.n_q < (1ll << 24) && t.n_k < (1ll << 24), HA_ERR_SHAPE, "%s: sequence too long (2^24 rows at most)", who);
-  HA_REQUIRE(t.d <= 128, HA_ERR_HEADDIM, "%s: FlashAttention only support head dimensions up to 128", who);
-  HA_REQUIRE(t.d == 64 || t.d == 128, HA_ERR_UNSUPPORTED, "%s: head dim %lld not built (64 and 128 are)", who,
-             (long long)t.d);
-  HA_REQUIRE(t.dv == t.d, HA_ERR_UNSUPPORTED, "%s: value head dim must equal the key head dim in this build", who);
+  HA_REQUIRE(t.d <= 128 && t.dv <= 128, HA_ERR_HEADDIM, "%s: FlashAttention only support head dimensions up to 128", who);
+  HA_REQUIRE(t.d >= 8 && t.dv >= 8 && t.d % 8 == 0 && t.dv % 8 == 0, HA_ERR_UNSUPPORTED,
+             "%s: head dims must be multiples of 8 (got %lld and %lld)", who, (long long)t.d, (long long)t.dv);
   HA_REQUIRE(t.segs >= 1 && t.kv_group >= 1 && t.heads % t.kv_group == 0, HA_ERR_SHAPE,
              "%s: segs >= 1 and kv_group dividing heads required", who);
   HA_REQUIRE(t.scale > 0.f && isfinite(t.scale), HA_ERR_SHAPE, "%s: softmax scale must be positive and finite", who);
@@ -47,7 +46,7 @@ int ha_check_operands(const ha_attn_operands& t, const char* who) {
   for (int i = 0; i < 4; ++i) {
     HA_REQUIRE(row_strides[i] > 0 && row_strides[i] * 2 < (1ll << 24), HA_ERR_UNSUPPORTED,
                "%s: row strides must be positive and below 16 MiB", who);
-    HA_REQUIRE((row_counts[i] - 1) * row_strides[i] * 2 + t.d * 2 <= (1ll << 32), HA_ERR_UNSUPPORTED,
+    HA_REQUIRE((row_counts[i] - 1) * row_strides[i] * 2 + 128 * 2 <= (1ll << 32), HA_ERR_UNSUPPORTED,
                "%s: one head of a tensor may span 4 GiB at most", who);
   }
   return HA_OK;
@@ -109,7 +108,7 @@ int block_attn(const ha_block_attn_args& a, hipStream_t stream) {
   p.smooth = a.smooth_block != 0;
   p.accumulate = a.accumulate != 0;
   p.idx64 = a.idx_type == HA_IDX_I64;
-  return ha_attn_launch(p, (int)a.t.d, a.t.dtype, true, false, stream);
+  return ha_attn_launch(p, (int)a.t.d, (int)a.t.dv, a.t.dtype, true, false, stream);
 }
 
 int flash_attn(const ha_attn_operands& t, int causal, int accumulate, hipStream_t stream) {
@@ -118,7 +117,7 @@ int flash_attn(const ha_attn_operands& t, int causal, int accumulate, hipStream_
   ha_attn_kernel_params p;
   fill_params(t, p);
   p.accumulate = accumulate != 0;
-  return ha_attn_launch(p, (int)t.d, t.dtype, false, causal != 0, stream);
+  return ha_attn_launch(p, (int)t.d, (int)t.dv, t.dtype, false, causal != 0, stream);
 }
 
 inline int64_t align256(int64_t v) { return (v + 255) & ~(int64_t)255; }
@@ -196,7 +195,7 @@ void layout_workspace(const ha_forward_args& a, const Plan& pl, Workspace& w) {
     for (int j = 0; j < nlev; ++j)
       if (pl.level_hyper[j]) longest = std::max<int64_t>(longest, a.causal ? pl.len[j] / 2 : a.n);
     w.units = a.lsh_num_projs <= 8 && longest / g.granule * g.units_per_granule <= max_units_per_segment(g.unit) &&
-              a.n % g.granule == 0;
+              a.n % g.granule == 0 && (a.d == 32 || a.d == 64 || a.d == 128);   // the widths the paired hash is built for
     const int64_t id_bytes = w.units ? 1 : 4;
     w.buckets_q = off; off += align256(a.batch * a.heads * a.n * id_bytes);
     w.buckets_k = off; off += align256(a.batch * a.kv_heads * a.n * id_bytes);
@@ -232,10 +231,9 @@ int check_forward(const ha_forward_args& a) {
   HA_REQUIRE(a.batch > 0 && a.heads > 0 && a.kv_heads > 0 && a.n > 0, HA_ERR_SHAPE, "ha_forward: sizes must be positive");
   HA_REQUIRE(a.heads % a.kv_heads == 0, HA_ERR_SHAPE, "ha_forward: kv_heads must divide heads");
   HA_REQUIRE(a.n < (1ll << 30), HA_ERR_SHAPE, "ha_forward: sequence too long");
-  HA_REQUIRE(a.d <= 128, HA_ERR_HEADDIM, "ha_forward: FlashAttention only support head dimensions up to 128");
-  HA_REQUIRE(a.d == 64 || a.d == 128, HA_ERR_UNSUPPORTED, "ha_forward: head dim %lld not built (64 and 128 are)",
-             (long long)a.d);
-  HA_REQUIRE(a.dv == a.d, HA_ERR_UNSUPPORTED, "ha_forward: value head dim must equal the key head dim in this build");
+  HA_REQUIRE(a.d <= 128 && a.dv <= 128, HA_ERR_HEADDIM, "ha_forward: FlashAttention only support head dimensions up to 128");
+  HA_REQUIRE(a.d >= 8 && a.dv >= 8 && a.d % 8 == 0 && a.dv % 8 == 0, HA_ERR_UNSUPPORTED,
+             "ha_forward: head dims must be multiples of 8 (got %lld and %lld)", (long long)a.d, (long long)a.dv);
   HA_REQUIRE(a.scale > 0.f && isfinite(a.scale), HA_ERR_SHAPE, "ha_forward: softmax scale must be positive and finite");
   HA_REQUIRE(a.block_size > 0 && a.sample_size >= 0 && a.sample_size % 128 == 0 && a.min_seq_len >= 0, HA_ERR_SHAPE,
              "ha_forward: block_size > 0 and sample_size a non-negative multiple of 128 required");
@@ -407,8 +405,8 @@ extern "C" int ha_forward_sort(const ha_forward_args* args, int64_t* q_idx_offse
   HA_REQUIRE(a.batch > 0 && a.heads > 0 && a.kv_heads > 0 && a.n > 0 && a.min_seq_len >= 0 && a.heads % a.kv_heads == 0,
              HA_ERR_SHAPE, "ha_forward_sort: sizes must be positive and kv_heads must divide heads");
   HA_REQUIRE(a.n < (1ll << 30), HA_ERR_SHAPE, "ha_forward_sort: sequence too long");
-  HA_REQUIRE(a.d == 64 || a.d == 128, HA_ERR_UNSUPPORTED, "ha_forward_sort: head dim %lld not built (64 and 128 are)",
-             (long long)a.d);
+  HA_REQUIRE(a.d >= 8 && a.d <= 128 && a.d % 8 == 0, HA_ERR_UNSUPPORTED,
+             "ha_forward_sort: head dim must be a multiple of 8 up to 128 (got %lld)", (long long)a.d);
   Plan pl;
   int st = make_plan(a, pl);
   if (st != HA_OK) return st;

@@ -796,6 +796,8 @@ Workspace carve(const ha_attn_operands& t, int64_t sample_size, void* base) {
 
 int check_grads(const ha_attn_operands& t, int64_t sample_size, const ha_attn_grads& g, const char* who) {
   HA_REQUIRE(g.dout && g.dq && g.dk && g.dv, HA_ERR_NULL, "%s: null gradient pointer", who);
+  HA_REQUIRE((t.d == 64 || t.d == 128) && t.dv == t.d, HA_ERR_UNSUPPORTED,
+             "%s: the backward is built for head dims 64 and 128 with a value dim equal to them", who);
   const int64_t strides[] = {g.do_stride_b, g.do_stride_h, g.do_stride_n, g.dq_stride_b, g.dq_stride_h, g.dq_stride_n,
                              g.dk_stride_b, g.dk_stride_h, g.dk_stride_n, g.dv_stride_b, g.dv_stride_h, g.dv_stride_n};
   for (int64_t s : strides) HA_REQUIRE(s % 8 == 0, HA_ERR_SHAPE, "%s: gradient rows must be 16-byte aligned", who);

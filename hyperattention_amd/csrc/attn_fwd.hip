@@ -219,7 +219,20 @@ __device__ __forceinline__ void half_step(const f32x16 (&s_use)[2], f32x16 (&s_f
 // PLAIN (gathered kernel only): the common configuration, for which the per-iteration bookkeeping of the
 // general one is compiled out: no smoothing, default samples (rows 0 .. sample_size-1), and both
 // 128-query tiles of the workgroup inside one key block, so no chunk is ever masked for half of it.
-template <typename T, int D, bool GATHER, bool CAUSAL, bool PLAIN = false>
+// Head dims below the built width D (NARROW kernels): a row holds fewer 16-byte pieces than its LDS slot.
+// A lane whose piece lies past the end of the row fetches these zeros instead, so the tiles hold the rows
+// zero-padded to D: zero columns change neither q.k nor the other columns of the output.
+__device__ __attribute__((aligned(16))) const unsigned char ha_zero_piece[16] = {0};
+
+template <bool NARROW>
+__device__ __forceinline__ const unsigned char* piece_address(const unsigned char* base, int row, uint32_t stride_bytes,
+                                                              uint32_t piece, int pieces_in_row) {
+  const unsigned char* a = row_address(base, row, stride_bytes, piece << 4);
+  if (NARROW && (int)piece >= pieces_in_row) a = ha_zero_piece;
+  return a;
+}
+
+template <typename T, int D, bool GATHER, bool CAUSAL, bool PLAIN = false, bool NARROW = false>
 __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_kernel(const ha_attn_kernel_params p) {
   typedef typename ElemTraits<T>::vec8 vec8;
   typedef typename ElemTraits<T>::vec4 vec4;
@@ -411,11 +424,11 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
 // are loop constants; only a tile that reaches past the last key (or lies before the first chunk:
 // row0 < 0, every lane reads row 0) computes and clamps row numbers per lane.  All branches are
 // wave-uniform.
-#define HA_LOAD_TILE(base, stride, rs, chunk, kk0, tile, SWZ)                                            \
+#define HA_LOAD_TILE(base, stride, rs, chunk, kk0, tile, SWZ, LIM)                                         \
   if (GATHER) {                                                                                          \
     _Pragma("unroll") for (int j = 0; j < LPW; ++j) {                                                    \
       const int r = (wave_s * LPW + j) * ROWS_PER_LOAD + my_lr;                                          \
-      global_to_lds_16(row_address(base, rs.rows[j], stride, (my_pp ^ SWZ(r)) << 4),                     \
+      global_to_lds_16(piece_address<NARROW>(base, rs.rows[j], stride, my_pp ^ SWZ(r), LIM),             \
                        (tile) + (wave_s * LPW + j) * 1024);                                              \
     }                                                                                                    \
   } else {                                                                                               \
@@ -425,7 +438,7 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
       _Pragma("unroll") for (int j = 0; j < LPW; ++j) {                                                  \
         const int r = (wave_s * LPW + j) * ROWS_PER_LOAD + my_lr;                                        \
         const uint32_t first_row = __builtin_amdgcn_readfirstlane((uint32_t)(row0 + j * ROWS_PER_LOAD) * (stride)); \
-        global_to_lds_16(row_address(base + first_row, my_lr, stride, (my_pp ^ SWZ(r)) << 4),            \
+        global_to_lds_16(piece_address<NARROW>(base + first_row, my_lr, stride, my_pp ^ SWZ(r), LIM),    \
                          (tile) + (wave_s * LPW + j) * 1024);                                            \
       }                                                                                                  \
     } else {                                                                                             \
@@ -433,7 +446,7 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
         const int r = (wave_s * LPW + j) * ROWS_PER_LOAD + my_lr;                                        \
         int row = row0 + j * ROWS_PER_LOAD + my_lr;                                                      \
         if (row0 < 0 || row >= p.n_k) row = 0;                                                           \
-        global_to_lds_16(row_address(base, row, stride, (my_pp ^ SWZ(r)) << 4),                          \
+        global_to_lds_16(piece_address<NARROW>(base, row, stride, my_pp ^ SWZ(r), LIM),                  \
                          (tile) + (wave_s * LPW + j) * 1024);                                            \
       }                                                                                                  \
     }                                                                                                    \
@@ -457,16 +470,17 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
 #pragma unroll
     for (int nb = 0; nb < 2; ++nb)
       if (wave_q_first + nb * 32 + col >= p.n_q) qrow[nb] = -1;
-    HA_LOAD_TILE(kb, k_rb, rows_k, k_chunk_shift, k_kk0, lds_k0, k_swizzle)
+    HA_LOAD_TILE(kb, k_rb, rows_k, k_chunk_shift, k_kk0, lds_k0, k_swizzle, p.qk_pieces)
 #pragma unroll
     for (int j = 0; j < PR; ++j) {
       // positions past the end read row 0 (finite data; their results are never written)
       const int r = j * ROWS_PER_LOAD + my_lr;
-      global_to_lds_16(row_address(qb, q_rows[j] < 0 ? 0 : q_rows[j], q_rb, (my_pp ^ (r & 7)) << 4), my_q + j * 1024);
+      global_to_lds_16(piece_address<NARROW>(qb, q_rows[j] < 0 ? 0 : q_rows[j], q_rb, my_pp ^ (r & 7), p.qk_pieces),
+                       my_q + j * 1024);
       if (my_pp == 0) lds_qrow[wave * 64 + r] = q_rows[j];
     }
-    HA_LOAD_TILE(vb, v_rb, rows_v, 0, v_kk0, lds_v0, v_swizzle)
-    HA_LOAD_TILE(kb, k_rb, rows_k1, 1 + k_chunk_shift, k_kk0, lds_k1, k_swizzle)
+    HA_LOAD_TILE(vb, v_rb, rows_v, 0, v_kk0, lds_v0, v_swizzle, p.v_pieces)
+    HA_LOAD_TILE(kb, k_rb, rows_k1, 1 + k_chunk_shift, k_kk0, lds_k1, k_swizzle, p.qk_pieces)
   }
   HA_FETCH_ROWS_K(2, rows_k)
   HA_FETCH_ROWS_V(1, rows_v)
@@ -578,12 +592,12 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
   _Pragma("unroll") for (int db = 0; db < DB; ++db) _Pragma("unroll") for (int nb = 0; nb < 2; ++nb)        \
       acc[db][nb] = Mfma<T>::run(vf[db], pb[nb], acc[db][nb]);
   /* consecutive rows known to lie inside the keys: no row numbers, no bounds */                             \
-#define HA_LOAD_TILE_INSIDE(base, stride, chunk, kk0, tile, SWZ)                                            \
+#define HA_LOAD_TILE_INSIDE(base, stride, chunk, kk0, tile, SWZ, LIM)                                         \
   _Pragma("unroll") for (int j = 0; j < LPW; ++j) {                                                         \
     const int r = (wave_s * LPW + j) * ROWS_PER_LOAD + my_lr;                                               \
     const uint32_t first_row =                                                                              \
         __builtin_amdgcn_readfirstlane((uint32_t)((chunk) * KC + (kk0) + j * ROWS_PER_LOAD) * (stride));    \
-    global_to_lds_16(row_address(base + first_row, my_lr, stride, (my_pp ^ SWZ(r)) << 4),                   \
+    global_to_lds_16(piece_address<NARROW>(base + first_row, my_lr, stride, my_pp ^ SWZ(r), LIM),           \
                      (tile) + (wave_s * LPW + j) * 1024);                                                   \
   }
   // INTERIOR (exact attention only): every row of the tiles the iteration loads exists and no score of
@@ -591,14 +605,14 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
 #define HA_ITERATION(ci, K_RD, K_WR, V_CUR, V_WR, INTERIOR)                                                 \
   {                                                                                                         \
     if (INTERIOR) {                                                                                         \
-      HA_LOAD_TILE_INSIDE(kb, k_rb, (ci) + 2 + k_chunk_shift, k_kk0, K_WR, k_swizzle)                       \
-      HA_LOAD_TILE_INSIDE(vb, v_rb, (ci) + 1, v_kk0, V_WR, v_swizzle)                                       \
+      HA_LOAD_TILE_INSIDE(kb, k_rb, (ci) + 2 + k_chunk_shift, k_kk0, K_WR, k_swizzle, p.qk_pieces)                       \
+      HA_LOAD_TILE_INSIDE(vb, v_rb, (ci) + 1, v_kk0, V_WR, v_swizzle, p.v_pieces)                                       \
     } else {                                                                                                \
       if (__builtin_expect((ci) + 2 <= n_chunks, true)) {                                                   \
-        HA_LOAD_TILE(kb, k_rb, rows_k, (ci) + 2 + k_chunk_shift, k_kk0, K_WR, k_swizzle) /* K tile ci+2 */  \
+        HA_LOAD_TILE(kb, k_rb, rows_k, (ci) + 2 + k_chunk_shift, k_kk0, K_WR, k_swizzle, p.qk_pieces) /* K tile ci+2 */  \
       }                                                                                                     \
       if (__builtin_expect((ci) + 1 < n_chunks, true)) {                                                    \
-        HA_LOAD_TILE(vb, v_rb, rows_v, (ci) + 1, v_kk0, V_WR, v_swizzle) /* V tile ci+1 */                  \
+        HA_LOAD_TILE(vb, v_rb, rows_v, (ci) + 1, v_kk0, V_WR, v_swizzle, p.v_pieces) /* V tile ci+1 */                  \
       }                                                                                                     \
       HA_FETCH_ROWS_K((ci) + 3, rows_k)                                                                     \
       HA_FETCH_ROWS_V((ci) + 2, rows_v)                                                                     \
@@ -658,7 +672,8 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
 #pragma unroll
     for (int j = 0; j < OUT_PIECES; ++j) {
       // positions past the end read row 0 (never written back): an unconditional load needs no zero fill
-      prev[j] = *reinterpret_cast<const vec8*>(row_address(ob, out_row[j] < 0 ? 0 : out_row[j], o_rb, my_pp * 16));
+      prev[j] = *reinterpret_cast<const vec8*>(
+          piece_address<NARROW>(ob, out_row[j] < 0 ? 0 : out_row[j], o_rb, my_pp, p.v_pieces));
     }
   }
   T* const lds_o = reinterpret_cast<T*>(my_q);
@@ -688,7 +703,7 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
 #pragma unroll
   for (int j = 0; j < OUT_PIECES; ++j) {
     const int lrow = j * ROWS_PER_LOAD + my_lr;
-    if (out_row[j] >= 0) {
+    if (out_row[j] >= 0 && (!NARROW || my_pp < p.v_pieces)) {
       vec8 o = *reinterpret_cast<const vec8*>(&lds_o[lrow * DV + ((my_pp ^ (lrow & 7)) * 8)]);
       if (p.accumulate) {
         const float w = lds_w[wave * 64 + lrow];
@@ -706,18 +721,24 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
 
 namespace {
 
-template <typename T, int D, bool GATHER, bool CAUSAL, bool PLAIN = false>
+template <typename T, int D, bool GATHER, bool CAUSAL, bool PLAIN = false, bool NARROW = false>
 int launch_one(const ha_attn_kernel_params& p, int grid, hipStream_t stream, const char* what) {
-  hipLaunchKernelGGL((ha_attn_fwd_kernel<T, D, GATHER, CAUSAL, PLAIN>), dim3(grid), dim3(WG_THREADS), 0, stream, p);
+  hipLaunchKernelGGL((ha_attn_fwd_kernel<T, D, GATHER, CAUSAL, PLAIN, NARROW>), dim3(grid), dim3(WG_THREADS), 0, stream, p);
   return ha_launch_status(what);
 }
 
 template <typename T, int D>
 int launch_variant(const ha_attn_kernel_params& p, int grid, bool gather, bool causal, hipStream_t stream) {
+  const bool narrow = p.qk_pieces != D / 8 || p.v_pieces != D / 8;
   if (gather) {
     const bool plain = !p.smooth && !p.sampled_idx && p.block_tiles % 2 == 0 && p.n_q % WG_QUERIES == 0;
+    if (narrow) return launch_one<T, D, true, false, false, true>(p, grid, stream, "ha_block_attn_fwd");
     if (plain) return launch_one<T, D, true, false, true>(p, grid, stream, "ha_block_attn_fwd");
     return launch_one<T, D, true, false>(p, grid, stream, "ha_block_attn_fwd");
+  }
+  if (narrow) {
+    if (causal) return launch_one<T, D, false, true, false, true>(p, grid, stream, "ha_flash_attn_fwd");
+    return launch_one<T, D, false, false, false, true>(p, grid, stream, "ha_flash_attn_fwd");
   }
   if (causal) return launch_one<T, D, false, true>(p, grid, stream, "ha_flash_attn_fwd");
   return launch_one<T, D, false, false>(p, grid, stream, "ha_flash_attn_fwd");
@@ -735,8 +756,14 @@ static ha_divisor make_divisor(int64_t y) {
   return d;
 }
 
-int ha_attn_launch(const ha_attn_kernel_params& params, int d, int dtype, bool gather, bool causal, hipStream_t stream) {
+int ha_attn_launch(const ha_attn_kernel_params& params, int d, int dv, int dtype, bool gather, bool causal,
+                   hipStream_t stream) {
   ha_attn_kernel_params p = params;
+  // the kernels are built for rows of 64 and 128 elements; other head dims (multiples of 8) run in the
+  // next width with the missing pieces of every row read as zeros
+  const int width = d <= 64 && dv <= 64 ? 64 : 128;
+  p.qk_pieces = d / 8;
+  p.v_pieces = dv / 8;
   const int64_t qtiles = (p.n_q + WG_QUERIES - 1) / WG_QUERIES;
   p.div_qtiles = make_divisor(qtiles);
   p.div_segs = make_divisor(p.segs);
@@ -747,9 +774,9 @@ int ha_attn_launch(const ha_attn_kernel_params& params, int d, int dtype, bool g
   const int64_t grid = qtiles * p.batch * p.heads * p.segs;
   if (grid <= 0 || grid >= (1ll << 31)) return ha_fail(HA_ERR_SHAPE, "attention: grid of %lld workgroups", (long long)grid);
   if (dtype == HA_F16) {
-    if (d == 64) return launch_variant<f16_t, 64>(p, (int)grid, gather, causal, stream);
+    if (width == 64) return launch_variant<f16_t, 64>(p, (int)grid, gather, causal, stream);
     return launch_variant<f16_t, 128>(p, (int)grid, gather, causal, stream);
   }
-  if (d == 64) return launch_variant<bf16_t, 64>(p, (int)grid, gather, causal, stream);
+  if (width == 64) return launch_variant<bf16_t, 64>(p, (int)grid, gather, causal, stream);
   return launch_variant<bf16_t, 128>(p, (int)grid, gather, causal, stream);
 }

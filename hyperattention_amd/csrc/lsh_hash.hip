@@ -319,6 +319,10 @@ int ha_hash_pair_u8(const void* q, const void* k, const void* proj, uint8_t* ids
   ten.heads[0] = (int)heads; ten.heads[1] = (int)kv_heads;
   ten.seqs0 = (int)(batch * heads);
   const int64_t seqs = batch * (heads + kv_heads);
+  if (d == 32) {
+    if (dtype == HA_F16) return launch_hash_mfma<f16_t, 32, true>(ten, seqs, proj, n, r, 0, 0, stream);
+    return launch_hash_mfma<bf16_t, 32, true>(ten, seqs, proj, n, r, 0, 0, stream);
+  }
   if (d == 64) {
     if (dtype == HA_F16) return launch_hash_mfma<f16_t, 64, true>(ten, seqs, proj, n, r, 0, 0, stream);
     return launch_hash_mfma<bf16_t, 64, true>(ten, seqs, proj, n, r, 0, 0, stream);
@@ -327,5 +331,5 @@ int ha_hash_pair_u8(const void* q, const void* k, const void* proj, uint8_t* ids
     if (dtype == HA_F16) return launch_hash_mfma<f16_t, 128, true>(ten, seqs, proj, n, r, 0, 0, stream);
     return launch_hash_mfma<bf16_t, 128, true>(ten, seqs, proj, n, r, 0, 0, stream);
   }
-  return ha_fail(HA_ERR_UNSUPPORTED, "ha_forward: head dim %lld not built (64 and 128 are)", (long long)d);
+  return ha_fail(HA_ERR_UNSUPPORTED, "ha_forward: paired hash not built for head dim %lld", (long long)d);
 }

@@ -219,9 +219,12 @@ class HyperAttention(torch.nn.Module):
 
         dim_v = value.shape[-1]
         proj = self.lsh.proj_dir
-        if dim not in ops.KERNEL_HEAD_DIMS or dim_v != dim:
-            # head dims the kernels are not built for (and a value dim different from the q/k dim) run
-            # zero-padded: zero columns change neither the projections, nor q.k, nor the wanted outputs
+        built = dim in ops.KERNEL_HEAD_DIMS and dim_v == dim
+        if not built and (dim % 8 or dim_v % 8 or ops._wants_grad(query, key, value)):
+            # The forward kernels take head dims that are multiples of 8 as they are, the value dim apart
+            # from the q/k dim.  Other head dims, and the backward for anything but 64 and 128 with equal
+            # dims, run zero-padded: zero columns change neither the projections, nor q.k, nor the wanted
+            # outputs
             assert dim <= 128 and dim_v <= 128, "FlashAttention only support head dimensions up to 128"
             wide = ops.padded_head_dim(max(dim, dim_v))
             pad = lambda x: torch.nn.functional.pad(x, (0, wide - x.shape[-1]))

@@ -211,16 +211,18 @@ def hyper_attn_func(q, k, v, q_sort_idx, k_sort_idx, block_size, sample_size=0, 
     which equals add_self_attentions(previous, this call) in fp32."""
     q, k, v = [x if x.stride(-1) == 1 else x.contiguous() for x in [q, k, v]]
     assert sample_size % 128 == 0
-    if _wants_grad(q, k, v) and v.shape[-1] == q.shape[-1] and q.shape[-1] in KERNEL_HEAD_DIMS:
+    built = v.shape[-1] == q.shape[-1] and q.shape[-1] in KERNEL_HEAD_DIMS
+    if _wants_grad(q, k, v) and built:
         assert resume is None, "resume has no backward"
         return HyperAttnFunc.apply(q, k, v, q_sort_idx, k_sort_idx, block_size, sample_size, softmax_scale,
                                    smooth_block, sampled_idx)
-    if v.shape[-1] != q.shape[-1] or q.shape[-1] not in KERNEL_HEAD_DIMS:
+    if not built and (_wants_grad(q, k, v) or q.shape[-1] % 8 or v.shape[-1] % 8):
         # A value head dim different from the q/k head dim (src/hyper_attn_triton.py:679,692-693;
-        # unit_tests/test_hyper_attention.py:120-133), or a head dim the kernels are not built for.
-        # Zero columns change neither q.k nor the wanted columns of the output, so both sides are
-        # zero-padded to a built width and the output is cut back: exact, at the price of the copies.
-        assert resume is None, "resume needs a head dim the kernels are built for"
+        # unit_tests/test_hyper_attention.py:120-133) or a head dim other than 64 and 128: the forward
+        # kernels take any multiples of 8 as they are (the missing pieces of a row are read as zeros).
+        # The backward, and head dims that are not multiples of 8, go through zero-padded copies: zero
+        # columns change neither q.k nor the wanted columns of the output, so this is exact.
+        assert resume is None, "resume needs head dims that are multiples of 8"
         d_qk, d_v = q.shape[-1], v.shape[-1]
         assert d_qk <= 128 and d_v <= 128, "FlashAttention only support head dimensions up to 128"
         wide = padded_head_dim(max(d_qk, d_v))
@@ -270,8 +272,9 @@ def flash_attn_func(q, k, v, bias=None, causal=False, softmax_scale=None):
     assert d <= 128, "FlashAttention only support head dimensions up to 128"
     if _wants_grad(q, k, v) and d in KERNEL_HEAD_DIMS:
         return FlashAttnFunc.apply(q, k, v, bias, causal, softmax_scale)
-    if d not in KERNEL_HEAD_DIMS:
-        # other head dims run zero-padded to a built width (exact; costs the padded copies)
+    if d not in KERNEL_HEAD_DIMS and (_wants_grad(q, k, v) or d % 8):
+        # the forward kernels take any multiple of 8; the backward and other head dims run zero-padded to a
+        # built width (exact; costs the padded copies)
         pad = lambda x: torch.nn.functional.pad(x, (0, padded_head_dim(d) - d))
         o, lse = flash_attn_func(pad(q), pad(k), pad(v), None, causal, softmax_scale or 1.0 / math.sqrt(d))
         return o[..., :d], lse

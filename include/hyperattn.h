@@ -138,7 +138,9 @@ typedef struct {
  * by the host, so the library cannot check it: an entry outside the range reads rows of another
  * segment or head (inside a causal recursion: future tokens) or past the tensor, and the backward adds
  * to such rows.  The Python operator layer checks the list on the host before every call.
- * n_q % 128 == 0, n_k % 128 == 0 (:695), sample_size % 128 == 0 (:911), d and dv in {64, 128}.
+ * n_q % 128 == 0, n_k % 128 == 0 (:695), sample_size % 128 == 0 (:911); d and dv (value dim, may differ from d: :679,692-693) multiples of 8
+ * up to 128: kernels are built for rows of 64 and 128 elements and read narrower rows as they are, the
+ * missing columns as zeros.
  * accumulate != 0: out/lse already hold a partial attention over a disjoint key set for every row;
  * the result is merged into them in place (add_self_attentions, src/attn_utils.py:6-24, fused).
  */
@@ -161,7 +163,7 @@ int ha_block_attn_fwd(const ha_block_attn_args* args, void* stream);
 /* Exact (flash) attention, forward.
  * replaces: flash_attn_func -> FlashAttnFunc.forward -> _flash_attn_forward -> _fwd_kernel with
  *           bias=None (src/flash_attn_triton.py:995-1012, :795-872, :57-267)
- * Any n_q, n_k >= 1; causal mask row >= col (:177); d == dv in {64, 128}.
+ * Any n_q, n_k >= 1; causal mask row >= col (:177); d, dv multiples of 8 up to 128.
  */
 int ha_flash_attn_fwd(const ha_attn_operands* t, int causal, void* stream);
 
@@ -175,7 +177,7 @@ int ha_flash_attn_fwd(const ha_attn_operands* t, int causal, void* stream);
  * (or, with accumulate, added to in full: a caller that differentiates several attention calls on
  * views of the same tensors, like the causal recursion, sums their gradients without extra passes).
  * Segments (segs, seg_stride_rows and the offsets) as in the forward; dout, dq follow q's segment
- * layout, dk, dv that of k, v.
+ * layout, dk, dv that of k, v.  Built for d == dv in {64, 128} (HA_ERR_UNSUPPORTED otherwise).
  * workspace: ha_attn_bwd_workspace_bytes(t, sample_size) bytes (sample_size = 0 for exact attention),
  * 256-byte aligned: two floats per query, and fp32 sums of the sampled keys, cleared by the call.
  */

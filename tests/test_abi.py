@@ -111,7 +111,9 @@ def test_attention_argument_errors(lib):
     assert lib.ha_flash_attn_fwd(ctypes.byref(_operands(dtype=3)), 0, None) == -2
     assert lib.ha_flash_attn_fwd(ctypes.byref(_operands(d=256, dv=256)), 0, None) == -4
     assert b"head dimensions up to 128" in lib.ha_last_error()
-    assert lib.ha_flash_attn_fwd(ctypes.byref(_operands(d=32, dv=32)), 0, None) == -5
+    assert lib.ha_flash_attn_fwd(ctypes.byref(_operands(d=36, dv=36)), 0, None) == -5   # not a multiple of 8
+    assert lib.ha_flash_attn_fwd(ctypes.byref(_operands(d=64, dv=4)), 0, None) == -5
+    assert b"multiples of 8" in lib.ha_last_error()
     assert lib.ha_flash_attn_fwd(ctypes.byref(_operands(scale=0.0)), 0, None) == -3
     assert lib.ha_flash_attn_fwd(ctypes.byref(_operands(q_stride_n=60)), 0, None) == -3
     # addressing limits: 2^24 rows, row strides below 16 MiB, one head within 4 GiB

@@ -139,12 +139,15 @@ def test_permuted_views_are_read_in_place(ha, causal):
 
 
 @pytest.mark.parametrize("causal", [False, True])
-def test_module_other_head_dim(ha, causal):
-    """input_dim 96: hashed with the module's own (96, r) projection, attention zero-padded to 128."""
-    q, k, v = (_randn((1, 2, 2048, 96), s, torch.float16) for s in (180, 181, 182))
-    m, proj = _module(ha, 96, torch.float16, 183, min_seq_len=512)
+@pytest.mark.parametrize("d,dv", [(96, 96), (32, 32), (40, 72), (64, 128), (128, 64), (100, 100)])
+def test_module_other_head_dim(ha, causal, d, dv):
+    """Head dims other than 64 and 128, and a value dim apart from the q/k dim: hashed with the module's own
+    (d, r) projection; multiples of 8 are read by the kernels as they are, 100 runs zero-padded."""
+    q, k = (_randn((1, 2, 2048, d), s, torch.float16) for s in (180, 181))
+    v = _randn((1, 2, 2048, dv), 182, torch.float16)
+    m, proj = _module(ha, d, torch.float16, 183, min_seq_len=512)
     attn, lse = m(q.cuda(), k.cuda(), v.cuda(), causal=causal, return_lse=True)
-    assert attn.shape == (1, 2, 2048, 96) and m.lsh.proj_dir.shape[-2] == 96
+    assert attn.shape == (1, 2, 2048, dv) and m.lsh.proj_dir.shape[-2] == d
     ro, rl = _oracle(q, k, v, proj, m, causal)
     assert_close(attn, ro, "attn", torch.float16)
     assert_close(lse, rl, "lse")
