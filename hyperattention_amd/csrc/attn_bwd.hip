@@ -422,7 +422,7 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 || PASS == HA_BWD_DQ_BLOCK ? 2
     for (int ks = 0; ks < KSTEPS; ++ks)
 #pragma unroll
       for (int e = 0; e < 8; ++e) part = __builtin_fmaf((float)of[ks][e], (float)x2f[ks][e], part);
-    st_delta = (part + __shfl_xor(part, 32)) * p.scale;
+    st_delta = ha_sum_xor32(part) * p.scale;
     if (hi == 0 && st_valid) p.stats[((int64_t)(b * p.heads + h0) * p.segs + seg) * p.n_q + st_row] = f32x2{st_lse2, st_delta};
   }
 

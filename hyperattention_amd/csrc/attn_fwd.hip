@@ -48,6 +48,11 @@ constexpr int WG_THREADS = 256;
 constexpr int WG_QUERIES = 256;  // sorted query positions per workgroup
 constexpr int KC = 64;           // keys per LDS tile
 constexpr float HALF_SUM_LIMIT = 16384.f;  // 2^14: a lane's half-step sum below this has no fp16 overflow
+// Reference exponent (log2 units) of a row that has seen no key yet.  Finite on purpose: a masked score
+// (-inf) then gives P = 2^(-inf) = 0 without any special case, where -inf - (-inf) would be a NaN that
+// sends every half-step of a masked chunk through the rescaling path; a real score gives 2^(+huge) = inf,
+// which takes that path once and sets the row's true exponent.
+constexpr float M_FLOOR = -1e30f;
 
 // Head dims whose kernel needs more than 256 registers keep the S^T accumulators in VGPRs by hand.
 template <int D>
@@ -108,14 +113,14 @@ __device__ __forceinline__ void half_step_rescale(const f32x16 (&s_use)[2], floa
     float v = s_use[nb][H * 8];
 #pragma unroll
     for (int e = 1; e < 8; ++e) v = fmaxf(v, s_use[nb][H * 8 + e]);
-    v = fmaxf(v, __shfl_xor(v, 32)) * scale_log2;
+    v = ha_max_xor32(v) * scale_log2;
     const float m_new = fmaxf(m_run[nb], v);
-    // nothing accumulated yet under m_run = -inf; otherwise 2^(old - new) <= 1
-    alpha[nb] = m_run[nb] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m_run[nb] - m_new);
+    // 2^(old - new) <= 1; nothing is accumulated yet under the floor exponent of a fresh row
+    alpha[nb] = __builtin_amdgcn_exp2f(m_run[nb] - m_new);
     m_run[nb] = m_new;
     l_run[nb] *= alpha[nb];
-    // rows that have seen no key yet (all masked) keep m_run = -inf; their P is 2^(-inf - 0) = 0
-    m_use[nb] = m_new == -INFINITY ? 0.f : m_new;
+    // rows that have seen no key yet (all masked) keep the floor; their P is 2^(-inf) = 0
+    m_use[nb] = m_new;
   }
   half_step_p<T, H>(s_use, m_use, scale_log2, pn, sum);
 }
@@ -490,7 +495,7 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
   f32x16 acc[DB][2];
 #pragma unroll
   for (int nb = 0; nb < 2; ++nb) {
-    m_run[nb] = -INFINITY;
+    m_run[nb] = M_FLOOR;
     l_run[nb] = 0.f;
 #pragma unroll
     for (int db = 0; db < DB; ++db)
@@ -499,8 +504,12 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
     if (p.accumulate && qrow[nb] >= 0) {
       // resume from a previous partial attention: it enters with weight exp(lse_prev - m) = 1; its
       // normalised output rows are added when the result is written
-      m_run[nb] = lb[qrow[nb]] * LOG2E;
-      l_run[nb] = hi == 0 ? 1.f : 0.f;
+      // (a previous result of -inf, a row that had no key at all, enters with weight 0)
+      const float m_prev = lb[qrow[nb]] * LOG2E;
+      if (m_prev > M_FLOOR) {
+        m_run[nb] = m_prev;
+        l_run[nb] = hi == 0 ? 1.f : 0.f;
+      }
     }
     m_init[nb] = m_run[nb];
   }
@@ -679,13 +688,13 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
   T* const lds_o = reinterpret_cast<T*>(my_q);
 #pragma unroll
   for (int nb = 0; nb < 2; ++nb) {
-    const float l_tot = l_run[nb] + __shfl_xor(l_run[nb], 32);
+    const float l_tot = ha_sum_xor32(l_run[nb]);
     const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
     const int lrow = nb * 32 + col;
     if (hi == 0) {
-      if (qrow[nb] >= 0) lb[qrow[nb]] = l_tot > 0.f ? (m_run[nb] + __builtin_amdgcn_logf(l_tot)) * LN2 : -INFINITY;
+      if (qrow[nb] >= 0) lb[qrow[nb]] = l_tot > 0.f && m_run[nb] > M_FLOOR ? (m_run[nb] + __builtin_amdgcn_logf(l_tot)) * LN2 : -INFINITY;
       // weight of the resumed rows: exp(lse_prev - m_final) / l_tot
-      lds_w[wave * 64 + lrow] = m_init[nb] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m_init[nb] - m_run[nb]) * inv;
+      lds_w[wave * 64 + lrow] = m_init[nb] > M_FLOOR ? __builtin_amdgcn_exp2f(m_init[nb] - m_run[nb]) * inv : 0.f;
     }
 #pragma unroll
     for (int db = 0; db < DB; ++db)

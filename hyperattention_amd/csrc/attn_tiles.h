@@ -64,6 +64,27 @@ struct Mfma<bf16_t> {
   }
 };
 
+// A lane's value and the value of the lane 32 away, in one of the two orders (symmetric uses only: max,
+// sum).  v_permlane32_swap exchanges the upper half of one register with the lower half of another; with
+// both holding v, every lane ends up with its own value in one of them and its partner's in the other.
+// No lane id and no LDS crossbar (ds_bpermute) are involved.  The s_nop covers the wait states the
+// instruction needs after a VALU write of its operands, which the compiler does not count for inline asm.
+__device__ __forceinline__ void ha_with_lane_xor32(float v, float& a, float& b) {
+  a = v;
+  b = v;
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+}
+__device__ __forceinline__ float ha_max_xor32(float v) {
+  float a, b;
+  ha_with_lane_xor32(v, a, b);
+  return fmaxf(a, b);
+}
+__device__ __forceinline__ float ha_sum_xor32(float v) {
+  float a, b;
+  ha_with_lane_xor32(v, a, b);
+  return a + b;
+}
+
 // Address of 16-byte piece `piece_bytes` of row `row`: a wave-uniform base plus a 32-bit byte offset,
 // so that a lane spends one 24-bit multiply-add on it instead of a 64-bit multiplication.  The entry
 // points check that row numbers and row strides in bytes stay below 2^24 and their products below 2^32.
