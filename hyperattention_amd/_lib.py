@@ -35,7 +35,7 @@ SYMBOLS = [
 ]
 
 HA_F16, HA_BF16 = 0, 1
-ABI_VERSION = 5
+ABI_VERSION = 6
 HA_IDX_I32, HA_IDX_I64 = 0, 1
 
 
@@ -95,6 +95,7 @@ class BlockAttnArgs(ctypes.Structure):
         ("sampled_stride_b", ctypes.c_int64), ("sampled_stride_h", ctypes.c_int64),
         ("block_size", ctypes.c_int64), ("sample_size", ctypes.c_int64),
         ("smooth_block", ctypes.c_int), ("accumulate", ctypes.c_int),
+        ("sampled_pos", ctypes.c_void_p), ("sample_bias", ctypes.c_float), ("mask_sampled_in_block", ctypes.c_int),
     ]
 
 

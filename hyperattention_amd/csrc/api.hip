@@ -91,6 +91,7 @@ void fill_params(const ha_attn_operands& t, ha_attn_kernel_params& p) {
   p.batch = (int)t.batch; p.heads = (int)t.heads; p.segs = (int)t.segs; p.kv_group = (int)t.kv_group;
   p.n_q = (int)t.n_q; p.n_k = (int)t.n_k;
   p.block_tiles = 1; p.sample_chunks = 0; p.smooth = 0; p.accumulate = 0; p.idx64 = 0;
+  p.sampled_pos = nullptr; p.sample_bias_raw = 0.f;
   p.scale_log2 = t.scale * LOG2E_F;
 }
 
@@ -108,7 +109,17 @@ int block_attn(const ha_block_attn_args& a, hipStream_t stream) {
   p.smooth = a.smooth_block != 0;
   p.accumulate = a.accumulate != 0;
   p.idx64 = a.idx_type == HA_IDX_I64;
-  return ha_attn_launch(p, (int)a.t.d, (int)a.t.dv, a.t.dtype, true, false, stream);
+  const bool reweight = a.sample_bias != 0.f || a.mask_sampled_in_block != 0;
+  if (reweight) {
+    HA_REQUIRE(isfinite(a.sample_bias), HA_ERR_SHAPE, "ha_block_attn_fwd: sample_bias must be finite");
+    HA_REQUIRE(!a.mask_sampled_in_block || a.sampled_pos, HA_ERR_NULL,
+               "ha_block_attn_fwd: mask_sampled_in_block needs sampled_pos");
+    HA_REQUIRE(a.t.d == a.t.dv && (a.t.d == 64 || a.t.d == 128), HA_ERR_UNSUPPORTED,
+               "ha_block_attn_fwd: the residual estimator is built for d == dv in {64, 128}");
+    p.sampled_pos = a.mask_sampled_in_block ? a.sampled_pos : nullptr;
+    p.sample_bias_raw = a.sample_bias / a.t.scale;
+  }
+  return ha_attn_launch(p, (int)a.t.d, (int)a.t.dv, a.t.dtype, true, false, reweight, stream);
 }
 
 int flash_attn(const ha_attn_operands& t, int causal, int accumulate, hipStream_t stream) {
@@ -117,7 +128,7 @@ int flash_attn(const ha_attn_operands& t, int causal, int accumulate, hipStream_
   ha_attn_kernel_params p;
   fill_params(t, p);
   p.accumulate = accumulate != 0;
-  return ha_attn_launch(p, (int)t.d, (int)t.dv, t.dtype, false, causal != 0, stream);
+  return ha_attn_launch(p, (int)t.d, (int)t.dv, t.dtype, false, causal != 0, false, stream);
 }
 
 inline int64_t align256(int64_t v) { return (v + 255) & ~(int64_t)255; }
@@ -458,7 +469,7 @@ extern "C" int ha_forward(const ha_forward_args* args, void* stream_) {
   auto hyper_level = [&](int j, bool accumulate) -> int {
     const int64_t seg_len = a.causal ? pl.len[j] / 2 : a.n;
     const int64_t segs = a.causal ? (1ll << j) : 1;
-    ha_block_attn_args b;
+    ha_block_attn_args b = {};
     b.t = t;
     b.t.n_q = b.t.n_k = seg_len;
     b.t.segs = segs;

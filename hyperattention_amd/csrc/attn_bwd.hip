@@ -938,6 +938,8 @@ extern "C" int ha_block_attn_bwd(const ha_block_attn_args* args, const ha_attn_g
   st = check_grads(a.t, a.sample_size, *grads, "ha_block_attn_bwd");
   if (st != HA_OK) return st;
   HA_REQUIRE(!a.accumulate, HA_ERR_UNSUPPORTED, "ha_block_attn_bwd: no backward of the fused merge (accumulate)");
+  HA_REQUIRE(a.sample_bias == 0.f && !a.mask_sampled_in_block, HA_ERR_UNSUPPORTED,
+             "ha_block_attn_bwd: no backward of the residual estimator (sample_bias, mask_sampled_in_block)");
   HA_REQUIRE(!a.smooth_block || a.block_size <= 128 * (MAX_SMOOTH_TILES - 1), HA_ERR_UNSUPPORTED,
              "ha_block_attn_bwd: smoothed blocks longer than %d rows are not built", 128 * (MAX_SMOOTH_TILES - 1));
   hipStream_t s = (hipStream_t)stream;

@@ -34,13 +34,17 @@ struct ha_attn_kernel_params {
   int sample_chunks;  // sample_size / 64
   int smooth, accumulate, idx64;
   int qk_pieces, v_pieces;  // 16-byte pieces in a row of q/k and of v/out (filled by ha_attn_launch)
+  // residual estimator (gathered kernel, REWEIGHT instances only)
+  const int32_t* sampled_pos;  // sorted-order position of every sampled key; null: nothing is masked
+  float sample_bias_raw;       // added to the raw q.k of a sampled key: bias / softmax scale
   float scale_log2;   // softmax scale * log2(e)
   // the divisors of the workgroup -> (head, segment, tile) decomposition as multiply-and-shift
   // constants (filled by ha_attn_launch): the kernel never divides
   ha_divisor div_qtiles, div_segs, div_heads, div_kv_heads, div_kv_group, div_block_tiles;
 };
 
-int ha_attn_launch(const ha_attn_kernel_params& p, int d, int dv, int dtype, bool gather, bool causal, hipStream_t stream);
+int ha_attn_launch(const ha_attn_kernel_params& p, int d, int dv, int dtype, bool gather, bool causal, bool reweight,
+                   hipStream_t stream);
 
 // argument checks shared by the forward and backward entry points (defined in api.hip); `who` names
 // the entry point in the error message

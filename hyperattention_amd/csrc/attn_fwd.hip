@@ -237,7 +237,7 @@ __device__ __forceinline__ const unsigned char* piece_address(const unsigned cha
   return a;
 }
 
-template <typename T, int D, bool GATHER, bool CAUSAL, bool PLAIN = false, bool NARROW = false>
+template <typename T, int D, bool GATHER, bool CAUSAL, bool PLAIN = false, bool NARROW = false, bool REWEIGHT = false>
 __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_kernel(const ha_attn_kernel_params p) {
   typedef typename ElemTraits<T>::vec8 vec8;
   typedef typename ElemTraits<T>::vec4 vec4;
@@ -554,6 +554,29 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
       if (8 * (i >> 2) + (i & 3) > slack) s[nb][i] = -INFINITY;                         \
   }
 
+  // Residual estimator (REWEIGHT instances of the general gathered kernel): the scores of the sampled
+  // chunks get a bias (log of the sample weight, in raw q.k units), and a sampled key that is among the
+  // block keys of this wave's query tile is dead.  Element i of a lane is slot
+  // (chunk - n_blk_chunks)*64 + mb*32 + 4*hi + 8*(i/4) + i%4 of the sample list; its key's position in the
+  // sorted order comes from sampled_pos (the same for all lanes of a lane half: broadcast loads).
+  const int32_t* const smp_pos = REWEIGHT && p.sampled_pos ? p.sampled_pos + sidx_off : nullptr;
+  const int win_first = my_lo - (my_lo >= nk_chunks ? nk_chunks : 0);  // first chunk of the tile's key window
+  const int win_chunks = my_hi - my_lo;
+#define HA_REWEIGHT(ci, mb, s)                                                          \
+  if (REWEIGHT && (ci) >= n_blk_chunks) {                                               \
+    const int slot0 = ((ci) - n_blk_chunks) * KC + (mb) * 32 + 4 * hi;                  \
+    _Pragma("unroll") for (int i = 0; i < 16; ++i) {                                    \
+      bool dead = false;                                                                \
+      if (smp_pos) {                                                                    \
+        int c = (smp_pos[slot0 + 8 * (i >> 2) + (i & 3)] >> 6) - win_first;             \
+        c += c < 0 ? nk_chunks : 0;                                                     \
+        dead = c < win_chunks;                                                          \
+      }                                                                                 \
+      _Pragma("unroll") for (int nb = 0; nb < 2; ++nb)                                  \
+        s[nb][i] = dead ? -INFINITY : s[nb][i] + p.sample_bias_raw;                     \
+    }                                                                                   \
+  }
+
   // ---- Q fragments (B operand), S^T of the first 32 keys ---------------------------------------
   vec8 qf[2][KSTEPS];
 #pragma unroll
@@ -629,12 +652,14 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
     /* causal: once a chunk lies wholly above this wave's queries, so do all later ones */                  \
     if (INTERIOR || !(CAUSAL && (ci) * KC > wave_q_first + 63)) {                                           \
       const bool masked = INTERIOR ? false : chunk_masked(ci);                                              \
-      if (__builtin_expect(masked, false)) { HA_APPLY_MASK(ci, 0, s_a) }                                                             \
+      if (__builtin_expect(masked, false)) { HA_APPLY_MASK(ci, 0, s_a) }                                    \
+      HA_REWEIGHT(ci, 0, s_a)                                                                               \
       half_step<T, D, 0>(s_a, s_b, K_RD, 0, V_CUR, 0, lo, qf, acc, m_run, l_run, pb, vf,                    \
                          p.scale_log2);                                                                     \
       half_step<T, D, 1>(s_a, s_b, K_RD, 0, V_CUR, 16 * D * 2, lo, qf, acc, m_run, l_run, pb, vf,           \
                          p.scale_log2);                                                                     \
-      if (__builtin_expect(masked, false)) { HA_APPLY_MASK(ci, 1, s_b) }                                                             \
+      if (__builtin_expect(masked, false)) { HA_APPLY_MASK(ci, 1, s_b) }                                    \
+      HA_REWEIGHT(ci, 1, s_b)                                                                               \
       half_step<T, D, 0>(s_b, s_a, K_RD, 32 * D * 2, V_CUR, 32 * D * 2, lo, qf, acc, m_run, l_run, pb, vf,  \
                          p.scale_log2);                                                                     \
       half_step<T, D, 1>(s_b, s_a, K_RD, 32 * D * 2, V_CUR, 48 * D * 2, lo, qf, acc, m_run, l_run, pb, vf,  \
@@ -726,19 +751,23 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
 #undef HA_FETCH_ROWS_V
 #undef HA_LOAD_TILE
 #undef HA_APPLY_MASK
+#undef HA_REWEIGHT
 }
 
 namespace {
 
-template <typename T, int D, bool GATHER, bool CAUSAL, bool PLAIN = false, bool NARROW = false>
+template <typename T, int D, bool GATHER, bool CAUSAL, bool PLAIN = false, bool NARROW = false, bool REWEIGHT = false>
 int launch_one(const ha_attn_kernel_params& p, int grid, hipStream_t stream, const char* what) {
-  hipLaunchKernelGGL((ha_attn_fwd_kernel<T, D, GATHER, CAUSAL, PLAIN, NARROW>), dim3(grid), dim3(WG_THREADS), 0, stream, p);
+  hipLaunchKernelGGL((ha_attn_fwd_kernel<T, D, GATHER, CAUSAL, PLAIN, NARROW, REWEIGHT>), dim3(grid), dim3(WG_THREADS), 0,
+                     stream, p);
   return ha_launch_status(what);
 }
 
 template <typename T, int D>
-int launch_variant(const ha_attn_kernel_params& p, int grid, bool gather, bool causal, hipStream_t stream) {
+int launch_variant(const ha_attn_kernel_params& p, int grid, bool gather, bool causal, bool reweight, hipStream_t stream) {
   const bool narrow = p.qk_pieces != D / 8 || p.v_pieces != D / 8;
+  if (gather && reweight)  // the entry point has checked that the head dims are the built ones
+    return launch_one<T, D, true, false, false, false, true>(p, grid, stream, "ha_block_attn_fwd");
   if (gather) {
     const bool plain = !p.smooth && !p.sampled_idx && p.block_tiles % 2 == 0 && p.n_q % WG_QUERIES == 0;
     if (narrow) return launch_one<T, D, true, false, false, true>(p, grid, stream, "ha_block_attn_fwd");
@@ -766,7 +795,7 @@ static ha_divisor make_divisor(int64_t y) {
 }
 
 int ha_attn_launch(const ha_attn_kernel_params& params, int d, int dv, int dtype, bool gather, bool causal,
-                   hipStream_t stream) {
+                   bool reweight, hipStream_t stream) {
   ha_attn_kernel_params p = params;
   // the kernels are built for rows of 64 and 128 elements; other head dims (multiples of 8) run in the
   // next width with the missing pieces of every row read as zeros
@@ -783,9 +812,9 @@ int ha_attn_launch(const ha_attn_kernel_params& params, int d, int dv, int dtype
   const int64_t grid = qtiles * p.batch * p.heads * p.segs;
   if (grid <= 0 || grid >= (1ll << 31)) return ha_fail(HA_ERR_SHAPE, "attention: grid of %lld workgroups", (long long)grid);
   if (dtype == HA_F16) {
-    if (width == 64) return launch_variant<f16_t, 64>(p, (int)grid, gather, causal, stream);
-    return launch_variant<f16_t, 128>(p, (int)grid, gather, causal, stream);
+    if (width == 64) return launch_variant<f16_t, 64>(p, (int)grid, gather, causal, reweight, stream);
+    return launch_variant<f16_t, 128>(p, (int)grid, gather, causal, reweight, stream);
   }
-  if (width == 64) return launch_variant<bf16_t, 64>(p, (int)grid, gather, causal, stream);
-  return launch_variant<bf16_t, 128>(p, (int)grid, gather, causal, stream);
+  if (width == 64) return launch_variant<bf16_t, 64>(p, (int)grid, gather, causal, reweight, stream);
+  return launch_variant<bf16_t, 128>(p, (int)grid, gather, causal, reweight, stream);
 }

@@ -14,6 +14,7 @@ operator by operator under torch autograd.
 from __future__ import annotations
 
 import ctypes
+import math
 
 import torch
 
@@ -185,6 +186,9 @@ class HyperAttention(torch.nn.Module):
         Optional keyword hooks (not in the reference, for reproducible runs): `rng` (torch.Generator
         for the projection), `proj_dir` (explicit (input_dim, lsh_num_projs) projection) and
         `sampled_idx` (explicit sampled key rows, shape (sample_size,)).
+        `residual_estimator=True` (not in the reference either; the estimator of the HyperAttention paper):
+        every hashed call weights its sampled keys by n_key / sample_size and leaves out those that are
+        already among the block keys of the query.  Forward only, head dims 64 and 128.
         """
         super().__init__()
         self.input_dim = input_dim
@@ -198,6 +202,7 @@ class HyperAttention(torch.nn.Module):
             proj = torch.as_tensor(kwargs['proj_dir']).reshape(1, 1, input_dim, lsh_num_projs)
             self.lsh.proj_dir = proj.to(self.lsh.proj_dir.dtype).clone()
         self.sampled_idx = kwargs.get('sampled_idx')
+        self.residual_estimator = bool(kwargs.get('residual_estimator', False))
 
     def forward(self, query: torch.tensor, key: torch.tensor, value: torch.tensor, scale=None, causal=False,
                 return_lse=False):
@@ -241,8 +246,10 @@ class HyperAttention(torch.nn.Module):
         n_key = key.shape[2]
         # gradients are taken operator by operator, as in the reference (each attention operator has its own
         # backward and the merges are differentiable tensor arithmetic); the one-call forward has none
+        if self.residual_estimator and ops._wants_grad(query, key, value):
+            raise NotImplementedError("residual_estimator has no backward")
         if (ops.forward_plan_supported(n_key, self.min_seq_len, causal is not False, self.lsh_num_projs)
-                and not ops._wants_grad(query, key, value)):
+                and not ops._wants_grad(query, key, value) and not self.residual_estimator):
             attn, lse = ops.hyper_forward(
                 query, key, value, proj, scale=scale, causal=causal is not False,
                 lsh_num_projs=self.lsh_num_projs, block_size=self.block_size, sample_size=self.sample_size,
@@ -253,7 +260,7 @@ class HyperAttention(torch.nn.Module):
                 lse = torch.nn.functional.pad(lse, (0, n_rounded - n_key))
             else:
                 lse = lse.unsqueeze(-1)
-        elif (causal is not False and n_key > self.min_seq_len
+        elif (causal is not False and n_key > self.min_seq_len and not self.residual_estimator
               and ops.forward_plan_supported(n_key, self.min_seq_len, True, self.lsh_num_projs)):
             # gradients wanted and every level has an even length: the recursion and its gradient on
             # segments of the whole tensors, grouped-query heads as they are
@@ -321,9 +328,12 @@ class HyperAttention(torch.nn.Module):
             num_keys = 1 << self.lsh_num_projs
             query_sort_idx = ops.bucket_argsort(self.lsh.hash(query, proj), num_keys)
             key_sort_idx = ops.bucket_argsort(self.lsh.hash(key, proj), num_keys)
+            estimator = {}
+            if self.residual_estimator and self.sample_size > 0:
+                estimator = dict(sample_bias=math.log(key.shape[2] / self.sample_size), mask_sampled_in_block=True)
             attn, lse = ops.hyper_attn_func(query.transpose(1, 2), key.transpose(1, 2), value.transpose(1, 2),
                                             query_sort_idx.transpose(1, 2), key_sort_idx.transpose(1, 2),
                                             self.block_size, self.sample_size, scale, self.smooth_block,
-                                            sampled_idx=self.sampled_idx)
+                                            sampled_idx=self.sampled_idx, **estimator)
         attn = attn.transpose(1, 2)
         return attn, lse.unsqueeze(-1)

@@ -199,8 +199,26 @@ def _block_attn_args(q, k, v, o, lse, q_sort_idx, k_sort_idx, block_size, sample
     return a, keep
 
 
+def _sampled_positions(k_sort_idx, sampled_idx, sample_size):
+    """Position of every sampled key row in its head's sorted key order, int32 (batch, nheads, sample_size),
+    plus the sample list expanded to that shape (None for the default rows 0..sample_size-1).
+    k_sort_idx: (batch, seqlen, nheads) permutations."""
+    batch, n, nheads = k_sort_idx.shape
+    order = k_sort_idx.transpose(1, 2).long()                                    # (b, h, n): row at each position
+    inverse = torch.empty_like(order)
+    inverse.scatter_(2, order, torch.arange(n, device=order.device).expand_as(order))  # position of each row
+    if sampled_idx is None:
+        rows, expanded = torch.arange(sample_size, device=order.device).expand(batch, nheads, -1), None
+    else:
+        rows = sampled_idx.to(device=order.device, dtype=torch.long)
+        rows = rows.expand(batch, nheads, sample_size) if rows.dim() < 3 else rows
+        expanded = rows.to(k_sort_idx.dtype).contiguous()
+    return inverse.gather(2, rows).to(torch.int32).contiguous(), expanded
+
+
 def hyper_attn_func(q, k, v, q_sort_idx, k_sort_idx, block_size, sample_size=0, softmax_scale=None,
-                    smooth_block=False, *, sampled_idx=None, resume=None):
+                    smooth_block=False, *, sampled_idx=None, resume=None, sample_bias=0.0,
+                    mask_sampled_in_block=False):
     """q, k: (batch, seqlen, nheads, headdim); v: (batch, seqlen, nheads, v_headdim);
     q_sort_idx, k_sort_idx: (batch, seqlen, nheads) permutations; returns o (batch, seqlen, nheads,
     v_headdim) and lse (batch, nheads, seqlen) fp32.  `sampled_idx` (keyword only, not in the
@@ -208,9 +226,20 @@ def hyper_attn_func(q, k, v, q_sort_idx, k_sort_idx, block_size, sample_size=0, 
     (nheads, sample_size) / (batch, nheads, sample_size) for a list per head; default 0..sample_size-1.
     `resume` (keyword only, not in the reference) is a pair (o, lse) of a previous partial attention
     over other keys, shaped like the results: the kernel continues from it and updates both in place,
-    which equals add_self_attentions(previous, this call) in fp32."""
+    which equals add_self_attentions(previous, this call) in fp32.
+    `sample_bias`, `mask_sampled_in_block` (keyword only, not in the reference): the residual estimator of
+    the HyperAttention paper.  The bias (e.g. log(seqlen_k / sample_size)) is added to the scaled score of
+    every sampled key; with the mask a sampled key that is also among the block keys of the query's tile is
+    left out of the sampled part.  Forward only, head dims 64 and 128."""
     q, k, v = [x if x.stride(-1) == 1 else x.contiguous() for x in [q, k, v]]
     assert sample_size % 128 == 0
+    reweight = bool(sample_bias) or bool(mask_sampled_in_block)
+    if reweight:
+        if _wants_grad(q, k, v):
+            raise NotImplementedError("the residual estimator (sample_bias, mask_sampled_in_block) has no backward")
+        assert v.shape[-1] == q.shape[-1] and q.shape[-1] in KERNEL_HEAD_DIMS, \
+            "the residual estimator is built for head dims 64 and 128"
+        assert sample_size > 0, "the residual estimator needs sampled keys"
     built = v.shape[-1] == q.shape[-1] and q.shape[-1] in KERNEL_HEAD_DIMS
     if _wants_grad(q, k, v) and built:
         assert resume is None, "resume has no backward"
@@ -252,8 +281,19 @@ def hyper_attn_func(q, k, v, q_sort_idx, k_sort_idx, block_size, sample_size=0, 
         assert o.stride(-1) == 1
     assert seqlen_k % 128 == 0, "keys sequence length must be divisible by 128"
 
+    pos = None
+    if mask_sampled_in_block:
+        # a position per (batch, head, slot): the sample list goes in that shape too (one set of strides)
+        if sampled_idx is not None:
+            check_sampled_idx(sampled_idx, seqlen_k)
+        pos, sampled_idx = _sampled_positions(k_sort_idx, sampled_idx, sample_size)
     a, keep = _block_attn_args(q, k, v, o, lse, q_sort_idx, k_sort_idx, block_size, sample_size, softmax_scale,
                                smooth_block, sampled_idx, accumulate=resume is not None)
+    if reweight:
+        a.sample_bias = float(sample_bias)
+        if pos is not None:
+            a.sampled_pos, a.mask_sampled_in_block = pos.data_ptr(), 1
+            a.sampled_stride_b, a.sampled_stride_h = pos.shape[1] * sample_size, sample_size
     with torch.cuda.device(q.device):
         _lib.check(_lib.lib().ha_block_attn_fwd(ctypes.byref(a), _stream(q)))
     return o, lse

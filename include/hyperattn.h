@@ -23,7 +23,7 @@
 extern "C" {
 #endif
 
-#define HA_ABI_VERSION 5
+#define HA_ABI_VERSION 6
 
 typedef enum {
   HA_OK = 0,
@@ -143,6 +143,15 @@ typedef struct {
  * missing columns as zeros.
  * accumulate != 0: out/lse already hold a partial attention over a disjoint key set for every row;
  * the result is merged into them in place (add_self_attentions, src/attn_utils.py:6-24, fused).
+ * Residual estimator (no counterpart in the reference, whose sampled loop is src/hyper_attn_triton.py:142-173:
+ * un-weighted, duplicates counted; this is the variant of the HyperAttention paper, off unless asked for):
+ *   sample_bias != 0: added to the scaled score of every sampled key, e.g. log(n_k / sample_size), which
+ *     weights each sample by n_k / sample_size in the soft-max sums;
+ *   mask_sampled_in_block != 0: a sampled key that is also among the block keys of the query's tile (its
+ *     block, or its smooth window) is left out of the sampled part, so no key is counted twice.  Needs
+ *     sampled_pos: for every entry of the sample list the position of that key row in the head's sorted key
+ *     order (int32, laid out and strided like sampled_idx; required even when sampled_idx is NULL).
+ * Forward only (ha_block_attn_bwd rejects it), d == dv in {64, 128}.
  */
 typedef struct {
   ha_attn_operands t;
@@ -156,6 +165,9 @@ typedef struct {
   int64_t block_size, sample_size;
   int smooth_block;
   int accumulate;
+  const int32_t* sampled_pos;
+  float sample_bias;
+  int mask_sampled_in_block;
 } ha_block_attn_args;
 
 int ha_block_attn_fwd(const ha_block_attn_args* args, void* stream);

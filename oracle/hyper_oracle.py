@@ -223,7 +223,8 @@ def block_key_positions(n_q: int, n_k: int, block_size: int, smooth_block: bool)
 
 def block_sampled_attention(q, k, v, q_sort_idx, k_sort_idx, block_size, sample_size=0,
                             scale=None, smooth_block=False, sampled_idx=None,
-                            dtype=torch.float64, round_dtype=None):
+                            dtype=torch.float64, round_dtype=None, sample_bias=0.0,
+                            mask_sampled_in_block=False):
     """Sorted block-diagonal + fixed-column attention, (b,h,n,d) layout.
 
     Follows src/hyper_attn_triton.py:70-192 (``_fwd_hyper_kernel``): tile ``t`` of 128 sorted
@@ -237,6 +238,11 @@ def block_sampled_attention(q, k, v, q_sort_idx, k_sort_idx, block_size, sample_
     Returns out (b,h,nq,dv) and lse (b,h,nq) in ``dtype``.  ``round_dtype``: the kernel's own
     roundings as in exact_attention (P to the value type before both P.V products, :135 and :167;
     out stored in that type, :189-192; lse float32, :688).
+    ``sample_bias`` / ``mask_sampled_in_block`` (NOT in the reference; the residual estimator of the
+    HyperAttention paper): the bias is added to the scaled score of every sampled key (log of the weight a
+    sample carries in the soft-max sums), and with the mask a sampled key that is among the valid block
+    keys of the query's tile is left out of the sampled part.  Pinned by the per-row definition in
+    tests/test_oracle.py.
     """
     q = torch.as_tensor(q).to(dtype)
     k = torch.as_tensor(k).to(dtype)
@@ -274,7 +280,11 @@ def block_sampled_attention(q, k, v, q_sort_idx, k_sort_idx, block_size, sample_
             if sample_size > 0:
                 ks = k[ib, ih][si[ib, ih]]
                 vs = v[ib, ih][si[ib, ih]]
-                s_smp = torch.matmul(qs, ks.t()) * scale
+                s_smp = torch.matmul(qs, ks.t()) * scale + sample_bias
+                if mask_sampled_in_block:
+                    # (tiles, width, s): sampled row j equals valid block key w of tile t
+                    same = (krow[:, :, None] == si[ib, ih][None, None, :]) & valid[:, :, None]
+                    s_smp = s_smp.masked_fill(same.any(dim=1)[:, None, :], float("-inf"))
                 scores = torch.cat([s_blk, s_smp], dim=-1)
             else:
                 scores = s_blk
@@ -311,16 +321,20 @@ def add_self_attentions(attn1, lse1, attn2, lse2):
 
 def forward_no_causal_mask(q, k, v, scale, proj, lsh_num_projs, block_size, sample_size,
                            min_seq_len, smooth_block, sampled_idx=None, dtype=torch.float64,
-                           detach_lse=False, round_dtype=None):
-    """Follows hyper_attention.py:103-132.  Returns attn (b,h,n,dv), lse (b,h,n,1)."""
+                           detach_lse=False, round_dtype=None, residual_estimator=False):
+    """Follows hyper_attention.py:103-132.  Returns attn (b,h,n,dv), lse (b,h,n,1).
+    ``residual_estimator`` (not in the reference): the hashed call weights its samples by
+    n_key / sample_size and leaves out those that lie in the query's block (block_sampled_attention)."""
     n_query = q.shape[2]
     if min_seq_len > n_query:  # :109
         attn, lse = exact_attention(q, k, v, scale, False, dtype, round_dtype=round_dtype)
     else:
         q_idx = stable_bucket_argsort(lsh_hash(q, proj))  # :116
         k_idx = stable_bucket_argsort(lsh_hash(k, proj))  # :117
+        est = dict(sample_bias=math.log(k.shape[2] / sample_size), mask_sampled_in_block=True) \
+            if residual_estimator and sample_size > 0 else {}
         attn, lse = block_sampled_attention(q, k, v, q_idx, k_idx, block_size, sample_size,
-                                            scale, smooth_block, sampled_idx, dtype, round_dtype=round_dtype)
+                                            scale, smooth_block, sampled_idx, dtype, round_dtype=round_dtype, **est)
     if detach_lse:
         lse = lse.detach()
     return attn, lse.unsqueeze(-1)
@@ -328,7 +342,7 @@ def forward_no_causal_mask(q, k, v, scale, proj, lsh_num_projs, block_size, samp
 
 def hyper_forward(q, k, v, proj, scale=None, causal=False, lsh_num_projs=8, block_size=256,
                   sample_size=256, min_seq_len=2048, smooth_block=False, sampled_idx=None,
-                  dtype=torch.float64, detach_lse=False, round_dtype=None):
+                  dtype=torch.float64, detach_lse=False, round_dtype=None, residual_estimator=False):
     """HyperAttention.forward with return_lse=True, (b,h,n,d) layout.
 
     Follows hyper_attention.py:25-101: non-causal dispatch (:48-49), causal leaf (:52-57),
@@ -357,7 +371,8 @@ def hyper_forward(q, k, v, proj, scale=None, causal=False, lsh_num_projs=8, bloc
     assert n_query == n_key  # :45
     kw = dict(proj=proj, lsh_num_projs=lsh_num_projs, block_size=block_size,
               sample_size=sample_size, min_seq_len=min_seq_len, smooth_block=smooth_block,
-              sampled_idx=sampled_idx, dtype=dtype, detach_lse=detach_lse, round_dtype=round_dtype)
+              sampled_idx=sampled_idx, dtype=dtype, detach_lse=detach_lse, round_dtype=round_dtype,
+              residual_estimator=residual_estimator)
     if causal is False:
         return forward_no_causal_mask(q, k, v, scale, **kw)
     if n_key <= min_seq_len:  # :52

@@ -199,6 +199,24 @@ def test_other_head_dims_leave_the_module_as_it_is(ha):
     assert m.lsh.proj_dir.shape == before.shape and torch.equal(m.lsh.proj_dir, before)
 
 
+@pytest.mark.parametrize("causal", [False, True])
+def test_module_residual_estimator(ha, causal):
+    """residual_estimator=True (not in the reference): samples weighted by n_key / sample_size, block keys left out
+    of them, in every hashed call of the recursion; against the oracle's option."""
+    dtype, n = torch.float16, 2048
+    q, k, v = (_randn((1, 2, n, 64), s, dtype) for s in (190, 191, 192))
+    m, proj = _module(ha, 64, dtype, 193, block_size=128, sample_size=128, min_seq_len=512, residual_estimator=True)
+    attn, lse = m(q.cuda(), k.cuda(), v.cuda(), causal=causal, return_lse=True)
+    ro, rl = O.hyper_forward(q, k, v, proj, causal=causal, block_size=128, sample_size=128, min_seq_len=512,
+                             residual_estimator=True)
+    assert_close(attn, ro, "attn", dtype)
+    assert_close(lse, rl, "lse")
+    plain, _ = _module(ha, 64, dtype, 193, block_size=128, sample_size=128, min_seq_len=512)
+    assert float((plain(q.cuda(), k.cuda(), v.cuda(), causal=causal).float() - attn.float()).abs().max()) > 1e-3
+    with pytest.raises(NotImplementedError):
+        m(q.cuda().requires_grad_(), k.cuda(), v.cuda(), causal=causal)
+
+
 def test_module_argument_errors(ha):
     m, _ = _module(ha, 64, torch.float16, 160)
     q = torch.zeros((1, 1, 256, 64), dtype=torch.float16, device="cuda")

@@ -314,6 +314,50 @@ def test_block_attention_resumes_partial_result(ha, dtype, shift):
     assert_close(lse, want_lse, "resumed lse")
 
 
+@pytest.mark.parametrize("dtype,d,smooth,block,per_head", [
+    (torch.float16, 64, False, 256, False),
+    (torch.bfloat16, 128, True, 256, True),
+    (torch.float16, 64, True, 128, False),
+])
+def test_residual_estimator_option(ha, dtype, d, smooth, block, per_head):
+    """sample_bias + mask_sampled_in_block (the HyperAttention paper's residual estimator; not in the reference)
+    against the oracle option, which tests/test_oracle.py pins by the per-row definition.  The sample list
+    has repeats and entries inside and outside every tile's key window."""
+    b, h, n, samples = 2, 2, 1024, 128
+    q, k, v, qi, ki = _sorted_inputs(b, h, n, d, dtype, 90)
+    g = _gen(91)
+    sampled = torch.randint(0, n, (h, samples) if per_head else (samples,), generator=g)
+    bias = float(np.log(n / samples))
+    kw = dict(sampled_idx=sampled.cuda(), sample_bias=bias, mask_sampled_in_block=True)
+    o, lse = ha.hyper_attn_func(q.transpose(1, 2).cuda(), k.transpose(1, 2).cuda(), v.transpose(1, 2).cuda(),
+                                qi.transpose(1, 2).cuda(), ki.transpose(1, 2).cuda(), block, samples, None, smooth, **kw)
+    s_full = sampled.view(1, h, samples).expand(b, h, samples) if per_head else sampled
+    ro, rl = O.block_sampled_attention(q, k, v, qi, ki, block, samples, None, smooth, s_full, sample_bias=bias,
+                                       mask_sampled_in_block=True)
+    # (bf16: the secondary bar of _util; the option has no reference arithmetic to be measured against)
+    assert_close(o.transpose(1, 2), ro, "estimator out", dtype)
+    assert_close(lse, rl, "estimator lse")
+    # the option changes the result (the plain operator counts the samples un-weighted and twice)
+    plain, _ = ha.hyper_attn_func(q.transpose(1, 2).cuda(), k.transpose(1, 2).cuda(), v.transpose(1, 2).cuda(),
+                                  qi.transpose(1, 2).cuda(), ki.transpose(1, 2).cuda(), block, samples, None, smooth,
+                                  sampled_idx=sampled.cuda())
+    assert float((plain.float() - o.float()).abs().max()) > 1e-3
+    # default sample list (rows 0 .. samples-1) with the mask, bias alone, and the error paths
+    o2, lse2 = ha.hyper_attn_func(q.transpose(1, 2).cuda(), k.transpose(1, 2).cuda(), v.transpose(1, 2).cuda(),
+                                  qi.transpose(1, 2).cuda(), ki.transpose(1, 2).cuda(), block, samples, None, smooth,
+                                  mask_sampled_in_block=True)
+    ro2, rl2 = O.block_sampled_attention(q, k, v, qi, ki, block, samples, None, smooth, None, mask_sampled_in_block=True)
+    assert_close(lse2, rl2, "default samples, masked: lse")
+    o3, lse3 = ha.hyper_attn_func(q.transpose(1, 2).cuda(), k.transpose(1, 2).cuda(), v.transpose(1, 2).cuda(),
+                                  qi.transpose(1, 2).cuda(), ki.transpose(1, 2).cuda(), block, samples, None, smooth,
+                                  sample_bias=bias)
+    ro3, rl3 = O.block_sampled_attention(q, k, v, qi, ki, block, samples, None, smooth, None, sample_bias=bias)
+    assert_close(lse3, rl3, "bias alone: lse")
+    with pytest.raises(NotImplementedError):
+        ha.hyper_attn_func(q.transpose(1, 2).cuda().requires_grad_(), k.transpose(1, 2).cuda(), v.transpose(1, 2).cuda(),
+                           qi.transpose(1, 2).cuda(), ki.transpose(1, 2).cuda(), block, samples, None, smooth, sample_bias=bias)
+
+
 def test_block_attention_value_dim_differs(ha):
     """unit_tests/test_hyper_attention.py:120-133: V narrower than Q and K gives the matching columns
     of the full-width result; the other way round (wider V) follows from the same definition."""

@@ -181,6 +181,71 @@ def test_block_sampled_bruteforce(smooth, block_size, sample_size, n):
         assert torch.allclose(lse[0, h], bl, atol=1e-11)
 
 
+@pytest.mark.parametrize("smooth", [False, True])
+def test_residual_estimator_per_row_definition(smooth):
+    """sample_bias / mask_sampled_in_block against the definition written out per row: every block key has
+    weight 1, every sampled key that is NOT among the row's block keys has weight w = exp(bias), the others 0;
+    out = sum(weight * exp(s) * v) / sum(weight * exp(s)), lse = log of the denominator."""
+    n, block, samples, scale, weight = 512, 256, 128, 0.3, 512 / 128
+    q, k, v = (_rand((1, 2, n, 16), s, torch.float32).double() for s in (24, 25, 26))
+    g = torch.Generator().manual_seed(27)
+    qi = torch.stack([torch.randperm(n, generator=g) for _ in range(2)]).view(1, 2, n)
+    ki = torch.stack([torch.randperm(n, generator=g) for _ in range(2)]).view(1, 2, n)
+    sampled = torch.randint(0, n, (samples,), generator=g)   # with repeats; about half fall in a row's block
+    out, lse = O.block_sampled_attention(q, k, v, qi, ki, block, samples, scale, smooth, sampled,
+                                         sample_bias=math.log(weight), mask_sampled_in_block=True)
+    T = block // 128
+    hits = 0
+    for h in range(2):
+        for i in range(0, n, 37):
+            t = i // 128
+            if smooth:
+                first = t * 128 + 64 - T * 64
+                cols = [int(ki[0, h, (first + u) % n]) for u in range(block)]
+            else:
+                lo = (t // T) * block
+                cols = [int(ki[0, h, p_]) for p_ in range(lo, lo + block)]
+            extra = [int(s_) for s_ in sampled if int(s_) not in set(cols)]
+            hits += samples - len(extra)
+            row = int(qi[0, h, i])
+            e_blk = torch.exp((k[0, h][cols] @ q[0, h, row]) * scale)
+            e_smp = weight * torch.exp((k[0, h][extra] @ q[0, h, row]) * scale)
+            den = e_blk.sum() + e_smp.sum()
+            want = ((e_blk[:, None] * v[0, h][cols]).sum(0) + (e_smp[:, None] * v[0, h][extra]).sum(0)) / den
+            assert torch.allclose(out[0, h, row], want, atol=1e-11)
+            assert abs(float(lse[0, h, row]) - math.log(float(den))) < 1e-11
+    assert hits > 0
+    # bias alone: the plain operator's sampled part with every sample weighted; no bias, no mask: the plain operator
+    plain = O.block_sampled_attention(q, k, v, qi, ki, block, samples, scale, smooth, sampled)
+    same = O.block_sampled_attention(q, k, v, qi, ki, block, samples, scale, smooth, sampled, sample_bias=0.0,
+                                     mask_sampled_in_block=False)
+    assert torch.equal(plain[0], same[0]) and torch.equal(plain[1], same[1])
+
+
+def test_residual_estimator_is_unbiased_for_the_row_sums():
+    """What the estimator is for: with the block keys removed from the samples and each remaining sample
+    weighted by (n - block) / (its count), the expectation of the estimated soft-max denominator over a
+    uniformly drawn sample of the non-block keys equals the exact denominator.  Checked in closed form by
+    enumerating ALL samples of size 1 (the mean over the n - block single-key samples, weight n - block)."""
+    n, block, scale = 256, 128, 0.4
+    q, k, v = (_rand((1, 1, n, 8), s, torch.float32).double() for s in (28, 29, 30))
+    idn = torch.arange(n).view(1, 1, n)
+    exact_den = torch.exp(torch.logsumexp((q[0, 0] @ k[0, 0].t()) * scale, dim=-1))
+    rows = torch.arange(0, n, 16)
+    acc = torch.zeros(len(rows), dtype=torch.float64)
+    for j in range(n):   # one sampled key j, repeated to fill a 128-slot list: each slot weighted (n - block) / 128
+        lse = O.block_sampled_attention(q, k, v, idn, idn, block, 128, scale, False, np.full(128, j),
+                                        sample_bias=math.log((n - block) / 128), mask_sampled_in_block=True)[1]
+        acc += torch.exp(lse[0, 0, rows])
+    # for a row of block B: every key outside B is the sample once (contributing its block sum + (n-block) e_j),
+    # every key inside B is masked (contributing the block sum alone): mean over the n - block outside keys
+    blk = (rows // block)
+    blk_den = torch.stack([torch.exp((k[0, 0][b * block:(b + 1) * block] @ q[0, 0, r]) * scale).sum()
+                           for r, b in zip(rows.tolist(), blk.tolist())])
+    mean_outside = (acc - block * blk_den) / (n - block)
+    assert torch.allclose(mean_outside, exact_den[rows], rtol=1e-10)
+
+
 def test_block_sampled_default_sample_is_first_rows():
     n = 256
     q, k, v = (_rand((1, 1, n, 8), s, torch.float32).double() for s in (30, 31, 32))
