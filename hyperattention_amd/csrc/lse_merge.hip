@@ -157,7 +157,8 @@ struct MergeLevels {
   int levels;
 };
 
-template <typename T>
+// MAXL: levels the instance is unrolled for (the recursion rarely goes deeper than 8)
+template <typename T, int MAXL>
 __global__ __launch_bounds__(256) void lse_merge_levels_kernel(const T* __restrict__ o_leaf, const float* __restrict__ lse_leaf,
                                                                T* __restrict__ out, float* __restrict__ lse_out,
                                                                float* __restrict__ leaf_shifted, MergeLevels lv,
@@ -174,9 +175,9 @@ __global__ __launch_bounds__(256) void lse_merge_levels_kernel(const T* __restri
   float x = lse_leaf[row];
   const float x_leaf = x;
   vec8 r = *reinterpret_cast<const vec8*>(o_leaf + at);
-  float c_of[MERGE_MAX_LEVELS], x_of[MERGE_MAX_LEVELS];
+  float c_of[MAXL], x_of[MAXL];
 #pragma unroll
-  for (int j = MERGE_MAX_LEVELS - 1; j >= 0; --j) {
+  for (int j = MAXL - 1; j >= 0; --j) {
     c_of[j] = 1.0f;
     x_of[j] = 0.0f;
     if (j < lv.levels && ((leaf_no >> (lv.levels - 1 - j)) & 1u)) {
@@ -196,7 +197,7 @@ __global__ __launch_bounds__(256) void lse_merge_levels_kernel(const T* __restri
   if (!leaf_shifted) return;
   float log_w = 0.0f;  // log of the product of the weights c of the shallower levels
 #pragma unroll
-  for (int j = 0; j < MERGE_MAX_LEVELS; ++j) {
+  for (int j = 0; j < MAXL; ++j) {
     if (j < lv.levels && ((leaf_no >> (lv.levels - 1 - j)) & 1u)) {
       lv.shifted[j][row] = x_of[j] - log1pf(-c_of[j]) - log_w;
       log_w += logf(c_of[j]);
@@ -242,11 +243,14 @@ extern "C" int ha_lse_merge_levels(const void* o_leaf, const float* lse_leaf, co
   HA_REQUIRE((items + 255) / 256 < (1ll << 31), HA_ERR_SHAPE, "ha_lse_merge_levels: too many rows");
   dim3 grid((unsigned)((items + 255) / 256));
   hipStream_t s = (hipStream_t)stream;
-  if (dtype == HA_F16)
-    hipLaunchKernelGGL((lse_merge_levels_kernel<f16_t>), grid, dim3(256), 0, s, (const f16_t*)o_leaf, lse_leaf,
-                       (f16_t*)out, lse_out, leaf_shifted, lv, rows, n, pieces);
-  else
-    hipLaunchKernelGGL((lse_merge_levels_kernel<bf16_t>), grid, dim3(256), 0, s, (const bf16_t*)o_leaf, lse_leaf,
-                       (bf16_t*)out, lse_out, leaf_shifted, lv, rows, n, pieces);
+#define HA_MERGE_LEVELS(TT, LL)                                                                                  \
+  hipLaunchKernelGGL((lse_merge_levels_kernel<TT, LL>), grid, dim3(256), 0, s, (const TT*)o_leaf, lse_leaf, (TT*)out, \
+                     lse_out, leaf_shifted, lv, rows, n, pieces)
+  if (dtype == HA_F16) {
+    if (levels <= 8) HA_MERGE_LEVELS(f16_t, 8); else HA_MERGE_LEVELS(f16_t, MERGE_MAX_LEVELS);
+  } else {
+    if (levels <= 8) HA_MERGE_LEVELS(bf16_t, 8); else HA_MERGE_LEVELS(bf16_t, MERGE_MAX_LEVELS);
+  }
+#undef HA_MERGE_LEVELS
   return ha_launch_status("ha_lse_merge_levels");
 }
