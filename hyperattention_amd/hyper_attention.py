@@ -203,6 +203,8 @@ class HyperAttention(torch.nn.Module):
             self.lsh.proj_dir = proj.to(self.lsh.proj_dir.dtype).clone()
         self.sampled_idx = kwargs.get('sampled_idx')
         self.residual_estimator = bool(kwargs.get('residual_estimator', False))
+        # workspace of the one-call forward, one per (device, stream), kept between calls
+        self._workspace = {}
 
     def forward(self, query: torch.tensor, key: torch.tensor, value: torch.tensor, scale=None, causal=False,
                 return_lse=False):
@@ -253,7 +255,8 @@ class HyperAttention(torch.nn.Module):
             attn, lse = ops.hyper_forward(
                 query, key, value, proj, scale=scale, causal=causal is not False,
                 lsh_num_projs=self.lsh_num_projs, block_size=self.block_size, sample_size=self.sample_size,
-                min_seq_len=self.min_seq_len, smooth_block=self.smooth_block, sampled_idx=self.sampled_idx)
+                min_seq_len=self.min_seq_len, smooth_block=self.smooth_block, sampled_idx=self.sampled_idx,
+                workspace=self._workspace)
             if causal is not False and n_key <= self.min_seq_len:
                 # the reference returns the exact kernel's padded 3-d lse for a top-level leaf
                 n_rounded = -(-n_key // 128) * 128

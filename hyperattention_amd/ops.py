@@ -446,9 +446,11 @@ def forward_plan_supported(n: int, min_seq_len: int, causal: bool, lsh_num_projs
 
 
 def _forward_args(q, k, v, out, lse, proj, *, scale, causal, lsh_num_projs, block_size, sample_size, min_seq_len,
-                  smooth_block, sampled_idx=None):
+                  smooth_block, sampled_idx=None, workspace=None):
     """ForwardArgs for (b,h,n,d) q and (b,h_kv,n,d) k, v with its workspace attached; the second result keeps
-    the tensors alive that the struct only points to."""
+    the tensors alive that the struct only points to (the workspace last).  `workspace`: a dict the caller
+    owns; the workspace tensor of the current (device, stream) is kept there and reused while it is large
+    enough, so that a caller that runs many forwards does not allocate one per call."""
     assert q.is_cuda and k.is_cuda
     assert q.stride(-1) == 1 and k.stride(-1) == 1 and (v is None or v.stride(-1) == 1)
     assert q.dtype == k.dtype and (v is None or v.dtype == q.dtype), "All tensors must have the same type"
@@ -485,23 +487,31 @@ def _forward_args(q, k, v, out, lse, proj, *, scale, causal, lsh_num_projs, bloc
     ws_bytes = _lib.lib().ha_forward_workspace_bytes(ctypes.byref(a))
     if ws_bytes < 0:
         _lib.check(int(ws_bytes))
-    ws = torch.empty(int(ws_bytes), device=q.device, dtype=torch.uint8)
+    ws = None
+    if workspace is not None:
+        slot = (q.device.index, torch.cuda.current_stream(q.device).cuda_stream)
+        ws = workspace.get(slot)
+    if ws is None or ws.numel() < int(ws_bytes):
+        ws = torch.empty(int(ws_bytes), device=q.device, dtype=torch.uint8)
+        if workspace is not None:
+            workspace[slot] = ws
     a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
     keep.append(ws)
     return a, keep
 
 
 def hyper_forward(q, k, v, proj, *, scale, causal, lsh_num_projs, block_size, sample_size, min_seq_len,
-                  smooth_block, sampled_idx=None):
+                  smooth_block, sampled_idx=None, workspace=None):
     """One-call forward for (b,h,n,d) q and (b,h_kv,n,d) k, v of any strides with a contiguous last
-    dimension (permuted views are read in place).  Returns contiguous out (b,h,n,dv) and lse (b,h,n) fp32."""
+    dimension (permuted views are read in place).  Returns contiguous out (b,h,n,dv) and lse (b,h,n) fp32.
+    `workspace`: see _forward_args."""
     assert v.is_cuda
     b, h, n, d = q.shape
     out = torch.empty((b, h, n, v.shape[-1]), device=q.device, dtype=q.dtype)
     lse = torch.empty((b, h, n), device=q.device, dtype=torch.float32)
     a, keep = _forward_args(q, k, v, out, lse, proj, scale=scale, causal=causal, lsh_num_projs=lsh_num_projs,
                             block_size=block_size, sample_size=sample_size, min_seq_len=min_seq_len,
-                            smooth_block=smooth_block, sampled_idx=sampled_idx)
+                            smooth_block=smooth_block, sampled_idx=sampled_idx, workspace=workspace)
     with torch.cuda.device(q.device):
         _lib.check(_lib.lib().ha_forward(ctypes.byref(a), _stream(q)))
     return out, lse
