@@ -206,7 +206,7 @@ void layout_workspace(const ha_forward_args& a, const Plan& pl, Workspace& w) {
     for (int j = 0; j < nlev; ++j)
       if (pl.level_hyper[j]) longest = std::max<int64_t>(longest, a.causal ? pl.len[j] / 2 : a.n);
     w.units = a.lsh_num_projs <= 8 && longest / g.granule * g.units_per_granule <= max_units_per_segment(g.unit) &&
-              a.n % g.granule == 0 && (a.d == 32 || a.d == 64 || a.d == 128);   // the widths the paired hash is built for
+              a.n % g.granule == 0;
     const int64_t id_bytes = w.units ? 1 : 4;
     w.buckets_q = off; off += align256(a.batch * a.heads * a.n * id_bytes);
     w.buckets_k = off; off += align256(a.batch * a.kv_heads * a.n * id_bytes);

@@ -2,81 +2,20 @@
 // Follows the definition in src/angular_lsh_triton.py:76-88 and :175-179 of the reference
 // (bit_j = [x . P[:, j] > 0], bin = sum_j bit_j << j, bucket = perm[bin], perm[i] = i ^ (i >> 1)).
 //
-// Two kernels.
-//
-// lsh_hash_mfma_kernel (head dims that are multiples of 32): a wave projects 16 rows at a time with
-// v_mfma_f32_16x16x32 (rows x 16 projection slots, fp32 accumulation), reading the rows straight from
-// HBM as MFMA operands, so the kernel is purely bandwidth bound.  fp32 accumulation cannot decide the
+// lsh_hash_mfma_kernel: a wave projects 16 rows at a time with v_mfma_f32_16x16x32 (rows x 16 projection
+// slots, fp32 accumulation), reading the rows straight from HBM as MFMA operands, so the kernel is purely
+// bandwidth bound.  Built for rows of 32, 64, 128 and 256 elements; a row of any other multiple of 8
+// elements runs in the next width with its missing elements (and the missing rows of the projection) read
+// as zeros.  fp32 accumulation cannot decide the
 // sign of a projection that nearly cancels, so a second MFMA on |x| and |P| gives sum |x_k P_kj|, which
 // bounds the accumulation error of any summation order (d * 2^-23 * sum, used with a factor 2 margin;
 // fp16/bf16 products are exact in fp32 and subnormal inputs are not flushed).  Whenever some
 // |projection| is inside that bound, the 16-row tile is recomputed in fp64 (products exact, sum exact
 // to 2^-53), which happens for well under 1 % of the tiles on random data.
-//
-// lsh_hash_kernel (any head dim that is a multiple of 8): one thread per row, rows staged through
-// LDS with coalesced 16-byte loads, all projections accumulated in fp64.
 #include "ha_common.h"
 #include "bucket_sort.h"
 
 namespace {
-
-template <typename T, int RMAX>
-__global__ void lsh_hash_kernel(const T* __restrict__ x, const T* __restrict__ proj,
-                                int32_t* __restrict__ buckets, int heads, int64_t n, int d, int r,
-                                int64_t sb, int64_t sh, int64_t sn, int64_t psb, int64_t psh) {
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  double* P = reinterpret_cast<double*>(smem);                         // [d][RMAX]
-  u32x4* rows = reinterpret_cast<u32x4*>(smem + (size_t)d * RMAX * 8);  // [blockDim.x][d/8] 16-byte chunks
-
-  const int tid = threadIdx.x;
-  const int nthreads = blockDim.x;
-  const int bh = blockIdx.y;
-  const int b = bh / heads, h = bh % heads;
-  const int64_t row0 = (int64_t)blockIdx.x * nthreads;
-  const int cpr = d >> 3;  // 16-byte chunks per row
-  // XOR swizzle of the chunk index by the row: only when it stays inside the row
-  const int swz = (cpr % 8 == 0) ? 7 : (((cpr & (cpr - 1)) == 0) ? cpr - 1 : 0);
-
-  const T* pbase = proj + b * psb + h * psh;
-  for (int i = tid; i < d * RMAX; i += nthreads) {
-    const int k = i / RMAX, j = i % RMAX;
-    P[i] = j < r ? (double)ha_to_float(pbase[(int64_t)k * r + j]) : 0.0;
-  }
-
-  const T* xbase = x + b * sb + h * sh;
-  const int total_chunks = nthreads * cpr;
-  for (int i = tid; i < total_chunks; i += nthreads) {
-    const int lr = i / cpr, c = i % cpr;
-    const int64_t grow = row0 + lr;
-    u32x4 val = {0u, 0u, 0u, 0u};
-    if (grow < n) val = *reinterpret_cast<const u32x4*>(xbase + grow * sn + c * 8);
-    rows[lr * cpr + (c ^ (lr & swz))] = val;
-  }
-  __syncthreads();
-
-  double acc[RMAX];
-#pragma unroll
-  for (int j = 0; j < RMAX; ++j) acc[j] = 0.0;
-
-  typedef typename ElemTraits<T>::vec8 vec8;
-  for (int c = 0; c < cpr; ++c) {
-    u32x4 raw = rows[tid * cpr + (c ^ (tid & swz))];
-    vec8 xv = __builtin_bit_cast(vec8, raw);
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const double xe = (double)(float)xv[e];
-      const double* pk = P + (c * 8 + e) * RMAX;
-#pragma unroll
-      for (int j = 0; j < RMAX; ++j) acc[j] = __builtin_fma(xe, pk[j], acc[j]);
-    }
-  }
-
-  int bin = 0;
-#pragma unroll
-  for (int j = 0; j < RMAX; ++j) bin |= (acc[j] > 0.0 ? 1 : 0) << j;
-  const int64_t grow = row0 + tid;
-  if (grow < n) buckets[(int64_t)bh * n + grow] = bin ^ (bin >> 1);
-}
 
 template <typename T>
 struct HashMfma;
@@ -113,7 +52,7 @@ struct HashTensors {
 
 template <typename T, int D, bool OUT8>
 __global__ __launch_bounds__(256) void lsh_hash_mfma_kernel(const HashTensors ten, const T* __restrict__ proj, int64_t n,
-                                                            int r, int64_t psb, int64_t psh) {
+                                                            int r, int64_t psb, int64_t psh, int d_real) {
   typedef typename ElemTraits<T>::vec8 vec8;
   constexpr int PARTS = D / 32;
   constexpr int ROWS = 16 / PARTS;            // data rows per tile
@@ -135,7 +74,9 @@ __global__ __launch_bounds__(256) void lsh_hash_mfma_kernel(const HashTensors te
   // the projection matrix goes through LDS once per block (one coalesced pass instead of a chain of
   // dependent 2-byte loads per lane)
   __shared__ T lds_p[D * 16];
-  for (int i = threadIdx.x; i < D * r; i += blockDim.x) lds_p[i] = pbase[i];
+  // rows of d_real <= D elements: the missing elements of a row and the missing rows of the projection are
+  // zeros (they add nothing to a dot product)
+  for (int i = threadIdx.x; i < D * r; i += blockDim.x) lds_p[i] = i < d_real * r ? pbase[i] : (T)0.f;
   __syncthreads();
   // B operands: P and |P| for every part: slot j, group kg holds P[part*32 + 8*kg + e][j]; slots >= r are zero
   vec8 pf[PARTS], pa[PARTS];
@@ -161,7 +102,7 @@ __global__ __launch_bounds__(256) void lsh_hash_mfma_kernel(const HashTensors te
     for (int u = 0; u < HASH_UNROLL; ++u) {
       const int64_t row = wave_row0 + (int64_t)(t0 + u) * ROWS + my_row;
       vec8 z = {};
-      if (row < n) z = *reinterpret_cast<const vec8*>(xbase + row * sn + my_part * 32 + 8 * kg);
+      if (row < n && my_part * 32 + 8 * kg < d_real) z = *reinterpret_cast<const vec8*>(xbase + row * sn + my_part * 32 + 8 * kg);
       xf[u] = z;
     }
 #pragma unroll
@@ -245,27 +186,11 @@ __global__ __launch_bounds__(256) void lsh_hash_mfma_kernel(const HashTensors te
 
 template <typename T, int D, bool OUT8>
 int launch_hash_mfma(const HashTensors& ten, int64_t seqs, const void* proj, int64_t n, int64_t r, int64_t psb, int64_t psh,
-                     hipStream_t stream) {
+                     int64_t d_real, hipStream_t stream) {
   const int64_t rows_per_block = 4 * HASH_TILES_PER_WAVE * (16 / (D / 32));
   dim3 grid((unsigned)((n + rows_per_block - 1) / rows_per_block), (unsigned)seqs);
-  hipLaunchKernelGGL((lsh_hash_mfma_kernel<T, D, OUT8>), grid, dim3(256), 0, stream, ten, (const T*)proj, n, (int)r, psb, psh);
-  return ha_launch_status("ha_lsh_hash");
-}
-
-template <typename T>
-int launch_hash(const void* x, const void* proj, int32_t* buckets, int64_t batch, int64_t heads,
-                int64_t n, int64_t d, int64_t r, int64_t sb, int64_t sh, int64_t sn, int64_t psb,
-                int64_t psh, hipStream_t stream) {
-  const int threads = d <= 64 ? 256 : (d <= 128 ? 128 : 64);
-  const int rmax = r <= 8 ? 8 : 16;
-  const size_t lds = (size_t)d * rmax * 8 + (size_t)threads * d * 2;
-  dim3 grid((unsigned)((n + threads - 1) / threads), (unsigned)(batch * heads));
-  if (rmax == 8)
-    hipLaunchKernelGGL((lsh_hash_kernel<T, 8>), grid, dim3(threads), lds, stream, (const T*)x,
-                       (const T*)proj, buckets, (int)heads, n, (int)d, (int)r, sb, sh, sn, psb, psh);
-  else
-    hipLaunchKernelGGL((lsh_hash_kernel<T, 16>), grid, dim3(threads), lds, stream, (const T*)x,
-                       (const T*)proj, buckets, (int)heads, n, (int)d, (int)r, sb, sh, sn, psb, psh);
+  hipLaunchKernelGGL((lsh_hash_mfma_kernel<T, D, OUT8>), grid, dim3(256), 0, stream, ten, (const T*)proj, n, (int)r, psb, psh,
+                     (int)d_real);
   return ha_launch_status("ha_lsh_hash");
 }
 
@@ -290,19 +215,16 @@ extern "C" int ha_lsh_hash(const void* x, const void* proj, int32_t* buckets, in
   ten.sb[0] = x_stride_b; ten.sh[0] = x_stride_h; ten.sn[0] = x_stride_n;
   ten.heads[0] = ten.heads[1] = (int)heads;
   ten.seqs0 = (int)(batch * heads);
+  // built for rows of 32, 64, 128 and 256 elements; a shorter row runs in the next width
 #define HA_HASH_MFMA(DD)                                                                                              \
-  if (d == DD) {                                                                                                      \
+  if (d <= DD) {                                                                                                      \
     if (dtype == HA_F16)                                                                                              \
-      return launch_hash_mfma<f16_t, DD, false>(ten, batch * heads, proj, n, r, proj_stride_b, proj_stride_h, s);     \
-    return launch_hash_mfma<bf16_t, DD, false>(ten, batch * heads, proj, n, r, proj_stride_b, proj_stride_h, s);      \
+      return launch_hash_mfma<f16_t, DD, false>(ten, batch * heads, proj, n, r, proj_stride_b, proj_stride_h, d, s);  \
+    return launch_hash_mfma<bf16_t, DD, false>(ten, batch * heads, proj, n, r, proj_stride_b, proj_stride_h, d, s);   \
   }
   HA_HASH_MFMA(32) HA_HASH_MFMA(64) HA_HASH_MFMA(128) HA_HASH_MFMA(256)
 #undef HA_HASH_MFMA
-  if (dtype == HA_F16)
-    return launch_hash<f16_t>(x, proj, buckets, batch, heads, n, d, r, x_stride_b, x_stride_h, x_stride_n,
-                              proj_stride_b, proj_stride_h, s);
-  return launch_hash<bf16_t>(x, proj, buckets, batch, heads, n, d, r, x_stride_b, x_stride_h, x_stride_n,
-                             proj_stride_b, proj_stride_h, s);
+  return ha_fail(HA_ERR_HEADDIM, "ha_lsh_hash: d must be a multiple of 8 in [8, 256]");
 }
 
 // Bucket ids of the queries and keys of one forward pass as one byte each (r <= 8 projections, one shared
@@ -319,17 +241,12 @@ int ha_hash_pair_u8(const void* q, const void* k, const void* proj, uint8_t* ids
   ten.heads[0] = (int)heads; ten.heads[1] = (int)kv_heads;
   ten.seqs0 = (int)(batch * heads);
   const int64_t seqs = batch * (heads + kv_heads);
-  if (d == 32) {
-    if (dtype == HA_F16) return launch_hash_mfma<f16_t, 32, true>(ten, seqs, proj, n, r, 0, 0, stream);
-    return launch_hash_mfma<bf16_t, 32, true>(ten, seqs, proj, n, r, 0, 0, stream);
+#define HA_HASH_PAIR(DD)                                                                                  \
+  if (d <= DD) {                                                                                          \
+    if (dtype == HA_F16) return launch_hash_mfma<f16_t, DD, true>(ten, seqs, proj, n, r, 0, 0, d, stream); \
+    return launch_hash_mfma<bf16_t, DD, true>(ten, seqs, proj, n, r, 0, 0, d, stream);                    \
   }
-  if (d == 64) {
-    if (dtype == HA_F16) return launch_hash_mfma<f16_t, 64, true>(ten, seqs, proj, n, r, 0, 0, stream);
-    return launch_hash_mfma<bf16_t, 64, true>(ten, seqs, proj, n, r, 0, 0, stream);
-  }
-  if (d == 128) {
-    if (dtype == HA_F16) return launch_hash_mfma<f16_t, 128, true>(ten, seqs, proj, n, r, 0, 0, stream);
-    return launch_hash_mfma<bf16_t, 128, true>(ten, seqs, proj, n, r, 0, 0, stream);
-  }
+  HA_HASH_PAIR(32) HA_HASH_PAIR(64) HA_HASH_PAIR(128)
+#undef HA_HASH_PAIR
   return ha_fail(HA_ERR_UNSUPPORTED, "ha_forward: paired hash not built for head dim %lld", (long long)d);
 }

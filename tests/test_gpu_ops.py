@@ -33,7 +33,9 @@ def ha():
 # ------------------------------------------------------------------------------------- hash
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("b,h,n,d,r", [(1, 2, 2048, 64, 8), (2, 3, 1000, 128, 8), (1, 1, 777, 64, 5),
-                                       (1, 2, 513, 32, 12), (1, 1, 300, 256, 16)])
+                                       (1, 2, 513, 32, 12), (1, 1, 300, 256, 16),
+                                       # rows shorter than the width the kernel is built for
+                                       (1, 2, 700, 96, 8), (2, 1, 300, 40, 7), (1, 1, 515, 8, 3), (1, 1, 257, 200, 9)])
 def test_hash_bit_exact(ha, dtype, b, h, n, d, r):
     x = _randn((b, h, n, d), 1, dtype)
     proj = _randn((1, 1, d, r), 2, dtype)
