@@ -346,7 +346,7 @@ def main():
     proj2 = m.lsh.proj_dir.reshape(1, 1, d, 8)
     ms = time_events(lambda: ops.lsh_hash(q, proj2), reps, torch)
     hash_bytes = rows_q * (d * 2 + 4)
-    kernels["lsh_hash(q)"] = {"ms": round(ms, 4), "bound": "hbm", "achieved_GBs": round(hash_bytes / ms / 1e6, 1),
+    kernels["lsh_hash operator (q alone, int32 ids)"] = {"ms": round(ms, 4), "bound": "hbm", "achieved_GBs": round(hash_bytes / ms / 1e6, 1),
                               "frac": round(hash_bytes / ms / 1e6 / HBM_PEAK_GBS, 4), "bytes": hash_bytes}
     bq = ops.lsh_hash(q, proj2)
     bk = ops.lsh_hash(k, proj2)
@@ -428,7 +428,7 @@ def main():
                 "launch_ms_by_level": [round(x, 4) for x in blk_ms]}
     sort_elems = sum((rows_q // 2 + rows_k // 2) if w["causal"] else (rows_q + rows_k) for _ in halves)
     sort_total = sum(sort_ms)
-    kernels["bucket_argsort(one launch per level and side)"] = {"ms": round(sort_total, 4), "bound": "hbm", "bytes": sort_elems * 8,
+    kernels["bucket_argsort operator (one call per level and side; the forward ranks once instead)"] = {"ms": round(sort_total, 4), "bound": "hbm", "bytes": sort_elems * 8,
                                              "achieved_GBs": round(sort_elems * 8 / sort_total / 1e6, 1),
                                              "frac": round(sort_elems * 8 / sort_total / 1e6 / HBM_PEAK_GBS, 4)}
     # the first stage of the one-call forward: bucket ids of q and k in one launch, one ranking of the rows,
@@ -436,7 +436,7 @@ def main():
     ms = time_events(lambda: ops.forward_sort(q, k, proj2, causal=w["causal"], lsh_num_projs=8,
                                               min_seq_len=w["min_seq_len"]), reps, torch)
     stage_bytes = (rows_q + rows_k) * d * 2 + sort_elems * 4
-    kernels["ha_forward_sort (hash q+k, rank, place: all levels)"] = {
+    kernels["first stage of the forward: hash q+k in one launch, rank once, place all levels (ha_forward_sort)"] = {
         "ms": round(ms, 4), "bound": "hbm", "bytes": stage_bytes, "achieved_GBs": round(stage_bytes / ms / 1e6, 1),
         "frac": round(stage_bytes / ms / 1e6 / HBM_PEAK_GBS, 4)}
     if leaf is not None:

@@ -25,6 +25,15 @@ struct BlockRef {
   int job, seg, chunk;
 };
 
+// Workgroups go to the 8 XCDs round-robin by their number, and each XCD has its own L2.  Re-numbered so that
+// an XCD works through consecutive chunks (units): the rows of a bucket from neighbouring chunks of a segment
+// are neighbours in the output, and their short runs then meet in one L2 line before it is written back.
+__device__ __forceinline__ int xcd_contiguous_block() {
+  const int total = (int)gridDim.x, lin = (int)blockIdx.x;
+  const int xq = total / 8, xr = total % 8, xcd = lin % 8;
+  return xcd * xq + (xcd < xr ? xcd : xr) + lin / 8;
+}
+
 __device__ __forceinline__ BlockRef locate_block(const ha_sort_jobs& jobs, int block, bool per_segment) {
   int j = 0;
   while (j + 1 < jobs.num_jobs &&
@@ -144,7 +153,7 @@ __global__ __launch_bounds__(SORT_THREADS) void sort_scatter_kernel(ha_sort_jobs
   __shared__ uint32_t wave_totals[SORT_WAVES];
   __shared__ int32_t to_global[256];            // global slot minus chunk-local slot, per digit
   __shared__ uint32_t staged[HA_SORT_CHUNK];    // (digit << 24) | row, in chunk-local sorted order
-  const BlockRef br = locate_block(jobs, blockIdx.x, false);
+  const BlockRef br = locate_block(jobs, xcd_contiguous_block(), false);
   const ha_sort_job& job = jobs.job[br.job];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
 #pragma unroll
@@ -295,23 +304,31 @@ __global__ __launch_bounds__(SORT_THREADS) void rank_units_kernel(RankArgs a) {
 __global__ __launch_bounds__(SORT_THREADS) void place_units_kernel(ha_place_jobs jobs) {
   __shared__ uint32_t wave_totals[SORT_WAVES];
   __shared__ int32_t delta[256];   // segment slot minus unit slot, per bucket
+  const int block = xcd_contiguous_block();
   int j = 0;
-  while (j + 1 < jobs.num_jobs && (int)blockIdx.x >= jobs.job[j + 1].first_block) ++j;
+  while (j + 1 < jobs.num_jobs && block >= jobs.job[j + 1].first_block) ++j;
   const ha_place_job& job = jobs.job[j];
   const ha_unit_grid& g = jobs.grid;
   const int tid = threadIdx.x;
-  const int local = (int)blockIdx.x - job.first_block;
+  const int local = block - job.first_block;
   const int seg = local / job.units_per_seg, u = local % job.units_per_seg;
   const int seq = seg / job.segs_per_seq, sis = seg % job.segs_per_seq;
   const int64_t first_row = job.seg_offset + (int64_t)sis * job.seg_stride;   // of the segment, in its sequence
   const int64_t first_unit = (int64_t)seq * g.units_per_seq + (first_row / g.granule) * g.units_per_granule;
   const uint32_t* h = job.hist + first_unit * 256 + tid;
+  // eight independent loads in flight at a time: one after the other, a segment of 32 units would cost the
+  // workgroup 32 memory round trips before it moves a single row
   uint32_t tot = 0, before = 0, mine = 0;
-  for (int k = 0; k < job.units_per_seg; ++k) {
-    const uint32_t c = h[(int64_t)k * 256];
-    before += k < u ? c : 0u;
-    mine = k == u ? c : mine;
-    tot += c;
+  for (int k0 = 0; k0 < job.units_per_seg; k0 += 8) {
+    uint32_t c[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) c[i] = k0 + i < job.units_per_seg ? h[(int64_t)(k0 + i) * 256] : 0u;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      before += k0 + i < u ? c[i] : 0u;
+      mine = k0 + i == u ? c[i] : mine;
+      tot += c[i];
+    }
   }
   const uint32_t seg_first = block_exclusive_scan(tot, wave_totals);
   const uint32_t unit_first = block_exclusive_scan(mine, wave_totals);
@@ -322,9 +339,15 @@ __global__ __launch_bounds__(SORT_THREADS) void place_units_kernel(ha_place_jobs
   const int len = (int)min((int64_t)g.unit, g.granule - (int64_t)w * g.unit);
   const uint32_t* src = job.sorted + (int64_t)seq * g.n + first_row + row0;
   int32_t* out = job.out + (int64_t)seg * job.seg_len;
-  for (int pos = tid; pos < len; pos += SORT_THREADS) {
-    const uint32_t v = src[pos];
-    out[pos + delta[v >> 16]] = (int32_t)row0 + (int32_t)(v & 0xFFFFu);
+  for (int pos0 = tid; pos0 < len; pos0 += 8 * SORT_THREADS) {
+    uint32_t v[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = src[min(pos0 + i * SORT_THREADS, len - 1)];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int pos = pos0 + i * SORT_THREADS;
+      if (pos < len) out[pos + delta[v[i] >> 16]] = (int32_t)row0 + (int32_t)(v[i] & 0xFFFFu);
+    }
   }
 }
 
