@@ -260,7 +260,8 @@ class HyperAttention(torch.nn.Module):
             if causal is not False and n_key <= self.min_seq_len:
                 # the reference returns the exact kernel's padded 3-d lse for a top-level leaf
                 n_rounded = -(-n_key // 128) * 128
-                lse = torch.nn.functional.pad(lse, (0, n_rounded - n_key))
+                if n_rounded != n_key:
+                    lse = torch.nn.functional.pad(lse, (0, n_rounded - n_key))
             else:
                 lse = lse.unsqueeze(-1)
         elif (causal is not False and n_key > self.min_seq_len and not self.residual_estimator

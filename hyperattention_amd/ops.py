@@ -446,11 +446,12 @@ def forward_plan_supported(n: int, min_seq_len: int, causal: bool, lsh_num_projs
 
 
 def _forward_args(q, k, v, out, lse, proj, *, scale, causal, lsh_num_projs, block_size, sample_size, min_seq_len,
-                  smooth_block, sampled_idx=None, workspace=None):
+                  smooth_block, sampled_idx=None, workspace=None, stream=None):
     """ForwardArgs for (b,h,n,d) q and (b,h_kv,n,d) k, v with its workspace attached; the second result keeps
     the tensors alive that the struct only points to (the workspace last).  `workspace`: a dict the caller
-    owns; the workspace tensor of the current (device, stream) is kept there and reused while it is large
-    enough, so that a caller that runs many forwards does not allocate one per call."""
+    owns; the workspace tensor of the current (device, stream) and the sizes the library asked for are kept
+    there and reused, so that a caller that runs many forwards neither allocates nor asks per call.
+    `stream`: the raw handle of the current stream, if the caller has it already."""
     assert q.is_cuda and k.is_cuda
     assert q.stride(-1) == 1 and k.stride(-1) == 1 and (v is None or v.stride(-1) == 1)
     assert q.dtype == k.dtype and (v is None or v.dtype == q.dtype), "All tensors must have the same type"
@@ -484,12 +485,19 @@ def _forward_args(q, k, v, out, lse, proj, *, scale, causal, lsh_num_projs, bloc
     a.k_stride_b, a.k_stride_h, a.k_stride_n = k.stride(0), k.stride(1), k.stride(2)
     if v is not None:
         a.v_stride_b, a.v_stride_h, a.v_stride_n = v.stride(0), v.stride(1), v.stride(2)
-    ws_bytes = _lib.lib().ha_forward_workspace_bytes(ctypes.byref(a))
-    if ws_bytes < 0:
-        _lib.check(int(ws_bytes))
+    shape_key = (b, h, hk, n, d, a.dv, lsh_num_projs, min_seq_len, a.causal)
+    ws_bytes = workspace.get(shape_key) if workspace is not None else None
+    if ws_bytes is None:
+        ws_bytes = _lib.lib().ha_forward_workspace_bytes(ctypes.byref(a))
+        if ws_bytes < 0:
+            _lib.check(int(ws_bytes))
+        if workspace is not None:
+            workspace[shape_key] = ws_bytes
     ws = None
     if workspace is not None:
-        slot = (q.device.index, torch.cuda.current_stream(q.device).cuda_stream)
+        if stream is None:
+            stream = torch.cuda.current_stream(q.device).cuda_stream
+        slot = (q.device.index, stream)
         ws = workspace.get(slot)
     if ws is None or ws.numel() < int(ws_bytes):
         ws = torch.empty(int(ws_bytes), device=q.device, dtype=torch.uint8)
@@ -509,11 +517,15 @@ def hyper_forward(q, k, v, proj, *, scale, causal, lsh_num_projs, block_size, sa
     b, h, n, d = q.shape
     out = torch.empty((b, h, n, v.shape[-1]), device=q.device, dtype=q.dtype)
     lse = torch.empty((b, h, n), device=q.device, dtype=torch.float32)
+    stream = torch.cuda.current_stream(q.device).cuda_stream
     a, keep = _forward_args(q, k, v, out, lse, proj, scale=scale, causal=causal, lsh_num_projs=lsh_num_projs,
                             block_size=block_size, sample_size=sample_size, min_seq_len=min_seq_len,
-                            smooth_block=smooth_block, sampled_idx=sampled_idx, workspace=workspace)
-    with torch.cuda.device(q.device):
-        _lib.check(_lib.lib().ha_forward(ctypes.byref(a), _stream(q)))
+                            smooth_block=smooth_block, sampled_idx=sampled_idx, workspace=workspace, stream=stream)
+    if q.device.index == torch.cuda.current_device():
+        _lib.check(_lib.lib().ha_forward(ctypes.byref(a), ctypes.c_void_p(stream)))
+    else:
+        with torch.cuda.device(q.device):
+            _lib.check(_lib.lib().ha_forward(ctypes.byref(a), ctypes.c_void_p(stream)))
     return out, lse
 
 
