@@ -146,9 +146,15 @@ def test_forward_plan_and_workspace(lib):
     f.lsh_num_projs, f.block_size, f.sample_size, f.min_seq_len = 8, 256, 256, 2048
     f.causal, f.scale, f.dtype = 1, 0.125, 0
     ws = lib.ha_forward_workspace_bytes(ctypes.byref(f))
-    # buckets (2 x 4 Mi x 4 B) + six levels of (q_idx + k_idx) (2 x 2 Mi x 4 B each) + histograms
-    assert ws >= 2 * 4194304 * 4 + 6 * 2 * 2097152 * 4
-    assert ws < 200 << 20
+    # byte-sized bucket ids of q and k (2 x 4 Mi) + per-unit orders (2 x 4 Mi x 4 B) + per-unit bucket counts
+    # (2 x 32 sequences x 64 units of 2048 rows x 256 x 4 B) + six levels of (q_idx + k_idx) (2 x 2 Mi x 4 B each)
+    assert ws == 2 * 4194304 + 2 * 4194304 * 4 + 2 * 32 * 64 * 1024 + 6 * 2 * 2097152 * 4
+    f.lsh_num_projs = 12   # 4096 buckets: int32 ids, a sort per level with two digit passes and their orders in between
+    ws12 = lib.ha_forward_workspace_bytes(ctypes.byref(f))
+    assert ws12 > 2 * 4194304 * 4 + 3 * 6 * 2 * 2097152 * 4 and ws12 < 400 << 20
+    f.lsh_num_projs = 17
+    assert lib.ha_forward_workspace_bytes(ctypes.byref(f)) > 0   # sized; the call itself rejects more than 16 projections
+    f.lsh_num_projs = 8
     f.n = 4095  # an odd length above min_seq_len needs the padded copy: not a shape of the one-call entry point
     assert lib.ha_forward_workspace_bytes(ctypes.byref(f)) == -5
     f.n = 131072 + 2  # the first halves (65537) are hashed and must be a multiple of 128
@@ -162,6 +168,37 @@ def test_forward_plan_and_workspace(lib):
     f.n, f.min_seq_len = 1000, 2048  # exact path: no workspace needed beyond the minimum
     assert lib.ha_forward_workspace_bytes(ctypes.byref(f)) == 256
     assert lib.ha_forward(ctypes.byref(f), None) == -1  # null tensors
+    # the first stage alone
+    offs = (ctypes.c_int64 * 48)()
+    levels = ctypes.c_int(0)
+    assert lib.ha_forward_sort(None, offs, offs, ctypes.byref(levels), None) == -1
+    assert lib.ha_forward_sort(ctypes.byref(f), offs, offs, ctypes.byref(levels), None) == -1  # null q, k
+    f.q = f.k = 256
+    f.d = 4
+    assert lib.ha_forward_sort(ctypes.byref(f), offs, offs, ctypes.byref(levels), None) == -5
+    f.d, f.n, f.min_seq_len, f.causal = 64, 1000, 2048, 1   # nothing hashed: no launch, no workspace needed
+    assert lib.ha_forward_sort(ctypes.byref(f), offs, offs, ctypes.byref(levels), None) == 0 and levels.value == 0
+    f.n, f.min_seq_len = 8192, 2048   # two hashed levels, but no workspace given
+    assert lib.ha_forward_sort(ctypes.byref(f), offs, offs, ctypes.byref(levels), None) == -1  # null projection
+    f.proj = 256
+    assert lib.ha_forward_sort(ctypes.byref(f), offs, offs, ctypes.byref(levels), None) == -6
+    assert levels.value == 2 and offs[0] > 0 and offs[1] > offs[0]
+
+
+def test_merge_levels_argument_errors(lib):
+    vp = ctypes.c_void_p
+    one = vp(256)
+    two = vp(512)
+    arr = (vp * 1)(256)
+    call = lambda levels, n, d, out=two, lse_out=two, dtype=0, o_un=arr: lib.ha_lse_merge_levels(
+        one, one, o_un, arr, arr, one, out, lse_out, levels, 4, n, d, dtype, None)
+    assert lib.ha_lse_merge_levels(None, None, None, None, None, None, None, None, 0, 1, 128, 64, 0, None) == -1
+    assert call(1, 256, 64, dtype=3) == -2
+    assert call(25, 1 << 25, 64) == -5            # more levels than the kernel is built for
+    assert call(1, 256, 60) == -3                 # d % 8
+    assert call(3, 1004, 64) == -3                # n not divisible by 2^levels
+    assert call(1, 256, 64, out=one) == -5        # in place
+    assert call(1, 256, 64, o_un=(vp * 1)(None)) == -1
 
 
 def test_backward_argument_errors_before_any_launch(lib):
