@@ -389,6 +389,21 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
   const uint32_t blk_idx_rb = (uint32_t)p.ki_sn << idx_shift;  // bytes between entries of the key order
   const unsigned char* const smp_idx =
       !PLAIN && p.sampled_idx ? (const unsigned char*)p.sampled_idx + (sidx_off << idx_shift) : nullptr;
+  // Smooth windows of neighbouring workgroups overlap (a workgroup's window is 640 keys wide and the next
+  // one starts 256 keys later).  Every workgroup therefore walks its window in the same phase of the global
+  // chunk number: it starts with the chunk whose number is a multiple of the window length and wraps
+  // around, so that workgroups running side by side read a chunk they share in the same iteration and one
+  // of them finds it in L2.  (The order in which a row's keys are summed changes, nothing else.)
+  int blk_rot = 0;
+  if (GATHER && !PLAIN && p.smooth && n_blk_chunks > 0) {
+    const int phase = uni_start % n_blk_chunks;
+    blk_rot = phase ? n_blk_chunks - phase : 0;
+  }
+  // window position (chunk, from the window's first) of block-part iteration ci
+  auto blk_pos = [&](int ci) -> int {
+    const int c = ci + blk_rot;
+    return c >= n_blk_chunks ? c - n_blk_chunks : c;
+  };
   auto fetch_rows = [&](int ci, int kk0, RowSource& rs) {
     // Consecutive rows (or row 0 for every lane) are written first and without a branch; an index run
     // then overwrites them by loads.  A vector write behind a branch that follows a load of the same
@@ -400,7 +415,7 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
     for (int j = 0; j < LPW; ++j) rs.rows[j] = (int)__umul24((uint32_t)(j * ROWS_PER_LOAD + my_lr), per_lane) + first;
     if (in_range) {
       if (ci < n_blk_chunks) {
-        int u = uni_start + ci;
+        int u = uni_start + (PLAIN ? ci : blk_pos(ci));
         if (!PLAIN) {  // smooth windows wrap around the key sequence
           u -= u >= nk_chunks ? nk_chunks : 0;
           u -= u >= nk_chunks ? nk_chunks : 0;
@@ -536,7 +551,11 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
   // ---- masks (wave-uniform decision per chunk) -------------------------------------------------
   auto chunk_masked = [&](int ci) -> bool {
     if (PLAIN) return false;
-    if (GATHER) return ci < n_blk_chunks && !(uni_start + ci >= my_lo && uni_start + ci < my_hi);
+    if (GATHER) {
+      if (ci >= n_blk_chunks) return false;
+      const int u = uni_start + blk_pos(ci);
+      return !(u >= my_lo && u < my_hi);
+    }
     const int k_first = ci * KC;
     return (CAUSAL && k_first + KC - 1 > wave_q_first) || (k_first + KC > p.n_k);
   };
