@@ -325,6 +325,45 @@ def test_forward_sort_is_the_stable_sort_of_every_level(ha, b, h, hk, n, d, msl,
         assert (n >> len(q_idx)) <= msl < (n >> (len(q_idx) - 1))
 
 
+def test_forward_sort_random_shapes(ha):
+    """Seeded random shapes (leaf lengths that are not powers of two, ragged units, skewed buckets from
+    clustered rows, 1 to 16 projections): every level's orders equal the stable sort of the library's own ids."""
+    from hyperattention_amd import ops
+    rng = np.random.default_rng(7)
+    for case in range(10):
+        levels = int(rng.integers(0, 4))
+        leaf = 128 * int(rng.integers(1, 41))            # 128 .. 5120 rows
+        n = leaf << levels
+        causal = bool(rng.integers(0, 2)) or levels > 0
+        r = int(rng.integers(1, 17))
+        hk = int(rng.integers(1, 3))
+        h = hk * int(rng.integers(1, 3))
+        d = int(rng.choice([32, 64, 96, 128]))
+        msl = leaf if causal else int(rng.integers(1, n + 1))
+        q = _randn((1, h, n, d), 400 + case, torch.float16).cuda()
+        k = _randn((1, hk, n, d), 500 + case, torch.float16).cuda()
+        if case % 2:   # clustered rows: a few directions plus noise, so that buckets are very uneven
+            centres = _randn((1, 1, 4, d), 600 + case, torch.float16).cuda()
+            q = (centres[:, :, torch.arange(n, device="cuda") % 4] + 0.05 * q).contiguous()
+        proj = _randn((1, 1, d, r), 700 + case, torch.float16).cuda()
+        q_idx, k_idx = ops.forward_sort(q, k, proj, causal=causal, lsh_num_projs=r, min_seq_len=msl)
+        bq, bk = ops.lsh_hash(q, proj), ops.lsh_hash(k, proj)
+        what = f"case {case}: n {n} leaf {leaf} levels {levels} causal {causal} r {r} heads {h}/{hk} d {d}"
+        assert len(q_idx) == (levels if causal else 1), what
+        for level in range(len(q_idx)):
+            half = (n >> (level + 1)) if causal else n
+            if msl > half:
+                assert q_idx[level] is None, what
+                continue
+            if causal:
+                want_q = bq.view(1, h << level, 2, half)[:, :, 1].sort(dim=-1, stable=True).indices
+                want_k = bk.view(1, hk << level, 2, half)[:, :, 0].sort(dim=-1, stable=True).indices
+            else:
+                want_q, want_k = bq.sort(dim=-1, stable=True).indices, bk.sort(dim=-1, stable=True).indices
+            assert torch.equal(q_idx[level].long(), want_q) and torch.equal(k_idx[level].long(), want_k), \
+                f"{what}, level {level}"
+
+
 def _check_sort_properties(ha, buckets):
     """the permutation of every head is a permutation, sorts its keys, and keeps equal keys in row order"""
     b, h, n = buckets.shape
