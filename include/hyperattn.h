@@ -274,7 +274,11 @@ int ha_lse_merge_levels(const void* o_leaf, const float* lse_leaf, const void* c
  * replaces: HyperAttention.forward / forward_no_causal_mask (hyper_attention.py:25-132) for the
  * shapes where every recursion level has an even length (n = leaf_len * 2^levels); other shapes
  * are composed by the caller from the operators above.
- * proj: (d, r) in dtype.  sampled_idx: int32 key rows local to each un-masked call (NULL = first
+ * proj: (d, r) in dtype, r = lsh_num_projs <= 16 (the reference takes any r, padded to 16 slots,
+ * src/angular_lsh_triton.py:116-144).  d, dv: multiples of 8 up to 128.  Workspace:
+ * ha_forward_workspace_bytes(args) bytes, 256-byte aligned; it holds the bucket ids, the per-unit orders
+ * and counts of the one ranking (r <= 8; above, a sort per level with its digit passes) and the int32
+ * orders of every hashed level.  sampled_idx: int32 key rows local to each un-masked call (NULL = first
  * sample_size rows), shared by all heads and levels; PRECONDITION as for ha_block_attn_fwd, with n_k the
  * key length of the shortest hashed level (n / 2^levels halvings down to the last length >= min_seq_len).  out (batch,heads,n,dv) dtype, lse
  * (batch,heads,n) fp32.  kv_heads divides heads (grouped-query: q head h reads kv head
