@@ -252,6 +252,46 @@ def test_module_backward(ha, causal, n, min_seq_len, block, sample, smooth, kv_h
         _check(got, want, f"module {name}", dtype)
 
 
+def test_module_backward_random_configurations(ha):
+    """Seeded random constructor arguments and shapes for the module under autograd (causal recursion on
+    segments with grouped heads, smoothed blocks, odd tile counts per block, no samples, more than 8
+    projections): gradients against torch autograd on the oracle, the reference's constant-log-sum-exp convention."""
+    rng = np.random.default_rng(21)
+    for case in range(6):
+        d = int(rng.choice([64, 128]))
+        dtype = [torch.float16, torch.bfloat16][int(rng.integers(0, 2))]
+        causal = case % 3 != 2
+        block = 128 * int(rng.integers(1, 4))
+        sample = 128 * int(rng.integers(0, 3))
+        smooth = bool(rng.integers(0, 2))
+        r = int(rng.integers(2, 13))
+        hk = int(rng.integers(1, 3))
+        h = hk * int(rng.integers(1, 3))
+        levels = int(rng.integers(1, 3)) if causal else 0
+        leaf = 128 * int(rng.integers(2, 4))
+        n = (leaf << levels) if causal else 128 * int(rng.integers(4, 9))
+        msl = leaf if causal else 128
+        sample = min(sample, leaf)
+        what = (f"case {case}: d {d} {dtype} causal {causal} n {n} min_seq_len {msl} block {block} sample {sample} "
+                f"smooth {smooth} r {r} heads {h}/{hk}")
+        q = _randn((1, h, n, d), 1200 + case, dtype)
+        k, v = (_randn((1, hk, n, d), s + case, dtype) for s in (1300, 1400))
+        do = _randn((1, h, n, d), 1500 + case, dtype)
+        m = ha.HyperAttention(input_dim=d, lsh_num_projs=r, block_size=block, sample_size=sample, min_seq_len=msl,
+                              smooth_block=smooth, rng=_gen(1600 + case)).to(device="cuda", dtype=dtype)
+        proj = m.lsh.proj_dir[0, 0].cpu()
+        expand = lambda x: x.repeat_interleave(h // hk, dim=1)
+        ref = _oracle_grads(lambda a, b_, c: O.hyper_forward(a, expand(b_), expand(c), proj, causal=causal,
+                                                             lsh_num_projs=r, block_size=block, sample_size=sample,
+                                                             min_seq_len=msl, smooth_block=smooth, detach_lse=True),
+                            q, k, v, do)
+        qg, kg, vg = (x.cuda().requires_grad_() for x in (q, k, v))
+        m(qg, kg, vg, causal=causal).backward(do.cuda())
+        torch.cuda.synchronize()
+        for got, want, name in zip((qg.grad, kg.grad, vg.grad), ref, ("dq", "dk", "dv")):
+            _check(got, want, f"{what}: {name}", dtype)
+
+
 def test_module_backward_twice_and_retain_graph(ha):
     # the backward neither consumes nor disturbs what it saved: two passes over one graph agree
     dtype, b, h, n, d = torch.bfloat16, 1, 2, 1024, 64

@@ -217,6 +217,41 @@ def test_module_residual_estimator(ha, causal):
         m(q.cuda().requires_grad_(), k.cuda(), v.cuda(), causal=causal)
 
 
+def test_random_configurations_against_the_oracle(ha):
+    """Seeded random constructor arguments and shapes (block sizes with an odd number of 128-key tiles, no
+    samples, smoothed blocks, grouped heads, both head dims and types, 1..10 projections, with and without the
+    causal recursion): the module against the oracle, output and log-sum-exp."""
+    rng = np.random.default_rng(11)
+    for case in range(12):
+        d = int(rng.choice([64, 128]))
+        dtype = [torch.float16, torch.bfloat16][int(rng.integers(0, 2))]
+        causal = bool(rng.integers(0, 2))
+        block = 128 * int(rng.integers(1, 5))
+        sample = 128 * int(rng.integers(0, 3))
+        smooth = bool(rng.integers(0, 2))
+        r = int(rng.integers(1, 11))
+        hk = int(rng.integers(1, 3))
+        h = hk * int(rng.integers(1, 3))
+        levels = int(rng.integers(1, 3)) if causal else 0
+        leaf = 128 * int(rng.integers(2, 6))
+        n = (leaf << levels) if causal else 128 * int(rng.integers(4, 17))
+        msl = leaf if causal else int(rng.integers(1, n + 1))
+        if causal:
+            sample = min(sample, leaf)      # the default sample list must fit the shortest hashed level
+        what = (f"case {case}: d {d} {dtype} causal {causal} n {n} min_seq_len {msl} block {block} sample {sample} "
+                f"smooth {smooth} r {r} heads {h}/{hk}")
+        q = _randn((1, h, n, d), 800 + case, dtype)
+        k, v = (_randn((1, hk, n, d), s + case, dtype) for s in (900, 1000))
+        m, proj = _module(ha, d, dtype, 1100 + case, lsh_num_projs=r, block_size=block, sample_size=sample,
+                          min_seq_len=msl, smooth_block=smooth)
+        attn, lse = m(q.cuda(), k.cuda(), v.cuda(), causal=causal, return_lse=True)
+        expand = lambda x: x.repeat_interleave(h // hk, dim=1)
+        args = (q, expand(k), expand(v), proj, m, causal)
+        ro, rl = _oracle(*args)
+        assert_close(attn, ro, what + ": attn", dtype, _reference_arithmetic(dtype, *args))
+        assert_close(lse, rl, what + ": lse")
+
+
 def test_module_argument_errors(ha):
     m, _ = _module(ha, 64, torch.float16, 160)
     q = torch.zeros((1, 1, 256, 64), dtype=torch.float16, device="cuda")
