@@ -271,9 +271,10 @@ class HyperAttention(torch.nn.Module):
             attn, lse = _CausalRecursionFunc.apply(self, scale, query.contiguous(), key.contiguous(), value.contiguous(),
                                                    proj)
         else:
-            if key.shape[1] != query.shape[1]:
-                # grouped-query inputs on the operator-by-operator path: it follows the reference, which
-                # wants as many k/v heads as q heads (hyper_attention.py:43,67-68)
+            if key.shape[1] != query.shape[1] and causal is not False:
+                # grouped-query inputs on the operator-by-operator recursion: it follows the reference, which
+                # folds halves into heads (hyper_attention.py:67-68), and that needs as many k/v heads as q
+                # heads; a single un-masked call takes the groups as they are
                 group = query.shape[1] // key.shape[1]
                 key, value = key.repeat_interleave(group, dim=1), value.repeat_interleave(group, dim=1)
             query, key, value = query.contiguous(), key.contiguous(), value.contiguous()

@@ -187,13 +187,14 @@ def _block_attn_args(q, k, v, o, lse, q_sort_idx, k_sort_idx, block_size, sample
     if sampled_idx is not None:
         check_sampled_idx(sampled_idx, k.shape[sn])
         keep = sampled_idx.to(device=q.device, dtype=q_sort_idx.dtype).contiguous()
-        assert keep.shape in ((sample_size,), (nheads, sample_size), (batch, nheads, sample_size)), \
-            "sampled_idx must be (sample_size,), (nheads, sample_size) or (batch, nheads, sample_size)"
+        k_heads = k.shape[sh]
+        assert keep.shape in ((sample_size,), (k_heads, sample_size), (batch, k_heads, sample_size)), \
+            "sampled_idx must be (sample_size,), (nheads, sample_size) or (batch, nheads, sample_size) (k/v heads)"
         a.sampled_idx = keep.data_ptr()
         if keep.dim() >= 2:
             a.sampled_stride_h = sample_size
         if keep.dim() == 3:
-            a.sampled_stride_b = nheads * sample_size
+            a.sampled_stride_b = k_heads * sample_size
     a.block_size, a.sample_size = block_size, sample_size
     a.smooth_block, a.accumulate = int(bool(smooth_block)), int(bool(accumulate))
     return a, keep
@@ -261,8 +262,11 @@ def hyper_attn_func(q, k, v, q_sort_idx, k_sort_idx, block_size, sample_size=0, 
         return o[..., :d_v], lse
     batch, seqlen_q, nheads, d = q.shape
     _, seqlen_k, _, _ = k.shape
-    assert k.shape == (batch, seqlen_k, nheads, d)
-    assert v.shape[:3] == (batch, seqlen_k, nheads)
+    # (the reference wants as many k/v heads as q heads; fewer, dividing them, are grouped-query heads: q head
+    # h reads k/v head h // (nheads // k_heads), and k_sort_idx, per-head sample lists and dk, dv go by k/v heads)
+    k_heads = k.shape[2]
+    assert k.shape == (batch, seqlen_k, k_heads, d) and nheads % k_heads == 0
+    assert v.shape[:3] == (batch, seqlen_k, k_heads)
     assert q_sort_idx.shape == q.shape[:3]
     assert k_sort_idx.shape == k.shape[:3]
     assert d <= 128, "FlashAttention only support head dimensions up to 128"
@@ -307,8 +311,9 @@ def flash_attn_func(q, k, v, bias=None, causal=False, softmax_scale=None):
     q, k, v = [x if x.stride(-1) == 1 else x.contiguous() for x in [q, k, v]]
     batch, seqlen_q, nheads, d = q.shape
     _, seqlen_k, _, _ = k.shape
-    assert k.shape == (batch, seqlen_k, nheads, d)
-    assert v.shape == (batch, seqlen_k, nheads, d)
+    k_heads = k.shape[2]   # fewer than nheads, dividing them: grouped-query heads (not in the reference)
+    assert k.shape == (batch, seqlen_k, k_heads, d) and nheads % k_heads == 0
+    assert v.shape == (batch, seqlen_k, k_heads, d)
     assert d <= 128, "FlashAttention only support head dimensions up to 128"
     if _wants_grad(q, k, v) and d in KERNEL_HEAD_DIMS:
         return FlashAttnFunc.apply(q, k, v, bias, causal, softmax_scale)

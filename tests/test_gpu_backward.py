@@ -223,6 +223,7 @@ def test_backward_grouped_query_heads_through_the_c_abi(ha, kind):
     (True, 2048, 512, 256, 256, True, 2),     # smoothed blocks
     (True, 1024, 600, 128, 128, False, 2),    # the off-diagonal call is exact (min_seq_len > n/2)
     (True, 2048, 256, 128, 128, False, 1),    # three levels; two query heads on one key/value head
+    (False, 1024, 256, 128, 128, True, 1),    # one un-masked call with grouped heads taken as they are
 ])
 def test_module_backward(ha, causal, n, min_seq_len, block, sample, smooth, kv_heads):
     # the module under autograd: operators with their own backward, merges as tensor arithmetic;

@@ -360,6 +360,25 @@ def test_residual_estimator_option(ha, dtype, d, smooth, block, per_head):
                            qi.transpose(1, 2).cuda(), ki.transpose(1, 2).cuda(), block, samples, None, smooth, sample_bias=bias)
 
 
+@pytest.mark.parametrize("smooth", [False, True])
+def test_operators_take_grouped_query_heads(ha, smooth):
+    """Fewer k/v heads than q heads (not in the reference, which wants them equal): the same bits as with the
+    k/v heads, their sort order and their per-head sample lists repeated for every query head of a group."""
+    b, h, hk, n, d = 2, 4, 2, 1024, 64
+    q, _, _, qi, _ = _sorted_inputs(b, h, n, d, torch.float16, 95)
+    _, k, v, _, ki = _sorted_inputs(b, hk, n, d, torch.float16, 96)
+    sampled = torch.randint(0, n, (hk, 128), generator=_gen(97))
+    c = lambda t: t.cuda().transpose(1, 2)
+    rep = lambda t: t.repeat_interleave(h // hk, dim=1)
+    got, got_lse = ha.hyper_attn_func(c(q), c(k), c(v), c(qi), c(ki), 256, 128, None, smooth, sampled_idx=sampled.cuda())
+    want, want_lse = ha.hyper_attn_func(c(q), c(rep(k)), c(rep(v)), c(qi), c(rep(ki)), 256, 128, None, smooth,
+                                        sampled_idx=rep(sampled.view(1, hk, 128)).view(h, 128).cuda())
+    assert torch.equal(got, want) and torch.equal(got_lse, want_lse)
+    fo, fl = ha.flash_attn_func(c(q), c(k), c(v), None, True)
+    wo, wl = ha.flash_attn_func(c(q), c(rep(k)), c(rep(v)), None, True)
+    assert torch.equal(fo, wo) and torch.equal(fl, wl)
+
+
 def test_block_attention_value_dim_differs(ha):
     """unit_tests/test_hyper_attention.py:120-133: V narrower than Q and K gives the matching columns
     of the full-width result; the other way round (wider V) follows from the same definition."""
