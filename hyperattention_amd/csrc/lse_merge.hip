@@ -176,19 +176,26 @@ __global__ __launch_bounds__(256) void lse_merge_levels_kernel(const T* __restri
   const float x_leaf = x;
   vec8 r = *reinterpret_cast<const vec8*>(o_leaf + at);
   float c_of[MAXL], x_of[MAXL];
+  vec8 v_of[MAXL];
+  // every load first, so that they are all in flight before the chain of weights (each level's weight needs
+  // the log-sum-exp the deeper levels left) starts
 #pragma unroll
   for (int j = MAXL - 1; j >= 0; --j) {
     c_of[j] = 1.0f;
     x_of[j] = 0.0f;
     if (j < lv.levels && ((leaf_no >> (lv.levels - 1 - j)) & 1u)) {
-      const float x2 = lv.lse_un[j][row];
-      const float c = (float)(T)(1.0f / (1.0f + __expf(x2 - x)));
-      const vec8 v2 = *reinterpret_cast<const vec8*>((const T*)lv.o_un[j] + at);
+      x_of[j] = lv.lse_un[j][row];
+      v_of[j] = *reinterpret_cast<const vec8*>((const T*)lv.o_un[j] + at);
+    }
+  }
 #pragma unroll
-      for (int e = 0; e < 8; ++e) r[e] = (T)(c * (float)r[e] + (1.0f - c) * (float)v2[e]);
+  for (int j = MAXL - 1; j >= 0; --j) {
+    if (j < lv.levels && ((leaf_no >> (lv.levels - 1 - j)) & 1u)) {
+      const float c = (float)(T)(1.0f / (1.0f + __expf(x_of[j] - x)));
+#pragma unroll
+      for (int e = 0; e < 8; ++e) r[e] = (T)(c * (float)r[e] + (1.0f - c) * (float)v_of[j][e]);
       x = x - __logf(c + 1.1920929e-07f);
       c_of[j] = c;
-      x_of[j] = x2;
     }
   }
   *reinterpret_cast<vec8*>(out + at) = r;
