@@ -484,7 +484,7 @@ def main():
 
     backward = None
     if not args.no_backward:
-        def fwd_bwd_ms(fn, tensors, reps):
+        def fwd_bwd_ms(fn, tensors, reps, sustain=False):
             """(ms of the forward under autograd, ms of the backward), each the mean over reps calls"""
             leaves = [x.detach().clone().requires_grad_() for x in tensors]
             o = fn(*leaves)
@@ -493,12 +493,20 @@ def main():
             f = time_events(lambda: fn(*leaves), reps, torch)
             o = fn(*leaves)
             bw = time_events(lambda: o.backward(do, retain_graph=True), reps, torch)
-            return f, bw
+            power = None
+            if sustain:
+                # the backward alone for a second, with board power and shader clock (gradients accumulate into
+                # the leaves, as in the timed calls)
+                power = sustained(lambda: o.backward(do, retain_graph=True), 1.0, torch)
+            return f, bw, power
 
-        f_ms, b_ms = fwd_bwd_ms(lambda a, b_, c: m(a, b_, c, causal=w["causal"]), (q, k, v), 5)
+        f_ms, b_ms, b_power = fwd_bwd_ms(lambda a, b_, c: m(a, b_, c, causal=w["causal"]), (q, k, v), 5,
+                                         sustain=not args.no_sustained)
         backward = {"fwd_autograd_ms": round(f_ms, 3), "bwd_ms": round(b_ms, 3), "fwd_bwd_ms": round(f_ms + b_ms, 3)}
+        if b_power:
+            backward["sustained"] = b_power
         if not args.no_exact and hk == h:
-            ef, eb = fwd_bwd_ms(lambda a, b_, c: ops.flash_attn_func(a.transpose(1, 2), b_.transpose(1, 2), c.transpose(1, 2),
+            ef, eb, _ = fwd_bwd_ms(lambda a, b_, c: ops.flash_attn_func(a.transpose(1, 2), b_.transpose(1, 2), c.transpose(1, 2),
                                                                     None, w["causal"], scale)[0], (q, k, v), 2)
             backward["exact_fwd_bwd_ms"] = round(ef + eb, 3)
             backward["speedup_of_hyper"] = round((ef + eb) / (f_ms + b_ms), 2)
