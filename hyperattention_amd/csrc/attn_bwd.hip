@@ -321,11 +321,20 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 || PASS == HA_BWD_DQ_BLOCK ? 2
   int group_next = 0;           // the query head (within the group) those rows belong to
   int stat_row_next = 0;        // dK/dV passes: source row of streamed row 16 * wave + lane % 16 of the next tile
                                 // (every wave fetches the statistics of 16 rows: no wave has more to do)
+  bool stat_past_end_next = false;
   float stat_lse = 0.f, stat_delta = 0.f;
   auto fetch_rows = [&](int c) {
 #pragma unroll
     for (int j = 0; j < LPW; ++j) rows_next[j] = stream_row(c, (wave_s * LPW + j) * RPL + my_lr);
-    if (KEY_ST) stat_row_next = stream_row(c, wave_s * 16 + (lane & 15));
+    if (KEY_ST) {
+      stat_row_next = stream_row(c, wave_s * 16 + (lane & 15));
+      // sampled keys: a streamed query past the end of the workgroup's range gets L = +inf below, so that
+      // P = 2^(s - inf) = 0 and dS = 0 * finite = 0 with no mask in the chunk
+      if (PASS == HA_BWD_DKV_SAMPLED) {
+        const int cc = (c < nc ? c : nc - 1) - group_of(c) * nc_head;
+        stat_past_end_next = y_first + cc * YC + wave_s * 16 + (lane & 15) >= y_end;
+      }
+    }
     group_next = group_of(c);
   };
   auto load_tile = [&](int buf) {  // the tile whose rows are in rows_next
@@ -342,7 +351,7 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 || PASS == HA_BWD_DQ_BLOCK ? 2
     }
     if (KEY_ST) {
       const f32x2 sd = stats_head(group_next)[stat_row_next];
-      stat_lse = sd[0];
+      stat_lse = stat_past_end_next ? __builtin_inff() : sd[0];
       stat_delta = sd[1];
     }
   };
@@ -361,7 +370,6 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 || PASS == HA_BWD_DQ_BLOCK ? 2
       for (int ks = 0; ks < KSTEPS; ++ks)
         of[ks] = *reinterpret_cast<const vec8*>(row_address(ob, st_row, o_rb, (ks * 16 + hi * 8) * 2));
     }
-    st_lse2 = p.lse[b * p.lse_sb + h0 * p.lse_sh + q_row0 + st_row] * LOG2E;
   }
   if (!STAGE_X) {
 #pragma unroll
@@ -373,9 +381,14 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 || PASS == HA_BWD_DQ_BLOCK ? 2
     // The stationary rows come through LDS (dK/dV passes; dQ passes at d = 64, where the 32 KB fit beside
     // two workgroups per CU): whole rows per 8 or 16 consecutive lanes (one 128- or 256-byte request per
     // row) instead of one 16-byte piece of 64 different rows per instruction.  Each wave stages its own
-    // 32 rows, so only the wave itself has to wait.
+    // 32 rows, so only the wave itself has to wait.  The row numbers (stationary rows, first tile) are
+    // waited for first; then the stationary rows, the queries' output rows (dQ passes: into the second
+    // pair of tile buffers, which the loop fills only after its first barrier) and the first tile are all
+    // asked for together: two memory round trips before the first chunk instead of three or four.
     constexpr int ROWS_PER_LOAD = 64 / PR;
     const int row_in_load = lane / PR, phys_piece = lane % PR;
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the row numbers
+    unsigned char* const o_stage = (wave_s < 2 ? lds_y1[1] : lds_y2[1]) + (wave_s & 1) * 32 * D * 2;
 #pragma unroll
     for (int j = 0; j < 32 / ROWS_PER_LOAD; ++j) {
       const int r = j * ROWS_PER_LOAD + row_in_load;  // 0..31: a stationary row of this wave
@@ -384,35 +397,26 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 || PASS == HA_BWD_DQ_BLOCK ? 2
       const int dst = (wave_s * 32 + j * ROWS_PER_LOAD) * D * 2;
       global_to_lds_16(row_address(x1b, row, x1_rb, piece), lds_x1 + dst);
       global_to_lds_16(row_address(x2b, row, x2_rb, piece), lds_x2 + dst);
+      if (!KEY_ST) global_to_lds_16(row_address(ob, row, o_rb, piece), o_stage + j * ROWS_PER_LOAD * D * 2);
     }
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): these rows, and the row numbers of the first tile
+  }
+
+  if (!KEY_ST) st_lse2 = p.lse[b * p.lse_sb + h0 * p.lse_sh + q_row0 + st_row] * LOG2E;
+  load_tile(0);
+  fetch_rows(1);
+
+  if (STAGE_X) {
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the stationary rows (and the first tile) have landed
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ++ks) {
       const int off = bwd_tile_offset<D>(wave_s * 32 + col, ks * 2 + hi);
       x1f[ks] = lds_read_k<T>(lds_x1, off);
       x2f[ks] = lds_read_k<T>(lds_x2, off);
-    }
-    if (!KEY_ST) {
-      // the queries' output rows (for D) follow through the first staging area, once it has been read
-      __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
-      __builtin_amdgcn_wave_barrier();
-#pragma unroll
-      for (int j = 0; j < 32 / ROWS_PER_LOAD; ++j) {
-        const int r = j * ROWS_PER_LOAD + row_in_load;
-        const int row = __shfl(st_row, r);
-        const uint32_t piece = (uint32_t)((phys_piece ^ bwd_swizzle<D>(r)) << 4);
-        global_to_lds_16(row_address(ob, row, o_rb, piece), lds_x1 + (wave_s * 32 + j * ROWS_PER_LOAD) * D * 2);
+      if (!KEY_ST) {
+        const unsigned char* const o_stage = (wave_s < 2 ? lds_y1[1] : lds_y2[1]) + (wave_s & 1) * 32 * D * 2;
+        of[ks] = lds_read_k<T>(o_stage, bwd_tile_offset<D>(col, ks * 2 + hi));
       }
     }
-  }
-
-  load_tile(0);
-  fetch_rows(1);
-
-  if (!KEY_ST && STAGE_X) {
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the output rows (and the first tile) have landed
-#pragma unroll
-    for (int ks = 0; ks < KSTEPS; ++ks) of[ks] = lds_read_k<T>(lds_x1, bwd_tile_offset<D>(wave_s * 32 + col, ks * 2 + hi));
   }
   if (!KEY_ST) {
     // D = sum_c dO * O of the lane's query: the two lanes of a column hold complementary pieces of the row.
@@ -481,8 +485,6 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 || PASS == HA_BWD_DQ_BLOCK ? 2
     } else if (PASS == HA_BWD_DKV_EXACT) {
       wave_in = !CAUSAL || y_hi >= st_lo;
       needs_mask = y_hi >= p.n_q || (CAUSAL && y_lo < st_hi);
-    } else if (PASS == HA_BWD_DKV_SAMPLED) {
-      needs_mask = y_hi >= y_end;
     }
 
     // One chunk of one wave as straight-line code, one copy with the mask and one without: the
@@ -535,8 +537,6 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 || PASS == HA_BWD_DQ_BLOCK ? 2
                 } else if (PASS == HA_BWD_DKV_EXACT) {
                   const int query = y_first + cc * YC + r0 + e;
                   ok = query < p.n_q && (!CAUSAL || st_pos <= query);
-                } else if (PASS == HA_BWD_DKV_SAMPLED) {
-                  ok = y_first + cc * YC + r0 + e < y_end;
                 }
                 pv = ok ? pv : 0.f;
               }
@@ -564,8 +564,11 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 || PASS == HA_BWD_DQ_BLOCK ? 2
             }
           }
     };
+    // the passes whose pairs are masked one by one: the diagonal and the end of the sequence in exact
+    // attention (the sampled keys' pass handles the end of its query range through L)
+    constexpr bool CAN_MASK = PASS == HA_BWD_DQ_EXACT || PASS == HA_BWD_DKV_EXACT;
     if (wave_in) {
-      if (needs_mask)
+      if (CAN_MASK && needs_mask)
         chunk_body(std::true_type{});
       else
         chunk_body(std::false_type{});
