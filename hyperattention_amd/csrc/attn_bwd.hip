@@ -583,11 +583,37 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 || PASS == HA_BWD_DQ_BLOCK ? 2
   // exact passes, whose rows are neighbours anyway, lose 1-3 % to the extra barrier and registers).
   constexpr bool TURN_RESULTS = PASS == HA_BWD_DQ_BLOCK || PASS == HA_BWD_DKV_BLOCK;
   if (TURN_RESULTS) {
+    constexpr int ROWS_PER_STORE = 64 / PR;
+    constexpr int NJ = 32 / ROWS_PER_STORE;
+    const int row_in_store = lane / PR, out_piece = lane % PR;
+    unsigned char* const base1 =
+        KEY_ST ? (unsigned char*)((T*)p.dk + b * p.dk_sb + hk * p.dk_sh + k_row0 * p.dk_sn)
+               : (unsigned char*)((T*)p.dq + b * p.dq_sb + h0 * p.dq_sh + q_row0 * p.dq_sn);
+    unsigned char* const base2 = (unsigned char*)((T*)p.dv + b * p.dv_sb + hk * p.dv_sh + k_row0 * p.dv_sn);
+    const int64_t stride1 = (KEY_ST ? p.dk_sn : p.dq_sn) * 2, stride2 = p.dv_sn * 2;
+    // the rows this lane writes (a piece of NJ rows of its wave), and, when the call adds to what is there,
+    // their present values: all asked for at once, ahead of the barrier and the turn through LDS (one
+    // memory round trip; fetched where each row is stored they were NJ round trips per tensor, one after
+    // the other, and a third of the block pass's time)
+    int rows_j[NJ];
+    bool valid_j[NJ];
+    vec8 old1[NJ], old2[NJ];
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+      const int r = j * ROWS_PER_STORE + row_in_store;
+      rows_j[j] = __shfl(st_row, r);  // lanes past the end hold the first row: a valid address
+      valid_j[j] = __shfl((int)st_valid, r) != 0;
+    }
+    if (p.accumulate) {
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) {
+        old1[j] = *reinterpret_cast<const vec8*>(base1 + rows_j[j] * stride1 + out_piece * 16);
+        if (KEY_ST) old2[j] = *reinterpret_cast<const vec8*>(base2 + rows_j[j] * stride2 + out_piece * 16);
+      }
+    }
     __syncthreads();
     unsigned char* const turn = lds_y1[0] + wave_s * (32 * D * 2);
-    constexpr int ROWS_PER_STORE = 64 / PR;
-    const int row_in_store = lane / PR, out_piece = lane % PR;
-    auto store_rows = [&](const f32x16 (&acc)[DB], unsigned char* base, int64_t row_stride_bytes) {
+    auto store_rows = [&](const f32x16 (&acc)[DB], unsigned char* base, int64_t row_stride_bytes, const vec8 (&old)[NJ]) {
       // [row][D] in the output type, 16-byte pieces XOR-ed with the row number
 #pragma unroll
       for (int db = 0; db < DB; ++db)
@@ -600,28 +626,18 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 || PASS == HA_BWD_DQ_BLOCK ? 2
           *reinterpret_cast<vec4*>(turn + col * (D * 2) + piece * 16 + hi * 8) = o;
         }
 #pragma unroll
-      for (int j = 0; j < 32 / ROWS_PER_STORE; ++j) {
+      for (int j = 0; j < NJ; ++j) {
         const int r = j * ROWS_PER_STORE + row_in_store;
-        const int row = __shfl(st_row, r);
-        const bool valid = __shfl((int)st_valid, r) != 0;
         vec8 o = *reinterpret_cast<const vec8*>(turn + r * (D * 2) + ((out_piece ^ (r & (PR - 1))) << 4));
-        if (valid) {
-          vec8* const dst = reinterpret_cast<vec8*>(base + row * row_stride_bytes + out_piece * 16);
-          if (p.accumulate) {
-            const vec8 old = *dst;
+        if (p.accumulate) {
 #pragma unroll
-            for (int e = 0; e < 8; ++e) o[e] = (T)((float)o[e] + (float)old[e]);
-          }
-          *dst = o;
+          for (int e = 0; e < 8; ++e) o[e] = (T)((float)o[e] + (float)old[j][e]);
         }
+        if (valid_j[j]) *reinterpret_cast<vec8*>(base + rows_j[j] * row_stride_bytes + out_piece * 16) = o;
       }
     };
-    if (!KEY_ST) {
-      store_rows(acc1, (unsigned char*)((T*)p.dq + b * p.dq_sb + h0 * p.dq_sh + q_row0 * p.dq_sn), p.dq_sn * 2);
-    } else {
-      store_rows(acc1, (unsigned char*)((T*)p.dk + b * p.dk_sb + hk * p.dk_sh + k_row0 * p.dk_sn), p.dk_sn * 2);
-      store_rows(acc2, (unsigned char*)((T*)p.dv + b * p.dv_sb + hk * p.dv_sh + k_row0 * p.dv_sn), p.dv_sn * 2);
-    }
+    store_rows(acc1, base1, stride1, old1);
+    if (KEY_ST) store_rows(acc2, base2, stride2, old2);
   }
   if (!TURN_RESULTS && !KEY_ST && st_valid) {
     unsigned char* const dqb = (unsigned char*)((T*)p.dq + b * p.dq_sb + h0 * p.dq_sh + q_row0 * p.dq_sn) + (int64_t)st_row * p.dq_sn * 2;
