@@ -170,6 +170,52 @@ def test_block_backward_int32_indices_and_sorted_buckets(ha):
         _check(got, want, f"block {name}", dtype)
 
 
+# ------------------------------------------------------------------------- adding to gradients that are there
+@pytest.mark.parametrize("kind,dtype,d", [("block", torch.bfloat16, 64), ("block", torch.float16, 128),
+                                          ("block_smooth", torch.float16, 64), ("flash_causal", torch.bfloat16, 64),
+                                          ("flash", torch.float16, 128)])
+def test_backward_accumulate_adds_to_what_is_there(ha, kind, dtype, d):
+    # ha_attn_grads.accumulate: dq, dk, dv hold values when the call starts and hold value + gradient when it
+    # ends (one rounding of the fp32 sum), through the C ABI, against the same call without the flag
+    import ctypes
+    from hyperattention_amd import _lib, ops
+    b, h, n, block, sample = 2, 3, 768, 256, 128
+    q, k, v, do = (_randn((b, h, n, d), 170 + i, dtype).cuda().transpose(1, 2).contiguous() for i in range(4))
+    o = torch.empty_like(q)
+    lse = torch.empty((b, h, n), device="cuda", dtype=torch.float32)
+    lib = _lib.lib()
+    stream = ops._stream(q)
+    if kind.startswith("block"):
+        qi, ki = (_perms(b, h, n, 175 + i).cuda().transpose(1, 2) for i in range(2))
+        a, keep = ops._block_attn_args(q, k, v, o, lse, qi, ki, block, sample, d ** -0.5, kind == "block_smooth", None)
+        _lib.check(lib.ha_block_attn_fwd(ctypes.byref(a), stream))
+        run = lambda g: _lib.check(lib.ha_block_attn_bwd(ctypes.byref(a), ctypes.byref(g), stream))
+        t = a.t
+    else:
+        t = ops._operands(q, k, v, o, lse, d ** -0.5, layout_bnhd=True, lse_row_stride=n)
+        causal = int(kind == "flash_causal")
+        _lib.check(lib.ha_flash_attn_fwd(ctypes.byref(t), causal, stream))
+        run = lambda g: _lib.check(lib.ha_flash_attn_bwd(ctypes.byref(t), causal, ctypes.byref(g), stream))
+    sample_size = sample if kind.startswith("block") else 0
+    plain = [torch.empty_like(x) for x in (q, k, v)]
+    g0, ws0 = ops._attn_grads(t, do, *plain, sample_size=sample_size)
+    run(g0)
+    base = [_randn((b, h, n, d), 180 + i, dtype).cuda().transpose(1, 2).contiguous() for i in range(3)]
+    added = [x.clone() for x in base]
+    g1, ws1 = ops._attn_grads(t, do, *added, accumulate=True, sample_size=sample_size)
+    run(g1)
+    torch.cuda.synchronize()
+    ulp = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
+    for got, grad, start, name in zip(added, plain, base, ("dq", "dk", "dv")):
+        # the kernel adds its fp32 sum to the stored value and rounds once, where `grad` is that sum rounded
+        # (the sampled keys' share is added by a second kernel, with a rounding of its own): a few roundings
+        # of values of the result's size, so the distance is of the order of one unit in the last place
+        want = grad.float() + start.float()
+        rel = float((got.float() - want).norm() / want.norm())
+        assert rel <= 1.5 * ulp, f"{kind} {name}: relative distance {rel:.3e}"
+        assert not torch.equal(got, start)
+
+
 # ------------------------------------------------------------------------- grouped-query heads
 @pytest.mark.parametrize("kind", ["flash", "flash_causal", "block"])
 def test_backward_grouped_query_heads_through_the_c_abi(ha, kind):
