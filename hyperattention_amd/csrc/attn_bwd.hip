@@ -901,9 +901,9 @@ int run_block_bwd(const ha_block_attn_args& a, const ha_attn_grads& g, hipStream
   st = launch_pass<T, D, HA_BWD_DKV_BLOCK, false>(p, bhk * (t.n_k / ST_ROWS), stream, "ha_block_attn_bwd: dk, dv of the blocks");
   if (st != HA_OK) return st;
   if (a.sample_size > 0) {
-    const int64_t n4 = (w.acc_floats + 3) / 4;
+    // the two arrays of sums lie one behind the other in the workspace (each a multiple of 256 bytes): one fill
+    const int64_t n4 = (int64_t)(((char*)w.dv32 - (char*)w.dk32) + align256(w.acc_floats * 4)) / 16;
     hipLaunchKernelGGL(ha_bwd_zero_kernel, dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, stream, (f32x4*)w.dk32, n4);
-    hipLaunchKernelGGL(ha_bwd_zero_kernel, dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, stream, (f32x4*)w.dv32, n4);
     st = ha_launch_status("attention backward: clear");
     if (st != HA_OK) return st;
     // every query attends every sampled key: the queries are cut into ranges, as long as possible (each
