@@ -20,7 +20,7 @@ struct ha_attn_bwd_params {
   const void *q, *k, *v, *dout;
   const void* out;   // the forward's output and log-sum-exp: read by the dq passes, which write `stats`
   const float* lse;
-  f32x2* stats;  // per query {log-sum-exp * log2(e), scale * sum_c dO*O}, contiguous (batch, heads, n_q): written
+  f32x2* stats;  // per query {log-sum-exp * log2(e), -sum_c dO*O}, contiguous (batch, heads, n_q): written
                  // by the dq pass of a call for the dk/dv passes that follow it
   void* dq;
   void *dk, *dv;       // written directly by the exact and the block passes

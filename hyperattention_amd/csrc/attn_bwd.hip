@@ -82,6 +82,9 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 || PASS == HA_BWD_DQ_BLOCK ? 2
   typedef typename ElemTraits<T>::vec8 vec8;
   typedef typename ElemTraits<T>::vec4 vec4;
   constexpr bool KEY_ST = PASS == HA_BWD_DKV_EXACT || PASS == HA_BWD_DKV_BLOCK || PASS == HA_BWD_DKV_SAMPLED;
+  // the gathered dK/dV passes start their dP accumulators from -D (below); the exact pass, at its register
+  // limit, subtracts D * scale per pair like the dQ passes
+  constexpr bool FOLD_D = PASS == HA_BWD_DKV_BLOCK || PASS == HA_BWD_DKV_SAMPLED;
   constexpr int KSTEPS = D / 16;  // MFMA k-steps over the head dim
   constexpr int DB = D / 32;      // 32-row blocks of the transposed gradients
   constexpr int PR = D / 8;       // 16-byte pieces per row
@@ -92,7 +95,7 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 || PASS == HA_BWD_DQ_BLOCK ? 2
   __shared__ __attribute__((aligned(1024))) unsigned char lds_y1[2][TILE_BYTES];
   __shared__ __attribute__((aligned(1024))) unsigned char lds_y2[2][TILE_BYTES];
   __shared__ __attribute__((aligned(16))) float lds_lse[2][YC];    // dK/dV passes: L (log2 units) of the streamed queries
-  __shared__ __attribute__((aligned(16))) float lds_delta[2][YC];  // and their D * scale
+  __shared__ __attribute__((aligned(16))) float lds_delta[2][YC];  // and their -D (gathered passes) or D * scale (exact pass)
   constexpr bool STAGE_X = KEY_ST || D <= 64;
   __shared__ __attribute__((aligned(1024))) unsigned char lds_x1[STAGE_X ? ST_ROWS * D * 2 : 16];  // staging of the
   __shared__ __attribute__((aligned(1024))) unsigned char lds_x2[STAGE_X ? ST_ROWS * D * 2 : 16];  // stationary rows
@@ -141,7 +144,7 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 || PASS == HA_BWD_DQ_BLOCK ? 2
   // query-side tensors of query head h0 + gi
   auto q_head = [&](int gi) { return (const unsigned char*)((const T*)p.q + b * p.q_sb + (h0 + gi) * p.q_sh + q_row0 * p.q_sn); };
   auto do_head = [&](int gi) { return (const unsigned char*)((const T*)p.dout + b * p.do_sb + (h0 + gi) * p.do_sh + q_row0 * p.do_sn); };
-  // per query: {L in log2 units, D * scale} with D_i = sum_c dO_ic O_ic (src/hyper_attn_triton.py:195-226),
+  // per query: {L in log2 units, -D} with D_i = sum_c dO_ic O_ic (src/hyper_attn_triton.py:195-226),
   // written by the dq pass of the call
   auto stats_head = [&](int gi) { return p.stats + ((int64_t)(b * p.heads + h0 + gi) * p.segs + seg) * p.n_q; };
   const int idx_shift = p.idx64 ? 3 : 2;
@@ -352,7 +355,7 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 || PASS == HA_BWD_DQ_BLOCK ? 2
     if (KEY_ST) {
       const f32x2 sd = stats_head(group_next)[stat_row_next];
       stat_lse = stat_past_end_next ? __builtin_inff() : sd[0];
-      stat_delta = sd[1];
+      stat_delta = FOLD_D ? sd[1] : -sd[1] * p.scale;  // the word holds -D
     }
   };
 
@@ -426,8 +429,9 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 || PASS == HA_BWD_DQ_BLOCK ? 2
     for (int ks = 0; ks < KSTEPS; ++ks)
 #pragma unroll
       for (int e = 0; e < 8; ++e) part = __builtin_fmaf((float)of[ks][e], (float)x2f[ks][e], part);
-    st_delta = ha_sum_xor32(part) * p.scale;
-    if (hi == 0 && st_valid) p.stats[((int64_t)(b * p.heads + h0) * p.segs + seg) * p.n_q + st_row] = f32x2{st_lse2, st_delta};
+    const float d_row = ha_sum_xor32(part);
+    st_delta = d_row * p.scale;
+    if (hi == 0 && st_valid) p.stats[((int64_t)(b * p.heads + h0) * p.segs + seg) * p.n_q + st_row] = f32x2{st_lse2, -d_row};
   }
 
   // per-lane LDS offsets of the operand reads
@@ -502,6 +506,17 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 || PASS == HA_BWD_DQ_BLOCK ? 2
           s[rb][i] = 0.f;
           dp[rb][i] = 0.f;
         }
+        if (FOLD_D) {
+          // dP' starts from -D of its streamed query (accumulator element 4g + e is row 8g + 4 hi + e of the
+          // 32-row block): the MFMAs then leave dP - D, and dS' = P' (dP - D) is one product; its factor
+          // `scale` is applied to the sums of dK at the end
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            const f32x4 nd = *reinterpret_cast<const f32x4*>(&lds_delta[buf][rb * 32 + g * 8 + hi * 4]);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) dp[rb][g * 4 + e] = nd[e];
+          }
+        }
 #pragma unroll
         for (int ks = 0; ks < KSTEPS; ++ks) {
           const vec8 a1 = lds_read_k<T>(y1, off_rows[ks] + rb * 32 * D * 2);
@@ -521,10 +536,8 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 || PASS == HA_BWD_DQ_BLOCK ? 2
           for (int g = 0; g < 4; ++g) {
             const int r0 = rb * 32 + g * 8 + hi * 4;  // streamed rows r0..r0+3 of the chunk
             f32x4 l4 = {st_lse2, st_lse2, st_lse2, st_lse2}, d4 = {st_delta, st_delta, st_delta, st_delta};
-            if (KEY_ST) {
-              l4 = *reinterpret_cast<const f32x4*>(&lds_lse[buf][r0]);
-              d4 = *reinterpret_cast<const f32x4*>(&lds_delta[buf][r0]);
-            }
+            if (KEY_ST) l4 = *reinterpret_cast<const f32x4*>(&lds_lse[buf][r0]);
+            if (KEY_ST && !FOLD_D) d4 = *reinterpret_cast<const f32x4*>(&lds_delta[buf][r0]);
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
               const int i = g * 4 + e;
@@ -540,8 +553,9 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 || PASS == HA_BWD_DQ_BLOCK ? 2
                 }
                 pv = ok ? pv : 0.f;
               }
-              // d4 holds D * scale: dS = P (dP - D) scale in one FMA and one product
-              const float dsv = pv * __builtin_fmaf(dp[rb][i], p.scale, -d4[e]);
+              // d4 holds D * scale: dS = P (dP - D) scale in one FMA and one product; the gathered dK/dV passes
+              // hold dP - D in dp already
+              const float dsv = FOLD_D ? pv * dp[rb][i] : pv * __builtin_fmaf(dp[rb][i], p.scale, -d4[e]);
               pb[rb][i >> 3][i & 7] = (T)pv;
               dsb[rb][i >> 3][i & 7] = (T)dsv;
             }
@@ -573,6 +587,14 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 || PASS == HA_BWD_DQ_BLOCK ? 2
       else
         chunk_body(std::false_type{});
     }
+  }
+
+  if (FOLD_D) {
+    // dK was summed without the factor `scale` of dS
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc1[db][i] *= p.scale;
   }
 
   // ---- results -------------------------------------------------------------------------------
@@ -794,7 +816,7 @@ int launch_pass(const ha_attn_bwd_params& p, int64_t grid, hipStream_t stream, c
 inline int64_t align256(int64_t v) { return (v + 255) & ~(int64_t)255; }
 
 struct Workspace {
-  f32x2* stats;  // per query {L * log2(e), D * scale}
+  f32x2* stats;  // per query {L * log2(e), -D}
   float* dk32;  // sums of the sampled keys, (batch, kv_heads, sample_size, d) fp32
   float* dv32;
   int64_t acc_floats;  // per accumulator
