@@ -364,6 +364,9 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 || PASS == HA_BWD_DQ_BLOCK ? 2
   fetch_rows(0);
   vec8 x1f[KSTEPS], x2f[KSTEPS];
   float st_lse2 = 0.f, st_delta = 0.f;  // dQ passes: L (log2 units) and D * scale of the lane's query
+  f32x16 neg_d;  // dQ passes: -D in every element, what the dP accumulators of a chunk start from
+#pragma unroll
+  for (int i = 0; i < 16; ++i) neg_d[i] = 0.f;
   vec8 of[KSTEPS];  // dQ passes: the lane's pieces of its query's output row
   const unsigned char* const ob = (const unsigned char*)((const T*)p.out + b * p.o_sb + h0 * p.o_sh + q_row0 * p.o_sn);
   const uint32_t o_rb = (uint32_t)p.o_sn * 2;
@@ -431,6 +434,8 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 || PASS == HA_BWD_DQ_BLOCK ? 2
       for (int e = 0; e < 8; ++e) part = __builtin_fmaf((float)of[ks][e], (float)x2f[ks][e], part);
     const float d_row = ha_sum_xor32(part);
     st_delta = d_row * p.scale;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) neg_d[i] = -d_row;
     if (hi == 0 && st_valid) p.stats[((int64_t)(b * p.heads + h0) * p.segs + seg) * p.n_q + st_row] = f32x2{st_lse2, -d_row};
   }
 
@@ -506,6 +511,7 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 || PASS == HA_BWD_DQ_BLOCK ? 2
           s[rb][i] = 0.f;
           dp[rb][i] = 0.f;
         }
+        if (!KEY_ST) dp[rb] = neg_d;
         if (FOLD_D) {
           // dP' starts from -D of its streamed query (accumulator element 4g + e is row 8g + 4 hi + e of the
           // 32-row block): the MFMAs then leave dP - D, and dS' = P' (dP - D) is one product; its factor
@@ -555,7 +561,7 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 || PASS == HA_BWD_DQ_BLOCK ? 2
               }
               // d4 holds D * scale: dS = P (dP - D) scale in one FMA and one product; the gathered dK/dV passes
               // hold dP - D in dp already
-              const float dsv = FOLD_D ? pv * dp[rb][i] : pv * __builtin_fmaf(dp[rb][i], p.scale, -d4[e]);
+              const float dsv = (FOLD_D || !KEY_ST) ? pv * dp[rb][i] : pv * __builtin_fmaf(dp[rb][i], p.scale, -d4[e]);
               pb[rb][i >> 3][i & 7] = (T)pv;
               dsb[rb][i >> 3][i & 7] = (T)dsv;
             }
@@ -589,8 +595,8 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 || PASS == HA_BWD_DQ_BLOCK ? 2
     }
   }
 
-  if (FOLD_D) {
-    // dK was summed without the factor `scale` of dS
+  if (FOLD_D || !KEY_ST) {
+    // dK (dQ) was summed without the factor `scale` of dS
 #pragma unroll
     for (int db = 0; db < DB; ++db)
 #pragma unroll
