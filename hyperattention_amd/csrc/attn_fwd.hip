@@ -273,17 +273,22 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
   // K and V rows of the tile (the same for all of them) come from HBM once and from L2 after that.
   const int wg = xcd_contiguous_id(blockIdx.x, gridDim.x);
   const int qtiles = (p.n_q + WG_QUERIES - 1) / WG_QUERIES;
+  // Exact causal attention: a workgroup takes the tile pair (qtiles-1-s, s), so that every workgroup of the
+  // launch has the same number of key chunks to go through.  The hardware hands out workgroups in order and
+  // a slot freed by a short one stays empty until the ones queued before it are placed: with one tile per
+  // workgroup (4 to 32 chunks in a 2048-row leaf) the slots of a CU stood empty for 8 us at a time.
+  constexpr bool PAIRED = CAUSAL && !GATHER;
+  const int wg_per_seq = PAIRED ? (qtiles + 1) / 2 : qtiles;  // what p.div_qtiles divides by
   const int wg_tile = fast_div(wg, p.div_kv_group);
   const int hg = wg - wg_tile * p.kv_group;
   const int vseq = fast_div(wg_tile, p.div_qtiles);
-  // causal: the tiles with the most keys go first, so that the last workgroups of the grid are short
-  const int qt_fwd = wg_tile - vseq * qtiles;
-  const int qt = CAUSAL ? qtiles - 1 - qt_fwd : qt_fwd;
+  const int slot = wg_tile - vseq * wg_per_seq;
   const int bhk = fast_div(vseq, p.div_segs);
   const int seg = vseq - bhk * p.segs;
   const int b = fast_div(bhk, p.div_kv_heads), hk = bhk - b * fast_div(p.heads, p.div_kv_group);
   const int h = hk * p.kv_group + hg;
 
+  auto run_tile = [&](const int qt) __attribute__((always_inline)) {
   // ---- row numbers of the queries: the first thing the workgroup has to wait for, so they are asked
   // for before the rest of the set-up (sorted query positions of this head: entries of 4 or 8 bytes,
   // the row number in the low word) ------------------------------------------------------------------
@@ -771,6 +776,16 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
 #undef HA_LOAD_TILE
 #undef HA_APPLY_MASK
 #undef HA_REWEIGHT
+  };  // run_tile
+  if (PAIRED) {
+    // the long tile first.  No barrier between the two: the last iteration of a tile ends with one, and after
+    // it a wave touches only its own part of the query region.
+    const int t_long = qtiles - 1 - slot;
+    run_tile(t_long);
+    if (slot != t_long) run_tile(slot);
+  } else {
+    run_tile(slot);
+  }
 }
 
 namespace {
@@ -821,7 +836,8 @@ int ha_attn_launch(const ha_attn_kernel_params& params, int d, int dv, int dtype
   const int width = d <= 64 && dv <= 64 ? 64 : 128;
   p.qk_pieces = d / 8;
   p.v_pieces = dv / 8;
-  const int64_t qtiles = (p.n_q + WG_QUERIES - 1) / WG_QUERIES;
+  int64_t qtiles = (p.n_q + WG_QUERIES - 1) / WG_QUERIES;
+  if (causal && !gather) qtiles = (qtiles + 1) / 2;  // exact causal attention: one workgroup per pair of tiles
   p.div_qtiles = make_divisor(qtiles);
   p.div_segs = make_divisor(p.segs);
   p.div_heads = make_divisor(p.heads);
