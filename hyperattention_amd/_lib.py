@@ -17,7 +17,7 @@ _BUILD = os.path.join(_PKG, "build")
 LIB_PATH = os.path.join(_PKG, "libhyperattn.so")
 
 SOURCES = ["api.hip", "lsh_hash.hip", "bucket_sort.hip", "gather_rows.hip", "lse_merge.hip", "attn_fwd.hip",
-           "attn_bwd.hip"]
+           "attn_bwd.hip", "power_probe.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
@@ -31,7 +31,7 @@ SYMBOLS = [
     "ha_bucket_argsort", "ha_bucket_argsort_static", "ha_gather_rows", "ha_block_attn_fwd", "ha_flash_attn_fwd",
     "ha_attn_bwd_workspace_bytes", "ha_block_attn_bwd", "ha_flash_attn_bwd", "ha_lse_merge",
     "ha_lse_merge_segments",
-    "ha_forward_workspace_bytes", "ha_forward", "ha_forward_sort", "ha_lse_merge_levels",
+    "ha_forward_workspace_bytes", "ha_forward", "ha_forward_sort", "ha_lse_merge_levels", "ha_power_probe",
 ]
 
 HA_F16, HA_BF16 = 0, 1
@@ -54,7 +54,7 @@ def build(verbose: bool = False) -> str:
             print(res.stderr)
         return obj
 
-    with ThreadPoolExecutor(max_workers=min(6, len(SOURCES))) as pool:
+    with ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as pool:
         objs = list(pool.map(compile_one, SOURCES))
     tmp = LIB_PATH + ".tmp"
     res = subprocess.run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", tmp, *objs],
@@ -169,6 +169,8 @@ def _declare(lib):
     lib.ha_lse_merge_levels.restype = ci
     lib.ha_lse_merge_levels.argtypes = [vp, vp, ctypes.POINTER(vp), ctypes.POINTER(vp), ctypes.POINTER(vp), vp, vp, vp,
                                         ci, i64, i64, i64, ci, vp]
+    lib.ha_power_probe.restype = ci
+    lib.ha_power_probe.argtypes = [ci, i64, ci, vp, vp]
     lib.ha_forward_sort.restype = ci
     lib.ha_forward_sort.argtypes = [ctypes.POINTER(ForwardArgs), ctypes.POINTER(i64), ctypes.POINTER(i64),
                                     ctypes.POINTER(ci), vp]

@@ -326,6 +326,19 @@ int ha_forward(const ha_forward_args* args, void* stream);
 int ha_forward_sort(const ha_forward_args* args, int64_t* q_idx_offset, int64_t* k_idx_offset, int* num_levels,
                     void* stream);
 
+/* ---------------------------------------------------------------------------------------------
+ * Measurement aid (no counterpart in the reference, not on the forward path): single-purpose loops that
+ * price the board's power limit.  `workgroups` workgroups of 256 threads each run `trips` trips of four
+ * half-step blocks (8 large MFMAs each, where the kind has them): HA_PROBE_MFMA on register operands only,
+ * HA_PROBE_LDS_MFMA with the attention kernels' LDS operand reads, HA_PROBE_SOFTMAX the soft-max arithmetic of
+ * the blocks alone, HA_PROBE_BLOCK all of it, HA_PROBE_BLOCK_WIDE all of it with 16 MFMAs per block (the d = 128 ratio).  One
+ * trip of one workgroup is 4 waves * 4 blocks * 8 (16) MFMAs of 32768 flops.
+ * sink: 256 floats of device memory (never written in practice).  bench.py times these loops with the board
+ * power sampled beside them.
+ */
+enum { HA_PROBE_MFMA = 0, HA_PROBE_LDS_MFMA = 1, HA_PROBE_SOFTMAX = 2, HA_PROBE_BLOCK = 3, HA_PROBE_BLOCK_WIDE = 4 };
+int ha_power_probe(int kind, int64_t trips, int workgroups, void* sink, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
