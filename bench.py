@@ -407,7 +407,8 @@ class Workload:
                                      rng=torch.Generator().manual_seed(seed)).to(device="cuda", dtype=self.tdt)
         self.scale = d ** -0.5
         self.proj2 = self.module.lsh.proj_dir.reshape(1, 1, d, 8)
-        self.workspace = {}
+        from hyperattention_amd import ops
+        self.workspace = ops.WorkspaceCache()
         self.out = torch.zeros((b, h, n, d), device="cuda", dtype=self.tdt)
         self.lse = torch.zeros((b, h, n), device="cuda", dtype=torch.float32)
 

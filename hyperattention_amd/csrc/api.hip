@@ -274,6 +274,20 @@ void forward_operands(const ha_forward_args& a, ha_attn_operands& t) {
   t.dtype = a.dtype;
 }
 
+// Row alignment of the tensors a forward pass reads and writes, checked before the first launch (the hash
+// and the attention kernels move rows in 16-byte pieces).
+int check_forward_layout(const ha_attn_operands& t, bool with_values, const char* who) {
+  HA_REQUIRE(((uintptr_t)t.q % 16) == 0 && ((uintptr_t)t.k % 16) == 0, HA_ERR_SHAPE, "%s: tensors must be 16-byte aligned", who);
+  const int64_t qk[] = {t.q_stride_b, t.q_stride_h, t.q_stride_n, t.k_stride_b, t.k_stride_h, t.k_stride_n};
+  for (int64_t s : qk) HA_REQUIRE(s % 8 == 0, HA_ERR_SHAPE, "%s: rows must be 16-byte aligned", who);
+  if (with_values) {
+    HA_REQUIRE(((uintptr_t)t.v % 16) == 0 && ((uintptr_t)t.out % 16) == 0, HA_ERR_SHAPE, "%s: tensors must be 16-byte aligned", who);
+    const int64_t vo[] = {t.v_stride_b, t.v_stride_h, t.v_stride_n};
+    for (int64_t s : vo) HA_REQUIRE(s % 8 == 0, HA_ERR_SHAPE, "%s: rows must be 16-byte aligned", who);
+  }
+  return HA_OK;
+}
+
 // Bucket ids of q and k, then the stable bucket order of the query and key segment of every hashed level
 // (hyper_attention.py:112-117 at every level of the recursion), as int32 rows local to the segment.
 int hash_and_sort(const ha_forward_args& a, const Plan& pl, const Workspace& w, const ha_attn_operands& t,
@@ -436,6 +450,8 @@ extern "C" int ha_forward_sort(const ha_forward_args* args, int64_t* q_idx_offse
   ha_forward_args b = a;
   b.dv = a.d;
   forward_operands(b, t);
+  st = check_forward_layout(t, false, "ha_forward_sort");
+  if (st != HA_OK) return st;
   return hash_and_sort(a, pl, w, t, (hipStream_t)stream);
 }
 
@@ -458,6 +474,8 @@ extern "C" int ha_forward(const ha_forward_args* args, void* stream_) {
 
   ha_attn_operands t;
   forward_operands(a, t);
+  st = check_forward_layout(t, true, "ha_forward");
+  if (st != HA_OK) return st;
 
   // 1. bucket ids, once for the whole tensors (the projection does not depend on the level), and
   // 2. the bucket order of every segment of every hashed level

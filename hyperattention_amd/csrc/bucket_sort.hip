@@ -461,8 +461,10 @@ constexpr int MAX_DEVICES = 64;
 std::mutex scratch_mutex;
 void* scratch_ptr[MAX_DEVICES] = {nullptr};
 
-// device address of `scratch` on the current device (0 on failure, with the status in *st)
-void* scratch_on_current_device(int* st) {
+// device address of `scratch` on the current device (0 on failure, with the status in *st).  The address is
+// asked for on the first call on a device; that call must not sit inside a stream capture (the runtime may
+// have to load the code object and the array then), so a first call under capture is refused.
+void* scratch_on_current_device(hipStream_t stream, int* st) {
   int dev = -1;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess || dev < 0 || dev >= MAX_DEVICES) {
@@ -471,6 +473,13 @@ void* scratch_on_current_device(int* st) {
   }
   std::lock_guard<std::mutex> lock(scratch_mutex);
   if (!scratch_ptr[dev]) {
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &capturing) != hipSuccess || capturing != hipStreamCaptureStatusNone) {
+      (void)hipGetLastError();
+      *st = ha_fail(HA_ERR_UNSUPPORTED, "ha_bucket_argsort_static: the first call on a device must be made outside "
+                    "stream capture (it looks up the scratch array's address)");
+      return nullptr;
+    }
     void* p = nullptr;
     e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
     if (e != hipSuccess || !p) {
@@ -496,7 +505,7 @@ extern "C" int ha_bucket_argsort_static(const int32_t* keys, void* idx_out, int 
              "ha_bucket_argsort with a workspace",
              (long long)need, (long long)HA_SORT_SCRATCH_BYTES);
   int st = HA_OK;
-  void* ws = scratch_on_current_device(&st);
+  void* ws = scratch_on_current_device((hipStream_t)stream, &st);
   if (!ws) return st;
   // every histogram entry and intermediate order that is read is written by the same call first: nothing
   // has to start at zero

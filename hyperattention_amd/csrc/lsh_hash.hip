@@ -40,14 +40,15 @@ constexpr int HASH_UNROLL = 8;           // tiles in flight per wave
 // MFMA row m = (data row)*PARTS + part; lane (m = lane%16, kg = lane/16) holds elements
 // part*32 + 8*kg .. +7 of its data row.  The C registers i = 0..3 of a lane are MFMA rows 4*kg + i
 // of projection slot lane%16; the partial projections of one data row are summed afterwards.
-// Up to two tensors per launch (queries and keys of one forward): blockIdx.y counts the (batch, head)
-// sequences of the first tensor, then those of the second.
+// Up to two tensors per launch (queries and keys of one forward): blockIdx.y + blockIdx.z * gridDim.y counts
+// the (batch, head) sequences of the first tensor, then those of the second (a grid dimension holds 65535).
 struct HashTensors {
   const void* x[2];
   void* out[2];        // bucket ids, (batch, heads, n) contiguous, int32 or (OUT8) one byte each
   int64_t sb[2], sh[2], sn[2];
   int heads[2];
   int seqs0;           // batch * heads of the first tensor
+  int seqs;            // sequences of both tensors together
 };
 
 template <typename T, int D, bool OUT8>
@@ -58,8 +59,10 @@ __global__ __launch_bounds__(256) void lsh_hash_mfma_kernel(const HashTensors te
   constexpr int ROWS = 16 / PARTS;            // data rows per tile
   constexpr int NS = PARTS >= 4 ? 1 : 4 / PARTS;  // data rows per lane (sums of C registers)
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int which = (int)blockIdx.y >= ten.seqs0 ? 1 : 0;
-  const int bh = (int)blockIdx.y - (which ? ten.seqs0 : 0);
+  const int seq = (int)(blockIdx.y + blockIdx.z * gridDim.y);
+  if (seq >= ten.seqs) return;  // the last layer of the grid may be partly empty
+  const int which = seq >= ten.seqs0 ? 1 : 0;
+  const int bh = seq - (which ? ten.seqs0 : 0);
   const int heads = ten.heads[which];
   const int b = bh / heads, h = bh % heads;
   const T* xbase = (const T*)ten.x[which] + b * ten.sb[which] + h * ten.sh[which];
@@ -185,10 +188,12 @@ __global__ __launch_bounds__(256) void lsh_hash_mfma_kernel(const HashTensors te
 }
 
 template <typename T, int D, bool OUT8>
-int launch_hash_mfma(const HashTensors& ten, int64_t seqs, const void* proj, int64_t n, int64_t r, int64_t psb, int64_t psh,
+int launch_hash_mfma(HashTensors ten, int64_t seqs, const void* proj, int64_t n, int64_t r, int64_t psb, int64_t psh,
                      int64_t d_real, hipStream_t stream) {
   const int64_t rows_per_block = 4 * HASH_TILES_PER_WAVE * (16 / (D / 32));
-  dim3 grid((unsigned)((n + rows_per_block - 1) / rows_per_block), (unsigned)seqs);
+  ten.seqs = (int)seqs;
+  const int64_t gy = seqs < 32768 ? seqs : 32768, gz = (seqs + gy - 1) / gy;
+  dim3 grid((unsigned)((n + rows_per_block - 1) / rows_per_block), (unsigned)gy, (unsigned)gz);
   hipLaunchKernelGGL((lsh_hash_mfma_kernel<T, D, OUT8>), grid, dim3(256), 0, stream, ten, (const T*)proj, n, (int)r, psb, psh,
                      (int)d_real);
   return ha_launch_status("ha_lsh_hash");
@@ -203,7 +208,7 @@ extern "C" int ha_lsh_hash(const void* x, const void* proj, int32_t* buckets, in
   HA_REQUIRE(x && proj && buckets, HA_ERR_NULL, "ha_lsh_hash: null pointer");
   HA_REQUIRE(dtype == HA_F16 || dtype == HA_BF16, HA_ERR_DTYPE, "ha_lsh_hash: Only support fp16 and bf16");
   HA_REQUIRE(batch > 0 && heads > 0 && n > 0, HA_ERR_SHAPE, "ha_lsh_hash: batch, heads, n must be positive");
-  HA_REQUIRE(batch * heads <= 65535, HA_ERR_SHAPE, "ha_lsh_hash: batch*heads must be <= 65535");
+  HA_REQUIRE(batch * heads < (1ll << 30), HA_ERR_SHAPE, "ha_lsh_hash: batch*heads must be below 2^30");
   HA_REQUIRE(r >= 1, HA_ERR_SHAPE, "ha_lsh_hash: Invalid value for num_projs");
   HA_REQUIRE(r <= 16, HA_ERR_UNSUPPORTED, "ha_lsh_hash: num_projs > 16 is not supported");
   HA_REQUIRE(d >= 8 && d <= 256 && d % 8 == 0, HA_ERR_HEADDIM, "ha_lsh_hash: d must be a multiple of 8 in [8, 256]");
@@ -233,7 +238,7 @@ int ha_hash_pair_u8(const void* q, const void* k, const void* proj, uint8_t* ids
                     int64_t heads, int64_t kv_heads, int64_t n, int64_t d, int64_t r, const int64_t (&q_strides)[3],
                     const int64_t (&k_strides)[3], int dtype, hipStream_t stream) {
   HA_REQUIRE(r >= 1 && r <= 8, HA_ERR_UNSUPPORTED, "ha_forward: byte-sized bucket ids need at most 8 projections");
-  HA_REQUIRE(batch * (heads + kv_heads) <= 65535, HA_ERR_SHAPE, "ha_forward: batch*(heads + kv_heads) must be <= 65535");
+  HA_REQUIRE(batch * (heads + kv_heads) < (1ll << 30), HA_ERR_SHAPE, "ha_forward: batch*(heads + kv_heads) must be below 2^30");
   HashTensors ten = {};
   ten.x[0] = q; ten.x[1] = k; ten.out[0] = ids_q; ten.out[1] = ids_k;
   ten.sb[0] = q_strides[0]; ten.sh[0] = q_strides[1]; ten.sn[0] = q_strides[2];

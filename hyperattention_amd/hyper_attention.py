@@ -204,7 +204,7 @@ class HyperAttention(torch.nn.Module):
         self.sampled_idx = kwargs.get('sampled_idx')
         self.residual_estimator = bool(kwargs.get('residual_estimator', False))
         # workspace of the one-call forward, one per (device, stream), kept between calls
-        self._workspace = {}
+        self._workspace = ops.WorkspaceCache()
 
     def forward(self, query: torch.tensor, key: torch.tensor, value: torch.tensor, scale=None, causal=False,
                 return_lse=False):

@@ -138,18 +138,29 @@ def padded_head_dim(d):
     return 64 if d <= 64 else 128
 
 
+_SAMPLED_BOUNDS = {}  # bounds of explicit sample lists already looked at
+
+
 def check_sampled_idx(sampled_idx, n_k: int):
     """An explicit sample list names key rows of the call it is used in: every entry must lie in
     [0, n_k).  Inside the causal recursion the same list serves every level, so n_k is the key length of
     the smallest hashed level; a larger entry would read keys of the second half there (future tokens)
-    or past the tensor.  The bounds of a list are computed once per tensor version."""
+    or past the tensor.  The bounds of a list are computed once per tensor version (a host read of a device
+    tensor: pass the list once before capturing a graph)."""
     if sampled_idx is None:
         return
-    cached = getattr(sampled_idx, "_ha_bounds", None)
-    if cached is None or cached[0] != sampled_idx._version:
+    # keyed by the tensor's identity, storage and version; an inference tensor has no version counter and is
+    # checked on every call
+    version = None if sampled_idx.is_inference() else sampled_idx._version
+    key = (id(sampled_idx), sampled_idx.data_ptr(), tuple(sampled_idx.shape), version)
+    cached = _SAMPLED_BOUNDS.get(key) if version is not None else None
+    if cached is None:
         lo, hi = (int(sampled_idx.min()), int(sampled_idx.max())) if sampled_idx.numel() else (0, -1)
-        cached = (sampled_idx._version, lo, hi)
-        sampled_idx._ha_bounds = cached
+        cached = (version, lo, hi)
+        if version is not None:
+            if len(_SAMPLED_BOUNDS) > 64:
+                _SAMPLED_BOUNDS.clear()
+            _SAMPLED_BOUNDS[key] = cached
     assert cached[1] >= 0 and cached[2] < n_k, \
         f"sampled_idx must lie in [0, {n_k}) (the key length of the shortest hashed call); got [{cached[1]}, {cached[2]}]"
 
@@ -437,6 +448,40 @@ class FlashAttnFunc(torch.autograd.Function):
 
 
 # ------------------------------------------------------------------------- whole forward pass
+class WorkspaceCache:
+    """Workspaces of the one-call forward kept between calls: one tensor per (device, stream), grown when a
+    larger shape arrives, and the sizes the library asked for per shape.
+
+    Under stream capture the cache is bypassed: a captured call gets a fresh tensor from the capturing graph's
+    own memory pool (two graphs captured on one stream must not share a workspace: their replays may overlap).
+    A tensor that is replaced by a larger one is kept alive in `retired`, because a graph captured earlier, or
+    work still queued on the stream, may point at it.  The cache is not part of a module's state: copies and
+    pickles of it start empty."""
+
+    def __init__(self):
+        self.sizes = {}
+        self.slots = {}
+        self.retired = []
+
+    def tensor(self, device, stream, nbytes, capturing=False):
+        if capturing:
+            return torch.empty(int(nbytes), device=device, dtype=torch.uint8)
+        slot = (device.index, stream)
+        ws = self.slots.get(slot)
+        if ws is None or ws.numel() < int(nbytes):
+            if ws is not None:
+                self.retired.append(ws)
+            ws = torch.empty(int(nbytes), device=device, dtype=torch.uint8)
+            self.slots[slot] = ws
+        return ws
+
+    def __deepcopy__(self, memo):
+        return WorkspaceCache()
+
+    def __reduce__(self):
+        return (WorkspaceCache, ())
+
+
 def forward_plan_supported(n: int, min_seq_len: int, causal: bool, lsh_num_projs: int) -> bool:
     """True when ha_forward covers this shape: every causal recursion level has an even length."""
     if lsh_num_projs > 16:
@@ -453,9 +498,9 @@ def forward_plan_supported(n: int, min_seq_len: int, causal: bool, lsh_num_projs
 def _forward_args(q, k, v, out, lse, proj, *, scale, causal, lsh_num_projs, block_size, sample_size, min_seq_len,
                   smooth_block, sampled_idx=None, workspace=None, stream=None):
     """ForwardArgs for (b,h,n,d) q and (b,h_kv,n,d) k, v with its workspace attached; the second result keeps
-    the tensors alive that the struct only points to (the workspace last).  `workspace`: a dict the caller
-    owns; the workspace tensor of the current (device, stream) and the sizes the library asked for are kept
-    there and reused, so that a caller that runs many forwards neither allocates nor asks per call.
+    the tensors alive that the struct only points to (the workspace last).  `workspace`: a WorkspaceCache the
+    caller owns; the workspace tensor of the current (device, stream) and the sizes the library asked for are
+    kept there and reused, so that a caller that runs many forwards neither allocates nor asks per call.
     `stream`: the raw handle of the current stream, if the caller has it already."""
     assert q.is_cuda and k.is_cuda
     assert q.stride(-1) == 1 and k.stride(-1) == 1 and (v is None or v.stride(-1) == 1)
@@ -491,23 +536,19 @@ def _forward_args(q, k, v, out, lse, proj, *, scale, causal, lsh_num_projs, bloc
     if v is not None:
         a.v_stride_b, a.v_stride_h, a.v_stride_n = v.stride(0), v.stride(1), v.stride(2)
     shape_key = (b, h, hk, n, d, a.dv, lsh_num_projs, min_seq_len, a.causal)
-    ws_bytes = workspace.get(shape_key) if workspace is not None else None
+    ws_bytes = workspace.sizes.get(shape_key) if workspace is not None else None
     if ws_bytes is None:
         ws_bytes = _lib.lib().ha_forward_workspace_bytes(ctypes.byref(a))
         if ws_bytes < 0:
             _lib.check(int(ws_bytes))
         if workspace is not None:
-            workspace[shape_key] = ws_bytes
-    ws = None
+            workspace.sizes[shape_key] = ws_bytes
     if workspace is not None:
         if stream is None:
             stream = torch.cuda.current_stream(q.device).cuda_stream
-        slot = (q.device.index, stream)
-        ws = workspace.get(slot)
-    if ws is None or ws.numel() < int(ws_bytes):
+        ws = workspace.tensor(q.device, stream, ws_bytes, capturing=torch.cuda.is_current_stream_capturing())
+    else:
         ws = torch.empty(int(ws_bytes), device=q.device, dtype=torch.uint8)
-        if workspace is not None:
-            workspace[slot] = ws
     a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
     keep.append(ws)
     return a, keep

@@ -78,7 +78,9 @@ int ha_bucket_argsort(const int32_t* keys, void* idx_out, int idx_type,
  * array of HA_SORT_SCRATCH_BYTES inside the library (one copy per GPU, held until the process ends); a
  * sort whose ha_bucket_argsort_workspace_bytes() exceeds it is rejected with HA_ERR_WORKSPACE.  The
  * device of the call is the current device.  All calls on one GPU share the array: calls that overlap
- * on one GPU (different streams or threads) race and must be serialised by the caller.
+ * on one GPU (different streams or threads) race and must be serialised by the caller.  The first call on a
+ * device looks up the array's address and must be made outside stream capture (HA_ERR_UNSUPPORTED
+ * otherwise): call it once before capturing.
  */
 #define HA_SORT_SCRATCH_BYTES (8 << 20)
 int ha_bucket_argsort_static(const int32_t* keys, void* idx_out, int idx_type,

@@ -262,3 +262,46 @@ def test_explicit_sample_lists_are_range_checked_on_the_host():
     lse = torch.zeros((1, 1, 256))
     with pytest.raises(AssertionError, match="sampled_idx must lie in"):
         ops._block_attn_args(q, q, q, q, lse, idx, idx, 128, 128, 0.125, False, torch.arange(200, 328))
+
+
+def test_workspace_cache_policy():
+    """The forward's workspace cache: one tensor per (device, stream) that only grows, a replaced tensor
+    stays alive (a captured graph or queued work may point at it), a call under stream capture never shares
+    or caches, and copies / pickles of a module start with an empty cache."""
+    import copy
+    import pickle
+    import torch
+    from hyperattention_amd import HyperAttention, ops
+    c = ops.WorkspaceCache()
+    cpu = torch.device("cpu")
+    a = c.tensor(cpu, 0, 1000)
+    assert a.numel() == 1000 and c.tensor(cpu, 0, 500) is a          # reused while it is large enough
+    b = c.tensor(cpu, 0, 4000)
+    assert b is not a and b.numel() == 4000 and any(t is a for t in c.retired)
+    other_stream = c.tensor(cpu, 1, 100)
+    assert other_stream is not b and c.tensor(cpu, 0, 100) is b      # one slot per stream
+    g1, g2 = c.tensor(cpu, 0, 100, capturing=True), c.tensor(cpu, 0, 100, capturing=True)
+    assert g1 is not g2 and g1 is not b and c.tensor(cpu, 0, 100) is b
+    c.sizes[("shape",)] = 123
+    for clone in (copy.deepcopy(c), pickle.loads(pickle.dumps(c))):
+        assert clone.slots == {} and clone.sizes == {} and clone.retired == []
+    m = HyperAttention(input_dim=64)
+    m._workspace.tensor(cpu, 0, 64)
+    m2 = copy.deepcopy(m)
+    assert m2._workspace.slots == {} and torch.equal(m2.lsh.proj_dir, m.lsh.proj_dir)
+    import io
+    buf = io.BytesIO()
+    torch.save(m, buf)
+    assert len(buf.getvalue()) < 100000
+
+
+def test_sampled_idx_bounds_of_an_inference_tensor():
+    """A sample list created under inference mode has no version counter: it is checked without one."""
+    import torch
+    from hyperattention_amd import ops
+    with torch.inference_mode():
+        idx = torch.arange(0, 128)
+    ops.check_sampled_idx(idx, 128)
+    with pytest.raises(AssertionError, match="sampled_idx must lie in"):
+        ops.check_sampled_idx(idx, 100)
+    assert not hasattr(idx, "_ha_bounds")

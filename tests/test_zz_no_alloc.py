@@ -23,12 +23,19 @@ def _sort_both(keys, seg_len, seg_stride, seg_offset, num_segments, num_keys, id
     _lib.check(L.ha_bucket_argsort(keys.data_ptr(), want.data_ptr(), code, num_segments, seg_len, seg_stride,
                                    seg_offset, num_keys, ws.data_ptr(), ws.numel(), stream))
     got = torch.full((num_segments, seg_len), -1, device=dev, dtype=idx_dtype)
+    # the first call on a device looks up the scratch array's address (and may make the runtime load it); from
+    # then on neither torch's allocator nor the driver (hipMemGetInfo) may see the device's memory change
+    _lib.check(L.ha_bucket_argsort_static(keys.data_ptr(), got.data_ptr(), code, num_segments, seg_len, seg_stride,
+                                          seg_offset, num_keys, stream))
+    got.fill_(-1)
     torch.cuda.synchronize()
     before = torch.cuda.memory_allocated(dev)
+    free_before = torch.cuda.mem_get_info(dev)[0]
     _lib.check(L.ha_bucket_argsort_static(keys.data_ptr(), got.data_ptr(), code, num_segments, seg_len, seg_stride,
                                           seg_offset, num_keys, stream))
     torch.cuda.synchronize()
     assert torch.cuda.memory_allocated(dev) == before
+    assert torch.cuda.mem_get_info(dev)[0] == free_before, "the driver saw an allocation during the call"
     return got.cpu().numpy(), want.cpu().numpy()
 
 
