@@ -92,10 +92,14 @@ void fill_params(const ha_attn_operands& t, ha_attn_kernel_params& p) {
   p.n_q = (int)t.n_q; p.n_k = (int)t.n_k;
   p.block_tiles = 1; p.sample_chunks = 0; p.smooth = 0; p.accumulate = 0; p.idx64 = 0;
   p.sampled_pos = nullptr; p.sample_bias_raw = 0.f;
+  p.n_q_last = (int)t.n_q;
+  p.rag_levels = -1; p.rag_split = 0; p.rag_n = 0;
+  for (int& c : p.rag_half) c = 0;
   p.scale_log2 = t.scale * LOG2E_F;
 }
 
-int block_attn(const ha_block_attn_args& a, hipStream_t stream) {
+// n_q_last: queries of the last segment of every head that exist (see ha_attn_kernel_params), or -1
+int block_attn(const ha_block_attn_args& a, hipStream_t stream, int64_t n_q_last = -1) {
   int st = ha_check_block_attn_args(a, "ha_block_attn_fwd");
   if (st != HA_OK) return st;
   ha_attn_kernel_params p;
@@ -109,6 +113,7 @@ int block_attn(const ha_block_attn_args& a, hipStream_t stream) {
   p.smooth = a.smooth_block != 0;
   p.accumulate = a.accumulate != 0;
   p.idx64 = a.idx_type == HA_IDX_I64;
+  if (n_q_last >= 0) p.n_q_last = (int)n_q_last;
   const bool reweight = a.sample_bias != 0.f || a.mask_sampled_in_block != 0;
   if (reweight) {
     HA_REQUIRE(isfinite(a.sample_bias), HA_ERR_SHAPE, "ha_block_attn_fwd: sample_bias must be finite");
@@ -122,29 +127,49 @@ int block_attn(const ha_block_attn_args& a, hipStream_t stream) {
   return ha_attn_launch(p, (int)a.t.d, (int)a.t.dv, a.t.dtype, true, false, reweight, stream);
 }
 
-int flash_attn(const ha_attn_operands& t, int causal, int accumulate, hipStream_t stream) {
+// Ragged segments of an exact launch inside a causal recursion with odd lengths (see ha_attn_kernel_params)
+struct Ragged {
+  int levels, split, n;
+  int half[HA_MAX_RAGGED_LEVELS + 1];
+};
+
+int flash_attn(const ha_attn_operands& t, int causal, int accumulate, hipStream_t stream, const Ragged* rag = nullptr) {
   int st = ha_check_operands(t, "ha_flash_attn_fwd");
   if (st != HA_OK) return st;
   ha_attn_kernel_params p;
   fill_params(t, p);
   p.accumulate = accumulate != 0;
+  if (rag) {
+    p.rag_levels = rag->levels; p.rag_split = rag->split; p.rag_n = rag->n;
+    for (int i = 0; i <= HA_MAX_RAGGED_LEVELS; ++i) p.rag_half[i] = rag->half[i];
+  }
   return ha_attn_launch(p, (int)t.d, (int)t.dv, t.dtype, false, causal != 0, false, stream);
 }
 
 inline int64_t align256(int64_t v) { return (v + 255) & ~(int64_t)255; }
 
-// Static shape of the causal divide-and-conquer (hyper_attention.py:51-96): lengths per level.
+// Static shape of the causal divide-and-conquer (hyper_attention.py:51-96).  A virtual head of odd length
+// gets a zero row appended before it is cut in two (:61-64), so lengths are counted with those rows: len[j]
+// is the length of a level-j virtual head as the recursion sees it, half[j] = ceil(len[j] / 2) the length of
+// its two halves.  Appended rows sit at the end of their virtual head, and so of every last descendant.
 struct Plan {
-  int levels;          // number of halvings
-  int64_t len[48];     // len[j] = sequence length of a virtual head at level j; len[levels] = leaf
+  int levels;            // number of halvings
+  int64_t len[48];       // len[levels] = leaf
+  int64_t half[48];
   bool level_hyper[48];  // off-diagonal of level j uses the hashed kernel (else exact, hyper_attention.py:109)
   bool any_hyper;
+  bool ragged;           // an odd length somewhere
+  int64_t n_hashed;      // rows per head as the hashed levels see them: n, plus the appended row of an odd n
+  int64_t granule;       // length of the shortest hashed half (n_hashed is a multiple of it)
 };
 
 int make_plan(const ha_forward_args& a, Plan& pl) {
   pl.levels = 0;
   pl.any_hyper = false;
+  pl.ragged = false;
   pl.len[0] = a.n;
+  pl.n_hashed = a.n;
+  pl.granule = a.n;
   if (!a.causal) {
     pl.level_hyper[0] = !(a.min_seq_len > a.n);  // hyper_attention.py:109
     pl.any_hyper = pl.level_hyper[0];
@@ -155,23 +180,29 @@ int make_plan(const ha_forward_args& a, Plan& pl) {
     }
     return HA_OK;
   }
+  // Only n itself can be odd: a level whose halves are hashed has halves of a multiple of 128 rows, and a
+  // level whose halves are shorter than min_seq_len is the last one.
   while (pl.len[pl.levels] > a.min_seq_len) {  // hyper_attention.py:52
-    const int64_t cur = pl.len[pl.levels];
-    HA_REQUIRE(cur % 2 == 0, HA_ERR_UNSUPPORTED,
-               "ha_forward: odd length %lld inside the causal recursion; compose this shape from the operators",
-               (long long)cur);
-    const int64_t half = cur / 2;
-    pl.level_hyper[pl.levels] = !(a.min_seq_len > half);
-    if (pl.level_hyper[pl.levels]) {
+    const int j = pl.levels;
+    const int64_t cur = pl.len[j];
+    pl.ragged = pl.ragged || (cur & 1);
+    const int64_t half = (cur + 1) / 2;
+    pl.half[j] = half;
+    pl.level_hyper[j] = !(a.min_seq_len > half);
+    if (pl.level_hyper[j]) {
       HA_REQUIRE(half % 128 == 0, HA_ERR_SHAPE, "ha_forward: keys sequence length must be divisible by 128");
       HA_REQUIRE(a.sampled_idx || a.sample_size <= half, HA_ERR_SHAPE,
                  "ha_forward: default sampled rows 0..sample_size-1 exceed the key length %lld of a level",
                  (long long)half);
       pl.any_hyper = true;
+      pl.granule = half;
     }
     pl.len[++pl.levels] = half;
-    HA_REQUIRE(pl.levels < 40, HA_ERR_SHAPE, "ha_forward: recursion too deep");
+    HA_REQUIRE(pl.levels < HA_MAX_RAGGED_LEVELS, HA_ERR_SHAPE, "ha_forward: recursion too deep");
   }
+  // a hashed half is a multiple of 128, so every hashed level but the first has an even length: the hashed
+  // levels see the sequence with at most one appended row, the one of an odd n
+  if (pl.any_hyper) pl.n_hashed = a.n + (a.n & 1);
   return HA_OK;
 }
 
@@ -195,31 +226,32 @@ void layout_workspace(const ha_forward_args& a, const Plan& pl, Workspace& w) {
   int64_t off = 0;
   memset(&w, 0, sizeof(w));
   const int nlev = a.causal ? pl.levels : 1;
+  const int64_t nh = pl.n_hashed;  // rows per head as the hashed levels see them
   if (pl.any_hyper) {
     ha_unit_grid& g = w.grid;
-    g.n = a.n;
-    g.granule = a.causal ? pl.len[pl.levels] : a.n;
+    g.n = nh;
+    g.granule = pl.granule;
     g.units_per_granule = (int)((g.granule + HA_SORT_CHUNK - 1) / HA_SORT_CHUNK);
     g.unit = (int)std::min<int64_t>(g.granule, HA_SORT_CHUNK);
-    g.units_per_seq = (int)(a.n / g.granule) * g.units_per_granule;
+    g.units_per_seq = (int)(nh / g.granule) * g.units_per_granule;
     int64_t longest = 0;
     for (int j = 0; j < nlev; ++j)
-      if (pl.level_hyper[j]) longest = std::max<int64_t>(longest, a.causal ? pl.len[j] / 2 : a.n);
+      if (pl.level_hyper[j]) longest = std::max<int64_t>(longest, a.causal ? pl.half[j] : a.n);
     w.units = a.lsh_num_projs <= 8 && longest / g.granule * g.units_per_granule <= max_units_per_segment(g.unit) &&
-              a.n % g.granule == 0;
+              nh % g.granule == 0;
     const int64_t id_bytes = w.units ? 1 : 4;
-    w.buckets_q = off; off += align256(a.batch * a.heads * a.n * id_bytes);
-    w.buckets_k = off; off += align256(a.batch * a.kv_heads * a.n * id_bytes);
+    w.buckets_q = off; off += align256(a.batch * a.heads * nh * id_bytes);
+    w.buckets_k = off; off += align256(a.batch * a.kv_heads * nh * id_bytes);
     if (w.units) {
-      w.sorted_q = off; off += align256(a.batch * a.heads * a.n * 4);
-      w.sorted_k = off; off += align256(a.batch * a.kv_heads * a.n * 4);
+      w.sorted_q = off; off += align256(a.batch * a.heads * nh * 4);
+      w.sorted_k = off; off += align256(a.batch * a.kv_heads * nh * 4);
       w.unit_hist_q = off; off += align256(a.batch * a.heads * g.units_per_seq * 256 * 4);
       w.unit_hist_k = off; off += align256(a.batch * a.kv_heads * g.units_per_seq * 256 * 4);
     }
   }
   for (int j = 0; j < nlev; ++j) {
     if (!pl.level_hyper[j]) continue;
-    const int64_t seg_len = a.causal ? pl.len[j] / 2 : a.n;
+    const int64_t seg_len = a.causal ? pl.half[j] : a.n;
     const int64_t segs = a.causal ? (1ll << j) : 1;
     const int64_t chunks = (seg_len + HA_SORT_CHUNK - 1) / HA_SORT_CHUNK;
     w.qidx[j] = off; off += align256(a.batch * a.heads * segs * seg_len * 4);
@@ -297,8 +329,8 @@ int hash_and_sort(const ha_forward_args& a, const Plan& pl, const Workspace& w, 
   int st;
   if (w.units) {
     const int64_t qs[3] = {t.q_stride_b, t.q_stride_h, t.q_stride_n}, ks[3] = {t.k_stride_b, t.k_stride_h, t.k_stride_n};
-    st = ha_hash_pair_u8(a.q, a.k, a.proj, ws + w.buckets_q, ws + w.buckets_k, a.batch, a.heads, a.kv_heads, a.n, a.d,
-                         a.lsh_num_projs, qs, ks, a.dtype, stream);
+    st = ha_hash_pair_u8(a.q, a.k, a.proj, ws + w.buckets_q, ws + w.buckets_k, a.batch, a.heads, a.kv_heads, pl.n_hashed,
+                         a.n, a.d, a.lsh_num_projs, qs, ks, a.dtype, stream);
     if (st != HA_OK) return st;
     const uint8_t* ids[2] = {ws + w.buckets_q, ws + w.buckets_k};
     uint32_t* sorted[2] = {(uint32_t*)(ws + w.sorted_q), (uint32_t*)(ws + w.sorted_k)};
@@ -312,7 +344,7 @@ int hash_and_sort(const ha_forward_args& a, const Plan& pl, const Workspace& w, 
     int64_t blocks = 0;
     for (int j = 0; j < nlev; ++j) {
       if (!pl.level_hyper[j]) continue;
-      const int64_t seg_len = a.causal ? pl.len[j] / 2 : a.n;
+      const int64_t seg_len = a.causal ? pl.half[j] : a.n;
       const int64_t segs = a.causal ? (1ll << j) : 1;
       for (int side = 0; side < 2; ++side) {
         HA_REQUIRE(jobs.num_jobs < HA_SORT_MAX_JOBS, HA_ERR_SHAPE, "ha_forward: too many sort jobs");
@@ -320,7 +352,7 @@ int hash_and_sort(const ha_forward_args& a, const Plan& pl, const Workspace& w, 
         job.sorted = sorted[side];
         job.hist = hist[side];
         job.out = (int32_t*)(ws + (side == 0 ? w.qidx[j] : w.kidx[j]));
-        job.seg_stride = a.causal ? pl.len[j] : a.n;
+        job.seg_stride = a.causal ? 2 * seg_len : a.n;
         job.seg_offset = (a.causal && side == 0) ? seg_len : 0;  // queries: second halves, keys: first halves
         job.seg_len = (int)seg_len;
         job.segs_per_seq = (int)segs;
@@ -335,10 +367,10 @@ int hash_and_sort(const ha_forward_args& a, const Plan& pl, const Workspace& w, 
 
   int32_t* bq = (int32_t*)(ws + w.buckets_q);
   int32_t* bk = (int32_t*)(ws + w.buckets_k);
-  st = ha_lsh_hash(a.q, a.proj, bq, a.batch, a.heads, a.n, a.d, a.lsh_num_projs, t.q_stride_b, t.q_stride_h,
+  st = ha_hash_i32(a.q, a.proj, bq, a.batch, a.heads, pl.n_hashed, a.n, a.d, a.lsh_num_projs, t.q_stride_b, t.q_stride_h,
                    t.q_stride_n, 0, 0, a.dtype, stream);
   if (st != HA_OK) return st;
-  st = ha_lsh_hash(a.k, a.proj, bk, a.batch, a.kv_heads, a.n, a.d, a.lsh_num_projs, t.k_stride_b, t.k_stride_h,
+  st = ha_hash_i32(a.k, a.proj, bk, a.batch, a.kv_heads, pl.n_hashed, a.n, a.d, a.lsh_num_projs, t.k_stride_b, t.k_stride_h,
                    t.k_stride_n, 0, 0, a.dtype, stream);
   if (st != HA_OK) return st;
   // all segmented sorts of all levels in one batch of launches per 8-bit digit
@@ -353,9 +385,9 @@ int hash_and_sort(const ha_forward_args& a, const Plan& pl, const Workspace& w, 
     bool multi = false;
     for (int j = 0; j < nlev; ++j) {
       if (!pl.level_hyper[j]) continue;
-      const int64_t seg_len = a.causal ? pl.len[j] / 2 : a.n;
+      const int64_t seg_len = a.causal ? pl.half[j] : a.n;
       const int64_t segs = a.causal ? (1ll << j) : 1;
-      const int64_t stride = a.causal ? pl.len[j] : a.n;
+      const int64_t stride = a.causal ? 2 * seg_len : a.n;
       const int64_t chunks = (seg_len + HA_SORT_CHUNK - 1) / HA_SORT_CHUNK;
       for (int side = 0; side < 2; ++side) {
         HA_REQUIRE(jobs.num_jobs < HA_SORT_MAX_JOBS, HA_ERR_SHAPE, "ha_forward: too many sort jobs");
@@ -485,13 +517,13 @@ extern "C" int ha_forward(const ha_forward_args* args, void* stream_) {
   }
 
   auto hyper_level = [&](int j, bool accumulate) -> int {
-    const int64_t seg_len = a.causal ? pl.len[j] / 2 : a.n;
+    const int64_t seg_len = a.causal ? pl.half[j] : a.n;
     const int64_t segs = a.causal ? (1ll << j) : 1;
     ha_block_attn_args b = {};
     b.t = t;
     b.t.n_q = b.t.n_k = seg_len;
     b.t.segs = segs;
-    b.t.seg_stride_rows = a.causal ? pl.len[j] : a.n;
+    b.t.seg_stride_rows = a.causal ? 2 * seg_len : a.n;
     b.t.q_seg_offset = a.causal ? seg_len : 0;
     b.t.k_seg_offset = 0;
     b.q_idx = ws + w.qidx[j];
@@ -505,7 +537,9 @@ extern "C" int ha_forward(const ha_forward_args* args, void* stream_) {
     b.sample_size = a.sample_size;
     b.smooth_block = a.smooth_block;
     b.accumulate = accumulate;
-    return block_attn(b, stream);
+    // an odd n: the last query of the last segment is the appended zero row; it is placed by its bucket like
+    // any other row and its result is dropped
+    return block_attn(b, stream, seg_len - (pl.n_hashed - a.n));
   };
 
   if (!a.causal) {
@@ -516,29 +550,32 @@ extern "C" int ha_forward(const ha_forward_args* args, void* stream_) {
     return flash_attn(f, 0, 0, stream);
   }
 
-  // 3. leaves: exact causal attention on every segment of the deepest level
-  {
+  // Exact launches over the segments of level `level` (leaves: level == pl.levels, whole segments with the
+  // causal mask; else the off-diagonal part of that level: second halves against first halves).  With an odd
+  // length somewhere the segments are ragged: the kernel finds each segment's rows from the plan.
+  auto exact_level = [&](int level, bool leaves) -> int {
     ha_attn_operands f = t;
-    f.n_q = f.n_k = pl.len[pl.levels];
-    f.segs = 1ll << pl.levels;
-    f.seg_stride_rows = pl.len[pl.levels];
-    f.q_seg_offset = f.k_seg_offset = 0;
-    st = flash_attn(f, 1, 0, stream);
-    if (st != HA_OK) return st;
-  }
+    const int64_t rows = leaves ? pl.len[level] : pl.half[level];
+    f.n_q = f.n_k = rows;
+    f.segs = 1ll << level;
+    f.seg_stride_rows = leaves ? rows : 2 * rows;
+    f.q_seg_offset = leaves ? 0 : rows;
+    f.k_seg_offset = 0;
+    if (!pl.ragged) return flash_attn(f, leaves ? 1 : 0, leaves ? 0 : 1, stream);
+    Ragged rag = {};
+    rag.levels = level;
+    rag.split = leaves ? 0 : 1;
+    rag.n = (int)a.n;
+    for (int i = 0; i <= level && i < pl.levels; ++i) rag.half[i] = (int)pl.half[i];
+    return flash_attn(f, leaves ? 1 : 0, leaves ? 0 : 1, stream, &rag);
+  };
+
+  // 3. leaves: exact causal attention on every segment of the deepest level
+  st = exact_level(pl.levels, true);
+  if (st != HA_OK) return st;
   // 4. off-diagonal parts, deepest level first, merged in place into the second halves
   for (int j = pl.levels - 1; j >= 0; --j) {
-    if (pl.level_hyper[j]) {
-      st = hyper_level(j, true);
-    } else {
-      ha_attn_operands f = t;
-      f.n_q = f.n_k = pl.len[j] / 2;
-      f.segs = 1ll << j;
-      f.seg_stride_rows = pl.len[j];
-      f.q_seg_offset = pl.len[j] / 2;
-      f.k_seg_offset = 0;
-      st = flash_attn(f, 0, 1, stream);
-    }
+    st = pl.level_hyper[j] ? hyper_level(j, true) : exact_level(j, false);
     if (st != HA_OK) return st;
   }
   return HA_OK;

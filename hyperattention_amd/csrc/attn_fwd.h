@@ -10,6 +10,8 @@ struct ha_divisor {
   int shift;
 };
 
+constexpr int HA_MAX_RAGGED_LEVELS = 30;
+
 struct ha_attn_kernel_params {
   const void* q;
   const void* k;
@@ -38,6 +40,18 @@ struct ha_attn_kernel_params {
   const int32_t* sampled_pos;  // sorted-order position of every sampled key; null: nothing is masked
   float sample_bias_raw;       // added to the raw q.k of a sampled key: bias / softmax scale
   float scale_log2;   // softmax scale * log2(e)
+  // Queries of the last segment of every head that exist (gathered kernel): an entry of its query order at or
+  // past this number names a row that is not there (the zero row the causal recursion appends to an odd
+  // length, hyper_attention.py:61-64); it is placed like any other row and its result is dropped.
+  int n_q_last;
+  // Ragged segments (exact kernels; rag_levels < 0: regular).  Inside a causal recursion with odd lengths the
+  // segments of a level neither start at multiples of one stride nor hold the same number of rows: level i
+  // cuts a segment of (padded) length 2*rag_half[i] into two, and the rows that exist are the first rag_n of
+  // the whole sequence.  Segment number `seg` has rag_levels bits, most significant first: bit i says which
+  // half of its level-i ancestor it lies in.  rag_split: the launch is the off-diagonal part of the level
+  // below (queries = second half, keys = first half of the segment, halves of rag_half[rag_levels] rows).
+  int rag_levels, rag_split, rag_n;
+  int rag_half[HA_MAX_RAGGED_LEVELS + 1];
   // the divisors of the workgroup -> (head, segment, tile) decomposition as multiply-and-shift
   // constants (filled by ha_attn_launch): the kernel never divides
   ha_divisor div_qtiles, div_segs, div_heads, div_kv_heads, div_kv_group, div_block_tiles;

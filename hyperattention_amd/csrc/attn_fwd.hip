@@ -288,18 +288,48 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
   const int b = fast_div(bhk, p.div_kv_heads), hk = bhk - b * fast_div(p.heads, p.div_kv_group);
   const int h = hk * p.kv_group + hg;
 
+  // ---- rows of this segment -----------------------------------------------------------------------
+  int n_q = p.n_q, n_k = p.n_k;
+  int64_t seg_q_row = p.q_seg_off + (int64_t)seg * p.seg_stride, seg_k_row = p.k_seg_off + (int64_t)seg * p.seg_stride;
+  if (!GATHER && p.rag_levels >= 0) {
+    // walk down from the whole sequence: where the segment starts and how many of its rows exist
+    int start = 0, real = p.rag_n;
+    for (int i = 0; i < p.rag_levels; ++i) {
+      const int c = p.rag_half[i];
+      if ((seg >> (p.rag_levels - 1 - i)) & 1) {
+        start += c;
+        real = max(real - c, 0);
+      } else {
+        real = min(real, c);
+      }
+    }
+    if (p.rag_split) {
+      const int c = p.rag_half[p.rag_levels];
+      seg_q_row = start + c;
+      seg_k_row = start;
+      n_q = min(max(real - c, 0), c);
+      n_k = min(real, c);
+    } else {
+      seg_q_row = seg_k_row = start;
+      n_q = n_k = real;
+    }
+  }
+  // gathered kernel: entries of the query order from this number on name a row that does not exist
+  const int q_rows_exist = (GATHER && seg == p.segs - 1) ? p.n_q_last : n_q;
+
   if constexpr (!PAIRED) {
     const int qt = slot;
+    if (qt * WG_QUERIES >= n_q) return;  // ragged launches: the grid is sized for the longest segment
 #include "attn_fwd_tile.inc"
   } else {
     // the long tile first.  No barrier between the two: the last iteration of a tile ends with one, and after
     // it a wave touches only its own part of the query region.
     const int t_long = qtiles - 1 - slot;
-    {
+    if (t_long * WG_QUERIES < n_q) {  // ragged launches: the grid is sized for the longest segment
       const int qt = t_long;
 #include "attn_fwd_tile.inc"
     }
-    if (slot != t_long) {  // an odd number of tiles: the middle one has no partner
+    if (slot != t_long && slot * WG_QUERIES < n_q) {  // an odd number of tiles: the middle one has no partner
       const int qt = slot;
 #include "attn_fwd_tile.inc"
     }

@@ -68,6 +68,11 @@ int ha_place_units(const ha_place_jobs& jobs, int total_blocks, hipStream_t stre
 
 // Bucket ids of the queries and keys of one forward pass as one byte each (at most 8 projections, one shared
 // projection matrix), one launch.  Strides: batch, head, row, in elements.  Defined in lsh_hash.hip.
+// Only the first n_read <= n rows of a sequence exist; the ids of the others are those of zero rows.
 int ha_hash_pair_u8(const void* q, const void* k, const void* proj, uint8_t* ids_q, uint8_t* ids_k, int64_t batch,
-                    int64_t heads, int64_t kv_heads, int64_t n, int64_t d, int64_t r, const int64_t (&q_strides)[3],
-                    const int64_t (&k_strides)[3], int dtype, hipStream_t stream);
+                    int64_t heads, int64_t kv_heads, int64_t n, int64_t n_read, int64_t d, int64_t r,
+                    const int64_t (&q_strides)[3], const int64_t (&k_strides)[3], int dtype, hipStream_t stream);
+// ha_lsh_hash (int32 ids) with the same n / n_read distinction
+int ha_hash_i32(const void* x, const void* proj, int32_t* buckets, int64_t batch, int64_t heads, int64_t n,
+                int64_t n_read, int64_t d, int64_t r, int64_t x_stride_b, int64_t x_stride_h, int64_t x_stride_n,
+                int64_t proj_stride_b, int64_t proj_stride_h, int dtype, hipStream_t stream);

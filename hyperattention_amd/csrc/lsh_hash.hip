@@ -49,6 +49,7 @@ struct HashTensors {
   int heads[2];
   int seqs0;           // batch * heads of the first tensor
   int seqs;            // sequences of both tensors together
+  int64_t n_read;      // rows of a sequence that exist; rows from there up to n hash as zero rows
 };
 
 template <typename T, int D, bool OUT8>
@@ -105,7 +106,7 @@ __global__ __launch_bounds__(256) void lsh_hash_mfma_kernel(const HashTensors te
     for (int u = 0; u < HASH_UNROLL; ++u) {
       const int64_t row = wave_row0 + (int64_t)(t0 + u) * ROWS + my_row;
       vec8 z = {};
-      if (row < n && my_part * 32 + 8 * kg < d_real) z = *reinterpret_cast<const vec8*>(xbase + row * sn + my_part * 32 + 8 * kg);
+      if (row < ten.n_read && my_part * 32 + 8 * kg < d_real) z = *reinterpret_cast<const vec8*>(xbase + row * sn + my_part * 32 + 8 * kg);
       xf[u] = z;
     }
 #pragma unroll
@@ -192,6 +193,7 @@ int launch_hash_mfma(HashTensors ten, int64_t seqs, const void* proj, int64_t n,
                      int64_t d_real, hipStream_t stream) {
   const int64_t rows_per_block = 4 * HASH_TILES_PER_WAVE * (16 / (D / 32));
   ten.seqs = (int)seqs;
+  if (ten.n_read <= 0 || ten.n_read > n) ten.n_read = n;
   const int64_t gy = seqs < 32768 ? seqs : 32768, gz = (seqs + gy - 1) / gy;
   dim3 grid((unsigned)((n + rows_per_block - 1) / rows_per_block), (unsigned)gy, (unsigned)gz);
   hipLaunchKernelGGL((lsh_hash_mfma_kernel<T, D, OUT8>), grid, dim3(256), 0, stream, ten, (const T*)proj, n, (int)r, psb, psh,
@@ -205,6 +207,15 @@ extern "C" int ha_lsh_hash(const void* x, const void* proj, int32_t* buckets, in
                            int64_t heads, int64_t n, int64_t d, int64_t r, int64_t x_stride_b,
                            int64_t x_stride_h, int64_t x_stride_n, int64_t proj_stride_b,
                            int64_t proj_stride_h, int dtype, void* stream) {
+  return ha_hash_i32(x, proj, buckets, batch, heads, n, n, d, r, x_stride_b, x_stride_h, x_stride_n, proj_stride_b,
+                     proj_stride_h, dtype, (hipStream_t)stream);
+}
+
+// ha_lsh_hash for sequences of which only the first n_read rows exist: the ids of rows n_read .. n-1 are those
+// of zero rows (the rows the causal recursion appends to odd lengths)
+int ha_hash_i32(const void* x, const void* proj, int32_t* buckets, int64_t batch, int64_t heads, int64_t n,
+                int64_t n_read, int64_t d, int64_t r, int64_t x_stride_b, int64_t x_stride_h, int64_t x_stride_n,
+                int64_t proj_stride_b, int64_t proj_stride_h, int dtype, hipStream_t stream) {
   HA_REQUIRE(x && proj && buckets, HA_ERR_NULL, "ha_lsh_hash: null pointer");
   HA_REQUIRE(dtype == HA_F16 || dtype == HA_BF16, HA_ERR_DTYPE, "ha_lsh_hash: Only support fp16 and bf16");
   HA_REQUIRE(batch > 0 && heads > 0 && n > 0, HA_ERR_SHAPE, "ha_lsh_hash: batch, heads, n must be positive");
@@ -214,12 +225,13 @@ extern "C" int ha_lsh_hash(const void* x, const void* proj, int32_t* buckets, in
   HA_REQUIRE(d >= 8 && d <= 256 && d % 8 == 0, HA_ERR_HEADDIM, "ha_lsh_hash: d must be a multiple of 8 in [8, 256]");
   HA_REQUIRE(x_stride_n % 8 == 0 && x_stride_h % 8 == 0 && x_stride_b % 8 == 0 && ((uintptr_t)x % 16) == 0,
              HA_ERR_SHAPE, "ha_lsh_hash: rows must be 16-byte aligned");
-  hipStream_t s = (hipStream_t)stream;
+  hipStream_t s = stream;
   HashTensors ten = {};
   ten.x[0] = x; ten.out[0] = buckets;
   ten.sb[0] = x_stride_b; ten.sh[0] = x_stride_h; ten.sn[0] = x_stride_n;
   ten.heads[0] = ten.heads[1] = (int)heads;
   ten.seqs0 = (int)(batch * heads);
+  ten.n_read = n_read;
   // built for rows of 32, 64, 128 and 256 elements; a shorter row runs in the next width
 #define HA_HASH_MFMA(DD)                                                                                              \
   if (d <= DD) {                                                                                                      \
@@ -233,10 +245,11 @@ extern "C" int ha_lsh_hash(const void* x, const void* proj, int32_t* buckets, in
 }
 
 // Bucket ids of the queries and keys of one forward pass as one byte each (r <= 8 projections, one shared
-// projection matrix), in one launch.  q: (batch, heads, n, d), k: (batch, kv_heads, n, d), d in {64, 128}.
+// projection matrix), in one launch.  q: (batch, heads, n_read, d), k: (batch, kv_heads, n_read, d), d in {64, 128};
+// ids: n >= n_read per sequence, the ids past n_read being those of zero rows.
 int ha_hash_pair_u8(const void* q, const void* k, const void* proj, uint8_t* ids_q, uint8_t* ids_k, int64_t batch,
-                    int64_t heads, int64_t kv_heads, int64_t n, int64_t d, int64_t r, const int64_t (&q_strides)[3],
-                    const int64_t (&k_strides)[3], int dtype, hipStream_t stream) {
+                    int64_t heads, int64_t kv_heads, int64_t n, int64_t n_read, int64_t d, int64_t r,
+                    const int64_t (&q_strides)[3], const int64_t (&k_strides)[3], int dtype, hipStream_t stream) {
   HA_REQUIRE(r >= 1 && r <= 8, HA_ERR_UNSUPPORTED, "ha_forward: byte-sized bucket ids need at most 8 projections");
   HA_REQUIRE(batch * (heads + kv_heads) < (1ll << 30), HA_ERR_SHAPE, "ha_forward: batch*(heads + kv_heads) must be below 2^30");
   HashTensors ten = {};
@@ -245,6 +258,7 @@ int ha_hash_pair_u8(const void* q, const void* k, const void* proj, uint8_t* ids
   ten.sb[1] = k_strides[0]; ten.sh[1] = k_strides[1]; ten.sn[1] = k_strides[2];
   ten.heads[0] = (int)heads; ten.heads[1] = (int)kv_heads;
   ten.seqs0 = (int)(batch * heads);
+  ten.n_read = n_read;
   const int64_t seqs = batch * (heads + kv_heads);
 #define HA_HASH_PAIR(DD)                                                                                  \
   if (d <= DD) {                                                                                          \

@@ -265,7 +265,7 @@ class HyperAttention(torch.nn.Module):
             else:
                 lse = lse.unsqueeze(-1)
         elif (causal is not False and n_key > self.min_seq_len and not self.residual_estimator
-              and ops.forward_plan_supported(n_key, self.min_seq_len, True, self.lsh_num_projs)):
+              and self.lsh_num_projs <= 16 and ops.forward_plan_even(n_key, self.min_seq_len)):
             # gradients wanted and every level has an even length: the recursion and its gradient on
             # segments of the whole tensors, grouped-query heads as they are
             attn, lse = _CausalRecursionFunc.apply(self, scale, query.contiguous(), key.contiguous(), value.contiguous(),

@@ -482,12 +482,26 @@ class WorkspaceCache:
         return (WorkspaceCache, ())
 
 
+def causal_plan(n: int, min_seq_len: int):
+    """Lengths of the causal recursion (hyper_attention.py:51-96): (halves, leaf).  halves[j] is the length of
+    the two halves a level-j virtual head is cut into, after the zero row an odd length gets appended
+    (:61-64); leaf the length the recursion stops at.  Only n itself can be odd in a shape the kernels take:
+    hashed halves are multiples of 128, and a level with shorter halves is the last."""
+    halves = []
+    while n > min_seq_len:
+        n = (n + 1) // 2
+        halves.append(n)
+    return halves, n
+
+
 def forward_plan_supported(n: int, min_seq_len: int, causal: bool, lsh_num_projs: int) -> bool:
-    """True when ha_forward covers this shape: every causal recursion level has an even length."""
-    if lsh_num_projs > 16:
-        return False
-    if not causal:
-        return True
+    """True when ha_forward covers this shape: any length, up to 16 projections."""
+    return lsh_num_projs <= 16
+
+
+def forward_plan_even(n: int, min_seq_len: int) -> bool:
+    """True when every level of the causal recursion has an even length (what the recursion under autograd,
+    which works on equal segments of the whole tensors, takes)."""
     while n > min_seq_len:
         if n % 2:
             return False
@@ -579,7 +593,8 @@ def forward_sort(q, k, proj, *, causal, lsh_num_projs, min_seq_len):
     """Bucket orders of every hashed level of the forward pass (ha_forward_sort): one hash launch for q and
     k, one ranking, one placement.  Returns (q_idx, k_idx): per level (0 = whole sequence) an int32 tensor
     (b, h * 2^level, half) / (b, h_kv * 2^level, half) of rows local to the level's query segment (second
-    halves) / key segment (first halves), or None where the level is exact.  The tensors are views of one
+    halves) / key segment (first halves), or None where the level is exact.  With an odd n the last query of
+    the last segment of every head is the zero row the recursion appends (it has no row in q).  The tensors are views of one
     workspace."""
     b, h, n, d = q.shape
     hk = k.shape[1]
@@ -592,13 +607,14 @@ def forward_sort(q, k, proj, *, causal, lsh_num_projs, min_seq_len):
     with torch.cuda.device(q.device):
         _lib.check(_lib.lib().ha_forward_sort(ctypes.byref(a), q_off, k_off, ctypes.byref(levels), _stream(q)))
     q_idx, k_idx = [], []
+    halves = causal_plan(n, min_seq_len)[0] if causal else [n]
     for j in range(levels.value):
         if q_off[j] < 0:
             q_idx.append(None)
             k_idx.append(None)
             continue
         segs = (1 << j) if causal else 1
-        half = (n >> (j + 1)) if causal else n
+        half = halves[j] if causal else n
         q_idx.append(ws[q_off[j]:q_off[j] + 4 * b * h * segs * half].view(torch.int32).view(b, h * segs, half))
         k_idx.append(ws[k_off[j]:k_off[j] + 4 * b * hk * segs * half].view(torch.int32).view(b, hk * segs, half))
     return q_idx, k_idx

@@ -155,8 +155,12 @@ def test_forward_plan_and_workspace(lib):
     f.lsh_num_projs = 17
     assert lib.ha_forward_workspace_bytes(ctypes.byref(f)) > 0   # sized; the call itself rejects more than 16 projections
     f.lsh_num_projs = 8
-    f.n = 4095  # an odd length above min_seq_len needs the padded copy: not a shape of the one-call entry point
-    assert lib.ha_forward_workspace_bytes(ctypes.byref(f)) == -5
+    f.n = 4096
+    ws_even = lib.ha_forward_workspace_bytes(ctypes.byref(f))
+    f.n = 4095  # an odd length: the hashed levels see the sequence with the appended zero row, 4096 rows
+    assert lib.ha_forward_workspace_bytes(ctypes.byref(f)) == ws_even > 0
+    f.n = 4097  # padded to 4098: halves of 2049 rows are hashed and must be a multiple of 128
+    assert lib.ha_forward_workspace_bytes(ctypes.byref(f)) == -3
     f.n = 131072 + 2  # the first halves (65537) are hashed and must be a multiple of 128
     assert lib.ha_forward_workspace_bytes(ctypes.byref(f)) == -3
     f.n, f.min_seq_len, f.sample_size = 2048, 128, 256  # the deepest hashed level has 128 keys < 256 default samples

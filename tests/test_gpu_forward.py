@@ -101,17 +101,52 @@ def test_causal_forward(ha, dtype, d, n, msl, block, sample):
         assert_close(lse, rl, "lse")
 
 
-def test_causal_odd_lengths_composed_path(ha):
-    # 2047 -> padded to 2048 -> halves of 1024: hashed off-diagonal, exact leaves.
-    # 1001 -> padded to 1002 -> halves of 501 < 600: exact off-diagonal (arbitrary length), exact leaves.
-    for n, msl in ((2047, 1024), (1001, 600)):
-        q, k, v = (_randn((1, 2, n, 64), s, torch.float16) for s in (140, 141, 142))
-        m, proj = _module(ha, 64, torch.float16, 143, block_size=256, sample_size=128, min_seq_len=msl)
-        attn, lse = m(q.cuda(), k.cuda(), v.cuda(), causal=True, return_lse=True)
-        ro, rl = _oracle(q, k, v, proj, m, True)
-        assert attn.shape == (1, 2, n, 64) and lse.shape == (1, 2, n, 1)
-        assert_close(attn, ro, "attn", torch.float16)
-        assert_close(lse, rl, "lse")
+def _no_composed_path(m, monkeypatch):
+    """the module may not fall back to the operator-by-operator recursion"""
+    def refuse(*a, **k):
+        raise AssertionError("the operator-by-operator recursion ran")
+    monkeypatch.setattr(m, "_forward_composed", refuse)
+
+
+@pytest.mark.parametrize("n,msl,block", [
+    (2047, 1024, 256),   # appended row -> 2048 -> halves of 1024: hashed off-diagonal part, exact leaves
+    (1001, 600, 256),    # -> 1002 -> halves of 501 < 600: exact off-diagonal part (any length), exact leaves
+    (4095, 512, 128),    # three hashed levels (2048, 1024, 512): the appended row is in the last segment of each
+    (1537, 1024, 128),   # -> 1538 -> halves of 769: exact, leaves of 769 and 768 rows
+])
+def test_causal_odd_lengths(ha, monkeypatch, n, msl, block):
+    """An odd length runs in the one-call forward (hyper_attention.py:61-64, 94-96): the zero row the reference
+    appends is hashed and placed like any other query of the hashed levels (its bucket shifts the blocks of
+    the rows behind it) and its result is dropped; the exact parts work on ragged segments."""
+    q, k, v = (_randn((1, 2, n, 64), s, torch.float16) for s in (140, 141, 142))
+    m, proj = _module(ha, 64, torch.float16, 143, block_size=block, sample_size=128, min_seq_len=msl)
+    _no_composed_path(m, monkeypatch)
+    attn, lse = m(q.cuda(), k.cuda(), v.cuda(), causal=True, return_lse=True)
+    ro, rl = _oracle(q, k, v, proj, m, True)
+    assert attn.shape == (1, 2, n, 64) and lse.shape == (1, 2, n, 1)
+    assert_close(attn, ro, "attn", torch.float16)
+    assert_close(lse, rl, "lse")
+
+
+def test_causal_odd_length_sort_places_the_appended_row(ha):
+    """The query order of every hashed level of an odd length is the stable bucket sort of the segment's rows
+    with the appended zero row (bucket of the zero vector: 0) as its last row."""
+    from hyperattention_amd import ops
+    n, msl = 4095, 512
+    q, k = (_randn((1, 2, n, 64), s, torch.float16).cuda() for s in (144, 145))
+    m, proj = _module(ha, 64, torch.float16, 146, min_seq_len=msl)
+    q_idx, k_idx = ops.forward_sort(q, k, m.lsh.proj_dir, causal=True, lsh_num_projs=8, min_seq_len=msl)
+    pad = lambda x: torch.nn.functional.pad(x, (0, 0, 0, 1))
+    bq = torch.from_numpy(np.asarray(O.lsh_hash(pad(q.cpu()).double(), proj.double()))).reshape(1, 2, n + 1)
+    bk = torch.from_numpy(np.asarray(O.lsh_hash(pad(k.cpu()).double(), proj.double()))).reshape(1, 2, n + 1)
+    assert int(bq[0, 0, n]) == 0
+    assert len(q_idx) == 3
+    for j, half in enumerate((2048, 1024, 512)):
+        segs = 1 << j
+        want_q = torch.sort(bq.reshape(1, 2 * segs, 2 * half)[:, :, half:], dim=2, stable=True)[1]
+        want_k = torch.sort(bk.reshape(1, 2 * segs, 2 * half)[:, :, :half], dim=2, stable=True)[1]
+        assert torch.equal(q_idx[j].cpu().long(), want_q), f"level {j} queries"
+        assert torch.equal(k_idx[j].cpu().long(), want_k), f"level {j} keys"
 
 
 def test_causal_composed_path_equals_fused_path(ha):
@@ -153,13 +188,15 @@ def test_module_other_head_dim(ha, causal, d, dv):
     assert_close(lse, rl, "lse")
 
 
-def test_grouped_query_on_the_composed_path(ha):
-    """An odd length takes the operator-by-operator recursion, which wants equal head counts
-    (hyper_attention.py:43,67-68): grouped-query k/v are expanded there."""
-    n, h, hk = 1001, 4, 2
+@pytest.mark.parametrize("n,msl", [(1001, 600), (2047, 512)])
+def test_grouped_query_with_an_odd_length(ha, monkeypatch, n, msl):
+    """Grouped-query k/v with an odd length: taken as they are by the one-call forward (the reference needs as
+    many k/v heads as q heads, hyper_attention.py:43,67-68: the oracle gets them expanded)."""
+    h, hk = 4, 2
     q = _randn((1, h, n, 64), 190, torch.float16)
     k, v = (_randn((1, hk, n, 64), s, torch.float16) for s in (191, 192))
-    m, proj = _module(ha, 64, torch.float16, 193, block_size=256, sample_size=128, min_seq_len=600)
+    m, proj = _module(ha, 64, torch.float16, 193, block_size=256, sample_size=128, min_seq_len=msl)
+    _no_composed_path(m, monkeypatch)
     attn, lse = m(q.cuda(), k.cuda(), v.cuda(), causal=True, return_lse=True)
     ro, rl = _oracle(q, k.repeat_interleave(2, dim=1), v.repeat_interleave(2, dim=1), proj, m, True)
     assert_close(attn, ro, "attn", torch.float16)
