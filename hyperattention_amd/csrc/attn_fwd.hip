@@ -5,8 +5,9 @@
 // bias "none" (src/flash_attn_triton.py:57-267); the resume-from-a-previous-partial-result mode
 // folds add_self_attentions (src/attn_utils.py:6-50) into the kernel.
 //
-// Work decomposition.  A workgroup of 4 waves owns 256 consecutive (sorted) query positions of one
-// (virtual) head; wave w owns 64 of them as two 32-wide MFMA column blocks.  Query rows and key
+// Work decomposition.  A workgroup owns 256 consecutive (sorted) query positions of one (virtual) head:
+// 4 waves of 64 queries (two 32-wide MFMA column blocks) at head dim 64, 8 waves of 32 queries at head
+// dim 128 (WaveShape below).  Query rows and key
 // rows go from HBM straight into LDS (global_load_lds, 16 bytes per lane, whole rows per
 // instruction, no staging registers), row-major with their 16-byte pieces XOR-swizzled by the row
 // number (the swizzle is applied on the source side: a lane fetches the piece that belongs in its
@@ -22,10 +23,11 @@
 // points its lanes at (key j, dv word w) receives V[key 0..3][dv base + i]: the V^T operand in
 // exactly the key order of the C registers.
 //
-// Software pipeline.  On this hardware a wave's MFMAs overlap only with vector instructions of the
-// SAME wave, so the loop body is a chain of straight-line blocks, one per half-step of 16 keys, and
+// Software pipeline.  The loop body is a chain of straight-line blocks, one per half-step of 16 keys, and
 // each block mixes three independent things: the exponentials of half-step u, the P.V MFMAs of
-// half-step u-1 and half of the S^T MFMAs of the next 32-key step.  Keys are streamed in tiles of 64
+// half-step u-1 and half of the S^T MFMAs of the next 32-key step, issued one MFMA and its share of the
+// vector work at a time (clustering the MFMAs of a block, with or without a raised wave priority, measured
+// 4 to 6 % slower); two waves per SIMD fill each other's gaps.  Keys are streamed in tiles of 64
 // rows; the K tiles are shifted by 32 keys against the V tiles (K tile c holds keys 64c-32..64c+31),
 // so the K rows read during an iteration all sit in one tile, which is read in that iteration only
 // and can be refilled in the next, and the V^T operands of a half-step are fetched one block ahead.
@@ -44,7 +46,6 @@
 
 namespace {
 
-constexpr int WG_THREADS = 256;
 constexpr int WG_QUERIES = 256;  // sorted query positions per workgroup
 constexpr int KC = 64;           // keys per LDS tile
 constexpr float HALF_SUM_LIMIT = 16384.f;  // 2^14: a lane's half-step sum below this has no fp16 overflow
@@ -54,10 +55,19 @@ constexpr float HALF_SUM_LIMIT = 16384.f;  // 2^14: a lane's half-step sum below
 // which takes that path once and sets the row's true exponent.
 constexpr float M_FLOOR = -1e30f;
 
-// Head dims whose kernel needs more than 256 registers keep the S^T accumulators in VGPRs by hand.
+// How a workgroup's 256 queries are split over its waves.  A wave's registers hold the output accumulators
+// of its queries (queries x head dim floats over 64 lanes), their query fragments and two S^T buffers: 64
+// queries per wave fit 256 registers at head dim 64, at head dim 128 only 32 do.  256 registers is what lets
+// two waves share a SIMD, and a wave on its own leaves the matrix pipe idle through every stretch of vector
+// work and every wait (one wave per SIMD with 64 queries and 512 registers ran the d = 128 loop at 1170
+// cycles per 16 keys where its MFMAs alone take 512).  So: 4 waves x 64 queries at d = 64 (two workgroups per
+// CU), 8 waves x 32 queries at d = 128 (one workgroup per CU, LDS-bound), two waves per SIMD either way.
 template <int D>
-struct S_IN_VGPR {
-  static constexpr bool value = D > 64;
+struct WaveShape {
+  static constexpr int NB = D <= 64 ? 2 : 1;        // 32-query MFMA column blocks per wave
+  static constexpr int QW = 32 * NB;                // queries per wave
+  static constexpr int WAVES = WG_QUERIES / QW;     // waves per workgroup
+  static constexpr int THREADS = 64 * WAVES;
 };
 
 // x / y for 0 <= x < 2^31 by the divisor's multiply-and-shift constants
@@ -74,11 +84,11 @@ struct LaneOffsets {
 // registers), rounded to T, and their sums.  m is the reference exponent (log2 units).
 // sums of the 8 values per query block of a half-step's P.  They go through the matrix pipe: v_dot2
 // does not overlap with the big MFMAs at all.
-template <typename T>
-__device__ __forceinline__ void half_step_sums(const typename ElemTraits<T>::vec8 (&pn)[2], float (&sum)[2]) {
+template <typename T, int NB>
+__device__ __forceinline__ void half_step_sums(const typename ElemTraits<T>::vec8 (&pn)[NB], float (&sum)[NB]) {
   typedef typename ElemTraits<T>::vec4 vec4;
 #pragma unroll
-  for (int nb = 0; nb < 2; ++nb) {
+  for (int nb = 0; nb < NB; ++nb) {
     const vec4 lo = __builtin_shufflevector(pn[nb], pn[nb], 0, 1, 2, 3);
     const vec4 hi = __builtin_shufflevector(pn[nb], pn[nb], 4, 5, 6, 7);
     f32x4 acc_sum = {0.f, 0.f, 0.f, 0.f};
@@ -87,27 +97,27 @@ __device__ __forceinline__ void half_step_sums(const typename ElemTraits<T>::vec
     sum[nb] = acc_sum[0];
   }
 }
-template <typename T, int H, bool SUMS = true>
-__device__ __forceinline__ void half_step_p(const f32x16 (&s_use)[2], const float (&m)[2], float scale_log2,
-                                            typename ElemTraits<T>::vec8 (&pn)[2], float (&sum)[2]) {
+template <typename T, int NB, int H>
+__device__ __forceinline__ void half_step_p(const f32x16 (&s_use)[NB], const float (&m)[NB], float scale_log2,
+                                            typename ElemTraits<T>::vec8 (&pn)[NB], float (&sum)[NB]) {
 #pragma unroll
-  for (int nb = 0; nb < 2; ++nb)
+  for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
     for (int e = 0; e < 8; ++e)
       pn[nb][e] = (T)__builtin_amdgcn_exp2f(__builtin_fmaf(s_use[nb][H * 8 + e], scale_log2, -m[nb]));
-  if (SUMS) half_step_sums<T>(pn, sum);
+  half_step_sums<T, NB>(pn, sum);
 }
 
 // The rare path of a half-step: raise the reference exponents to the row maxima of the half-step,
 // rescale the row sums and redo the half-step's P.  alpha is what everything accumulated under the old
 // exponents has to be multiplied by.
-template <typename T, int D, int H>
-__device__ __forceinline__ void half_step_rescale(const f32x16 (&s_use)[2], float scale_log2,
-                                                  float (&alpha)[2], float (&m_run)[2], float (&l_run)[2],
-                                                  typename ElemTraits<T>::vec8 (&pn)[2], float (&sum)[2]) {
-  float m_use[2];
+template <typename T, int NB, int H>
+__device__ __forceinline__ void half_step_rescale(const f32x16 (&s_use)[NB], float scale_log2,
+                                                  float (&alpha)[NB], float (&m_run)[NB], float (&l_run)[NB],
+                                                  typename ElemTraits<T>::vec8 (&pn)[NB], float (&sum)[NB]) {
+  float m_use[NB];
 #pragma unroll
-  for (int nb = 0; nb < 2; ++nb) {
+  for (int nb = 0; nb < NB; ++nb) {
     // only this half-step's values: the other half of the step raises the exponents itself if it has
     // to, and the two rare paths of a step then share no work the compiler would compute up front
     float v = s_use[nb][H * 8];
@@ -122,7 +132,7 @@ __device__ __forceinline__ void half_step_rescale(const f32x16 (&s_use)[2], floa
     // rows that have seen no key yet (all masked) keep the floor; their P is 2^(-inf) = 0
     m_use[nb] = m_new;
   }
-  half_step_p<T, H>(s_use, m_use, scale_log2, pn, sum);
+  half_step_p<T, NB, H>(s_use, m_use, scale_log2, pn, sum);
 }
 
 // One block of the pipeline: half-step H (16 keys) of the 32-key step whose S^T is s_use.
@@ -131,14 +141,16 @@ __device__ __forceinline__ void half_step_rescale(const f32x16 (&s_use)[2], floa
 //   VALU  : P of this half-step from s_use -> pb (for the next block) and the row sums
 //   LDS   : V^T of this half-step's keys (v_key_off.. of v_tile) -> vf (for the next block)
 template <typename T, int D, int H>
-__device__ __forceinline__ void half_step(const f32x16 (&s_use)[2], f32x16 (&s_fill)[2],
+__device__ __forceinline__ void half_step(const f32x16 (&s_use)[WaveShape<D>::NB], f32x16 (&s_fill)[WaveShape<D>::NB],
                                           const unsigned char* k_tile, int k_row_off,
                                           const unsigned char* v_tile, int v_key_off, const LaneOffsets<D>& lo,
-                                          const typename ElemTraits<T>::vec8 (&qf)[2][D / 16],
-                                          f32x16 (&acc)[D / 32][2], float (&m_run)[2], float (&l_run)[2],
-                                          typename ElemTraits<T>::vec8 (&pb)[2],
+                                          const typename ElemTraits<T>::vec8 (&qf)[WaveShape<D>::NB][D / 16],
+                                          f32x16 (&acc)[D / 32][WaveShape<D>::NB], float (&m_run)[WaveShape<D>::NB],
+                                          float (&l_run)[WaveShape<D>::NB],
+                                          typename ElemTraits<T>::vec8 (&pb)[WaveShape<D>::NB],
                                           typename ElemTraits<T>::vec8 (&vf)[D / 32], float scale_log2) {
   typedef typename ElemTraits<T>::vec8 vec8;
+  constexpr int NB = WaveShape<D>::NB;
   constexpr int KH = D / 32;  // k-steps of this half
   constexpr int DB = D / 32;
 
@@ -155,63 +167,53 @@ __device__ __forceinline__ void half_step(const f32x16 (&s_use)[2], f32x16 (&s_f
 #pragma unroll
   for (int db = 0; db < DB; ++db)
 #pragma unroll
-    for (int nb = 0; nb < 2; ++nb) acc[db][nb] = Mfma<T>::run(vf[db], pb[nb], acc[db][nb]);
-  if (S_IN_VGPR<D>::value) {
+    for (int nb = 0; nb < NB; ++nb) acc[db][nb] = Mfma<T>::run(vf[db], pb[nb], acc[db][nb]);
+  if (H == 0) {
 #pragma unroll
-    for (int k2 = 0; k2 < KH; ++k2)
+    for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-      for (int nb = 0; nb < 2; ++nb) Mfma<T>::run_vgpr_acc(kf[k2], qf[nb][H * KH + k2], s_fill[nb], H == 0 && k2 == 0);
-  } else {
-    if (H == 0) {
-#pragma unroll
-      for (int nb = 0; nb < 2; ++nb)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) s_fill[nb][i] = 0.f;
-    }
-#pragma unroll
-    for (int k2 = 0; k2 < KH; ++k2)
-#pragma unroll
-      for (int nb = 0; nb < 2; ++nb) s_fill[nb] = Mfma<T>::run(kf[k2], qf[nb][H * KH + k2], s_fill[nb]);
+      for (int i = 0; i < 16; ++i) s_fill[nb][i] = 0.f;
   }
+#pragma unroll
+  for (int k2 = 0; k2 < KH; ++k2)
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) s_fill[nb] = Mfma<T>::run(kf[k2], qf[nb][H * KH + k2], s_fill[nb]);
 
-  vec8 pn[2];
-  float sum[2];
-  half_step_p<T, H, !S_IN_VGPR<D>::value>(s_use, m_run, scale_log2, pn, sum);
-  // Issue order of the block: each of its 2*D/16 large MFMAs is followed by a share of the P
-  // arithmetic (3 plain VALU, 2 exp), so the softmax fills the issue slots behind every MFMA instead
-  // of running as one burst after the last of them.  Measured 3 % faster than the scheduler's own order.
+  vec8 pn[NB];
+  float sum[NB];
+  half_step_p<T, NB, H>(s_use, m_run, scale_log2, pn, sum);
+  // Issue order of the block: each of its NB*D/16 large MFMAs is followed by a share of the P arithmetic (8 NB
+  // multiply-adds, 4 NB conversions, 8 NB exponentials in all), so the soft-max fills the issue slots behind
+  // every MFMA instead of running as one burst after the last of them.  Measured 3 % faster than the
+  // scheduler's own order.
+  constexpr int MFMAS = NB * D / 16;
 #pragma unroll
-  for (int g = 0; g < 2 * D / 16; ++g) {
-    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
-    __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);  // three VALU
-    __builtin_amdgcn_sched_group_barrier(0x400, 2, 0);  // two transcendental
+  for (int g = 0; g < MFMAS; ++g) {
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                          // one MFMA
+    __builtin_amdgcn_sched_group_barrier(0x002, (12 * NB + MFMAS - 1) / MFMAS, 0);  // its share of plain VALU
+    __builtin_amdgcn_sched_group_barrier(0x400, 8 * NB / MFMAS, 0);             // and of the transcendentals
   }
-  if (S_IN_VGPR<D>::value) {
-    // The S^T MFMAs written as assembly get none of the compiler's wait states between an MFMA and a
-    // vector instruction that reads its result.  They are all issued before this point, the MFMAs of
-    // the sums after it, the matrix pipe completes in order, and the branch below waits for the sums:
-    // so when the next block reads S^T, those MFMAs have completed.
-    __builtin_amdgcn_sched_barrier(0);
-    half_step_sums<T>(pn, sum);
-  }
-  // One compare for both query blocks: their sums are >= 0 or NaN, so the total is below the limit
-  // only if both are.  Not "total >= limit": a NaN (row that has seen nothing yet) must take the rare
+  // One compare for all query blocks: their sums are >= 0 or NaN, so the total is below the limit
+  // only if every one is.  Not "total >= limit": a NaN (row that has seen nothing yet) must take the rare
   // path too.
-  const bool redo = !(sum[0] + sum[1] < HALF_SUM_LIMIT);
+  float total = sum[0];
+#pragma unroll
+  for (int nb = 1; nb < NB; ++nb) total += sum[nb];
+  const bool redo = !(total < HALF_SUM_LIMIT);
   if (__builtin_expect(__builtin_amdgcn_ballot_w64(redo) != 0, false)) {
-    float alpha[2];
-    half_step_rescale<T, D, H>(s_use, scale_log2, alpha, m_run, l_run, pn, sum);
+    float alpha[NB];
+    half_step_rescale<T, NB, H>(s_use, scale_log2, alpha, m_run, l_run, pn, sum);
     // the accumulators hold everything up to the previous half-step (its P.V was issued above; the
     // P.V of this half-step is added by the next block, under the new exponents)
 #pragma unroll
     for (int db = 0; db < DB; ++db)
 #pragma unroll
-      for (int nb = 0; nb < 2; ++nb)
+      for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc[db][nb][i] *= alpha[nb];
   }
 #pragma unroll
-  for (int nb = 0; nb < 2; ++nb) {
+  for (int nb = 0; nb < NB; ++nb) {
     l_run[nb] += sum[nb];
     pb[nb] = pn[nb];
   }
@@ -238,9 +240,12 @@ __device__ __forceinline__ const unsigned char* piece_address(const unsigned cha
 }
 
 template <typename T, int D, bool GATHER, bool CAUSAL, bool PLAIN = false, bool NARROW = false, bool REWEIGHT = false>
-__global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_kernel(const ha_attn_kernel_params p) {
+__global__ __launch_bounds__(WaveShape<D>::THREADS, 2) void ha_attn_fwd_kernel(const ha_attn_kernel_params p) {
   typedef typename ElemTraits<T>::vec8 vec8;
   typedef typename ElemTraits<T>::vec4 vec4;
+  constexpr int NB = WaveShape<D>::NB;        // 32-query column blocks per wave
+  constexpr int QW = WaveShape<D>::QW;        // queries per wave
+  constexpr int WAVES = WaveShape<D>::WAVES;  // waves per workgroup
   constexpr int DV = D;
   constexpr int KSTEPS = D / 16;  // MFMA k-steps of Q.K^T
   constexpr int DB = DV / 32;     // 32-row blocks of O^T
@@ -248,10 +253,11 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 ? 2 : 1)) void ha_attn_fwd_ker
 
   // Separate LDS objects (two K tiles, two V tiles of KC rows, the query rows): the compiler then
   // knows that a tile being filled from HBM and a tile being read do not alias, and does not
-  // serialise them.  The query region (one tile per wave) is reused for the output rows at the end.
+  // serialise them.  The query region (QW rows per wave) is reused for the output rows at the end.
   constexpr int TILE_BYTES = KC * D * 2;
   // The key tiles ask for the larger alignment only to be placed first: LDS offsets below 64 KB fit
   // the immediate field of the LDS reads, which matters at d = 128 where the workgroup uses 130 KB.
+  constexpr int Q_WAVE_BYTES = QW * D * 2;  // a wave's part of the query region
   __shared__ __attribute__((aligned(1024))) unsigned char lds_k0[TILE_BYTES];
   __shared__ __attribute__((aligned(1024))) unsigned char lds_k1[TILE_BYTES];
   __shared__ __attribute__((aligned(1024))) unsigned char lds_v0[TILE_BYTES];
@@ -340,7 +346,7 @@ namespace {
 
 template <typename T, int D, bool GATHER, bool CAUSAL, bool PLAIN = false, bool NARROW = false, bool REWEIGHT = false>
 int launch_one(const ha_attn_kernel_params& p, int grid, hipStream_t stream, const char* what) {
-  hipLaunchKernelGGL((ha_attn_fwd_kernel<T, D, GATHER, CAUSAL, PLAIN, NARROW, REWEIGHT>), dim3(grid), dim3(WG_THREADS), 0,
+  hipLaunchKernelGGL((ha_attn_fwd_kernel<T, D, GATHER, CAUSAL, PLAIN, NARROW, REWEIGHT>), dim3(grid), dim3(WaveShape<D>::THREADS), 0,
                      stream, p);
   return ha_launch_status(what);
 }

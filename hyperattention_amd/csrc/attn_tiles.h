@@ -28,17 +28,6 @@ struct Mfma<f16_t> {
   static __device__ __forceinline__ f32x16 run(f16x8 a, f16x8 b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
   }
-  // The same MFMA with its accumulator pinned to VGPRs and its B operand to AGPRs.  A kernel that
-  // needs more than 256 registers gets the AGPR form for every MFMA the compiler selects, and a vector
-  // instruction cannot read an AGPR: accumulators that the soft-max reads (S^T) would cost a copy per
-  // value.  Written as assembly the instruction keeps them where the FMAs can use them, while the
-  // query fragments (B) sit in AGPRs for the whole kernel.  first: accumulate onto zero.
-  static __device__ __forceinline__ void run_vgpr_acc(f16x8 a, f16x8 b, f32x16& c, bool first) {
-    if (first)
-      asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "a"(b));
-    else
-      asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "a"(b));
-  }
   // c[*] + a[0] + a[1] + a[2] + a[3] on the matrix pipe: the 4x4x4 MFMA works on 16 independent
   // blocks of 4 lanes; with an all-ones A a lane's four results are all the sum of its own four B values
   static __device__ __forceinline__ f32x4 quad_sum(f16x4 a, f32x4 c) {
@@ -50,12 +39,6 @@ template <>
 struct Mfma<bf16_t> {
   static __device__ __forceinline__ f32x16 run(bf16x8 a, bf16x8 b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
-  }
-  static __device__ __forceinline__ void run_vgpr_acc(bf16x8 a, bf16x8 b, f32x16& c, bool first) {
-    if (first)
-      asm("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "a"(b));
-    else
-      asm("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "a"(b));
   }
   static __device__ __forceinline__ f32x4 quad_sum(bf16x4 a, f32x4 c) {
     typedef short s16x4 __attribute__((ext_vector_type(4)));
