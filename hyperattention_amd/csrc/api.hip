@@ -93,6 +93,7 @@ void fill_params(const ha_attn_operands& t, ha_attn_kernel_params& p) {
   p.block_tiles = 1; p.sample_chunks = 0; p.smooth = 0; p.accumulate = 0; p.idx64 = 0;
   p.sampled_pos = nullptr; p.sample_bias_raw = 0.f;
   p.n_q_last = (int)t.n_q;
+  p.tiles_per_wg = 1;
   p.rag_levels = -1; p.rag_split = 0; p.rag_n = 0;
   for (int& c : p.rag_half) c = 0;
   p.scale_log2 = t.scale * LOG2E_F;

@@ -44,6 +44,9 @@ struct ha_attn_kernel_params {
   // past this number names a row that is not there (the zero row the causal recursion appends to an odd
   // length, hyper_attention.py:61-64); it is placed like any other row and its result is dropped.
   int n_q_last;
+  // Streaming gathered kernel: consecutive query tiles of one (virtual) head per workgroup (the last
+  // workgroup of a head may have fewer); 1: the one-tile kernels
+  int tiles_per_wg;
   // Ragged segments (exact kernels; rag_levels < 0: regular).  Inside a causal recursion with odd lengths the
   // segments of a level neither start at multiples of one stride nor hold the same number of rows: level i
   // cuts a segment of (padded) length 2*rag_half[i] into two, and the rows that exist are the first rag_n of

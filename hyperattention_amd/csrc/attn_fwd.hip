@@ -44,6 +44,8 @@
 #include "attn_tiles.h"
 #include "attn_fwd.h"
 
+#include <stdlib.h>
+
 namespace {
 
 constexpr int WG_QUERIES = 256;  // sorted query positions per workgroup
@@ -342,6 +344,8 @@ __global__ __launch_bounds__(WaveShape<D>::THREADS, 2) void ha_attn_fwd_kernel(c
   }
 }
 
+#include "attn_fwd_stream.inc"
+
 namespace {
 
 template <typename T, int D, bool GATHER, bool CAUSAL, bool PLAIN = false, bool NARROW = false, bool REWEIGHT = false>
@@ -358,6 +362,11 @@ int launch_variant(const ha_attn_kernel_params& p, int grid, bool gather, bool c
     return launch_one<T, D, true, false, false, false, true>(p, grid, stream, "ha_block_attn_fwd");
   if (gather) {
     const bool plain = !p.smooth && !p.sampled_idx && p.block_tiles % 2 == 0 && p.n_q % WG_QUERIES == 0;
+    if (p.tiles_per_wg > 1) {  // set by ha_attn_launch for the instances built below
+      if (plain) hipLaunchKernelGGL((ha_attn_fwd_stream_kernel<T, D, true>), dim3(grid), dim3(WaveShape<D>::THREADS), 0, stream, p);
+      else hipLaunchKernelGGL((ha_attn_fwd_stream_kernel<T, D, false>), dim3(grid), dim3(WaveShape<D>::THREADS), 0, stream, p);
+      return ha_launch_status("ha_block_attn_fwd");
+    }
     if (narrow) return launch_one<T, D, true, false, false, true>(p, grid, stream, "ha_block_attn_fwd");
     if (plain) return launch_one<T, D, true, false, true>(p, grid, stream, "ha_block_attn_fwd");
     return launch_one<T, D, true, false>(p, grid, stream, "ha_block_attn_fwd");
@@ -392,6 +401,26 @@ int ha_attn_launch(const ha_attn_kernel_params& params, int d, int dv, int dtype
   p.v_pieces = dv / 8;
   int64_t qtiles = (p.n_q + WG_QUERIES - 1) / WG_QUERIES;
   if (causal && !gather) qtiles = (qtiles + 1) / 2;  // exact causal attention: one workgroup per pair of tiles
+  // Gathered attention with whole 256-query tiles, whole key blocks and an even number of at least four key
+  // chunks per tile can run as a stream: a workgroup takes a run of tiles of its head
+  // (ha_attn_fwd_stream_kernel), as long a run as still leaves every CU its full set of resident workgroups.
+  // It is the default where it measured faster: head dim 128 (one workgroup per CU, nothing else covers a
+  // workgroup's set-up and output stage) in the plain configuration, 4 to 7 % on a level of 64 tiles per head
+  // at 8 chunks per tile.  At head dim 64 the second workgroup of the CU covers them already and the stream
+  // measured 2 to 5 % slower; with smooth windows (18 chunks per tile) it measured the same.
+  p.tiles_per_wg = 1;
+  const char* stream_env = getenv("HA_STREAM_TILES");  // measurement aid: force the run length (1: off)
+  const bool plain = !p.smooth && !p.sampled_idx && p.block_tiles % 2 == 0;
+  if (gather && !reweight && p.qk_pieces == width / 8 && p.v_pieces == width / 8 && p.n_q % WG_QUERIES == 0 && qtiles >= 2 &&
+      p.sample_chunks % 2 == 0 && p.n_k % (p.block_tiles * 128) == 0 && 2 * p.block_tiles + p.sample_chunks >= 4 &&
+      (stream_env || (width == 128 && plain))) {
+    const int64_t slots = 256 * (width == 64 ? 2 : 1);  // workgroups the chip holds at once
+    int r = 16;
+    while (r > 1 && (r > qtiles || (qtiles / r) * p.batch * p.heads * p.segs < slots)) r /= 2;
+    if (stream_env) r = atoi(stream_env) < 1 ? 1 : (atoi(stream_env) > qtiles ? (int)qtiles : atoi(stream_env));
+    p.tiles_per_wg = r;
+    qtiles = (qtiles + r - 1) / r;
+  }
   p.div_qtiles = make_divisor(qtiles);
   p.div_segs = make_divisor(p.segs);
   p.div_heads = make_divisor(p.heads);

@@ -316,6 +316,44 @@ def test_block_attention_resumes_partial_result(ha, dtype, shift):
     assert_close(lse, want_lse, "resumed lse")
 
 
+@pytest.mark.parametrize("run", [2, 3, 8])
+@pytest.mark.parametrize("dtype,d,block,sample,smooth,resume", [
+    (torch.bfloat16, 128, 256, 256, False, True),    # the shape the library streams by default (plain, d = 128)
+    (torch.bfloat16, 128, 256, 128, True, False),    # smooth windows: the general instance
+    (torch.float16, 64, 256, 128, False, True),
+    (torch.float16, 64, 128, 256, False, False),     # one 128-key block per 128 queries
+    (torch.float16, 128, 384, 0, True, True),        # no samples, a block that is not a power of two
+])
+def test_streaming_kernel_equals_the_one_tile_kernel(ha, monkeypatch, run, dtype, d, block, sample, smooth, resume):
+    """A workgroup that takes a run of query tiles (the library's choice for large d = 128 launches; forced here
+    by the library's measurement switch) computes bit for bit what one workgroup per tile computes: output and
+    log-sum-exp, with and without a partial result to resume, whole runs and a last run that is shorter."""
+    b, h, n = 1, 2, 2304                       # 9 tiles of 256: runs of 2, 3 and 8 all leave a shorter last run or none
+    q, k, v, qi, ki = _sorted_inputs(b, h, n, d, dtype, 90)
+    c = lambda t: t.cuda()
+
+    def call(tiles):
+        monkeypatch.setenv("HA_STREAM_TILES", str(tiles))
+        kw = {}
+        if resume:
+            g = _gen(95)
+            o_prev = torch.randn((b, n, h, d), generator=g).to(dtype).cuda()
+            l_prev = torch.randn((b, h, n), generator=g).cuda()
+            l_prev[:, :, ::5] = float("-inf")
+            o_prev[:, ::5] = 0
+            kw["resume"] = (o_prev, l_prev)
+        o, lse = ha.hyper_attn_func(c(q).transpose(1, 2), c(k).transpose(1, 2), c(v).transpose(1, 2),
+                                    c(qi).transpose(1, 2), c(ki).transpose(1, 2), block, sample, None, smooth, **kw)
+        torch.cuda.synchronize()
+        return o.clone(), lse.clone()
+
+    o1, l1 = call(1)
+    o2, l2 = call(run)
+    assert torch.isfinite(o1.float()).all()
+    assert torch.equal(o1, o2), f"out differs, max {float((o1.float() - o2.float()).abs().max()):.3e}"
+    assert torch.equal(l1, l2), f"lse differs, max {float((l1 - l2).abs().max()):.3e}"
+
+
 @pytest.mark.parametrize("dtype,d,smooth,block,per_head", [
     (torch.float16, 64, False, 256, False),
     (torch.bfloat16, 128, True, 256, True),
