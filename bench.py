@@ -54,13 +54,15 @@ HBM_PEAK_GBS = 8000.0
 
 
 def kernel_source_digest():
-    """sha256 (first 16 hex digits) of the attention kernel's source: the counter summaries under profiles/
-    record the digest of the source they were measured on."""
-    path = os.path.join(ROOT, "hyperattention_amd", "csrc", "attn_fwd.hip")
+    """sha256 (first 16 hex digits) of the attention kernels' sources: the counter summaries under profiles/
+    record the digest of the sources they were measured on."""
+    h = hashlib.sha256()
     try:
-        return hashlib.sha256(open(path, "rb").read()).hexdigest()[:16]
+        for name in ("attn_fwd.hip", "attn_fwd_tile.inc", "attn_fwd_stream.inc", "attn_tiles.h"):
+            h.update(open(os.path.join(ROOT, "hyperattention_amd", "csrc", name), "rb").read())
     except OSError:
         return None
+    return h.hexdigest()[:16]
 
 
 def quoted_traffic(workload):
