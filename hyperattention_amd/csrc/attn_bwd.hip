@@ -111,12 +111,15 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 || PASS == HA_BWD_DQ_BLOCK ? 2
   const int st_total = PASS == HA_BWD_DKV_SAMPLED ? p.sample_size : (KEY_ST ? p.n_k : p.n_q);
   const int st_tiles = (st_total + ST_ROWS - 1) / ST_ROWS;
   const int splits = PASS == HA_BWD_DKV_SAMPLED ? (p.n_q + p.q_split - 1) / p.q_split : 1;
+  // Exact causal attention: a workgroup takes the pair of stationary tiles (s, T-1-s), the one that streams more
+  // rows first (the last query tile sees every key, the first key tile is seen by every query), so that every
+  // workgroup of a launch streams the same number of rows.  The hardware hands out workgroups in order, and a
+  // slot freed by a short one stays empty until the ones queued before it are placed.
+  constexpr bool PAIRED = CAUSAL && (PASS == HA_BWD_DQ_EXACT || PASS == HA_BWD_DKV_EXACT);
+  const int wg_per_seq = PAIRED ? (st_tiles + 1) / 2 : st_tiles;
   int rest = xcd_contiguous_id(blockIdx.x, gridDim.x);
-  int tile = rest % st_tiles;
-  rest /= st_tiles;
-  // causal dq: the tiles with the most keys first, so that the last workgroups of the grid are short
-  // (the dk/dv tiles are in that order as they come: the first key tile streams the most queries)
-  if (PASS == HA_BWD_DQ_EXACT && CAUSAL) tile = st_tiles - 1 - tile;
+  const int slot = rest % wg_per_seq;
+  rest /= wg_per_seq;
   const int split = rest % splits;
   const int vseq = rest / splits;   // (batch, head, segment)
   const int seg = vseq % p.segs;
@@ -168,582 +171,21 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 || PASS == HA_BWD_DQ_BLOCK ? 2
   const uint32_t y1_rb = KEY_ST ? q_rb : k_rb, y2_rb = KEY_ST ? do_rb : v_rb;
   const int n_y = KEY_ST ? p.n_q : p.n_k;  // rows on the streamed side
 
-  // ---- the stationary row of this lane's MFMA column ------------------------------------------
-  const int st_pos = tile * ST_ROWS + wave * 32 + col;  // position in the stationary order
-  const bool st_valid = st_pos < st_total;
-  int st_row;  // original row
-  {
-    const int pos = st_valid ? st_pos : 0;
-    if (PASS == HA_BWD_DQ_BLOCK)
-      st_row = *reinterpret_cast<const int*>(row_address(q_idx_head(0), pos, qi_rb, 0));
-    else if (PASS == HA_BWD_DKV_BLOCK)
-      st_row = *reinterpret_cast<const int*>(row_address(k_idx, pos, ki_rb, 0));
-    else if (PASS == HA_BWD_DKV_SAMPLED)
-      st_row = s_idx ? *reinterpret_cast<const int*>(row_address(s_idx, pos, si_rb, 0)) : pos;
-    else
-      st_row = pos;
-  }
-  // ---- the streamed chunks of this workgroup ---------------------------------------------------
-  const int T_blk = p.block_tiles;
-  const int nkc = p.n_k / YC;  // gathered passes: n_k % 128 == 0
-  int nc = 0;                  // number of streamed chunks
-  int y_first = 0;             // exact / sampled passes: first streamed row
-  int y_end = n_y;             // exact / sampled passes: end of the valid streamed rows
-  int blk_start = 0, n_blk = 0;  // dQ of the gathered kernel: first chunk (sorted keys) and count of the block part
-  int t_first = 0;               // dK/dV of the block part, plain blocks: first attending query tile
-  if (PASS == HA_BWD_DQ_EXACT) {
-    if (CAUSAL) {
-      const int qend = (tile + 1) * ST_ROWS;
-      y_end = y_end < qend ? y_end : qend;
-    }
-    nc = (y_end + YC - 1) / YC;
-  } else if (PASS == HA_BWD_DKV_EXACT) {
-    y_first = CAUSAL ? tile * ST_ROWS : 0;
-    nc = y_end > y_first ? (y_end - y_first + YC - 1) / YC : 0;
-  } else if (PASS == HA_BWD_DKV_SAMPLED) {
-    y_first = split * p.q_split;
-    const int e = y_first + p.q_split;
-    y_end = e < p.n_q ? e : p.n_q;
-    nc = (y_end - y_first + YC - 1) / YC;
-  } else if (PASS == HA_BWD_DQ_BLOCK) {
-    // the key window of reference query tile `tile` (src/hyper_attn_triton.py:99-107)
-    const int block_id = tile / T_blk;
-    const int first = block_id * T_blk * 128;
-    int last = first + T_blk * 128;
-    last = last < p.n_k ? last : p.n_k;
-    n_blk = last > first ? (last - first) / YC : 0;
-    blk_start = first / YC;
-    if (p.smooth) {
-      int sk = (tile * 128 - (T_blk - 1) * 64) % p.n_k;
-      sk += sk < 0 ? p.n_k : 0;
-      blk_start = sk / YC;
-    }
-    nc = n_blk + p.sample_size / YC;
-  } else {  // HA_BWD_DKV_BLOCK: the query tiles whose window holds this key tile
-    const int n_qt = p.n_q / 128;
-    if (!p.smooth) {
-      const int block_id = tile / T_blk;
-      t_first = block_id * T_blk;
-      int t_last = t_first + T_blk;
-      t_last = t_last < n_qt ? t_last : n_qt;
-      nc = t_last > t_first ? 2 * (t_last - t_first) : 0;
-    } else {
-      // list them (ascending), with one flag per 64-key half of this tile: bit 30 lower, bit 31 upper
-      if (wave_s == 0) {
-        int count = 0;
-        for (int t0 = 0; t0 < n_qt; t0 += 64) {
-          const int t = t0 + lane;
-          bool m0 = false, m1 = false;
-          if (t < n_qt) {
-            const int block_id = t / T_blk;
-            const int first = block_id * T_blk * 128;
-            int last = first + T_blk * 128;
-            last = last < p.n_k ? last : p.n_k;
-            const int cnt = last > first ? (last - first) / YC : 0;
-            int sk = (t * 128 - (T_blk - 1) * 64) % p.n_k;
-            sk += sk < 0 ? p.n_k : 0;
-            int o0 = 2 * tile - sk / YC;
-            o0 += o0 < 0 ? nkc : 0;
-            int o1 = 2 * tile + 1 - sk / YC;
-            o1 += o1 < 0 ? nkc : 0;
-            m0 = o0 < cnt;
-            m1 = o1 < cnt;
-          }
-          const bool any = m0 || m1;
-          const uint64_t mask = __ballot(any);
-          if (any) {
-            const int pos = count + __popcll(mask & ((1ull << lane) - 1));
-            if (pos < MAX_SMOOTH_TILES) lds_tiles[pos] = t | (m0 ? 1 << 30 : 0) | (m1 ? (int)(1u << 31) : 0);
-          }
-          count += __popcll(mask);
-        }
-        if (lane == 0) lds_ntiles = count < MAX_SMOOTH_TILES ? count : MAX_SMOOTH_TILES;
-      }
-      __syncthreads();
-      nc = 2 * lds_ntiles;
-    }
-  }
-  const int nc_head = __builtin_amdgcn_readfirstlane(nc);  // chunks per query head
-  nc = nc_head * n_group;
-
-  // Original row of streamed row r (0..63) of chunk c, clamped to rows that exist; chunks past the
-  // end repeat the last one.  Gathered passes read an index array here.
-  auto attending_tile = [&](int k) -> int {  // dK/dV of the block part: k-th attending query tile with its flags
-    if (PASS != HA_BWD_DKV_BLOCK) return 0;
-    return p.smooth ? lds_tiles[k] : ((t_first + k) | (int)(3u << 30));
-  };
-  auto group_of = [&](int c) -> int { return n_group == 1 ? 0 : (c < nc ? c : nc - 1) / nc_head; };
-  auto stream_row = [&](int c, int r) -> int {
-    c = c < nc ? c : nc - 1;
-    const int gi = group_of(c);
-    c -= gi * nc_head;
-    if (PASS == HA_BWD_DQ_BLOCK) {
-      if (c < n_blk) {
-        int u = blk_start + c;
-        u -= u >= nkc ? nkc : 0;
-        return *reinterpret_cast<const int*>(row_address(k_idx, u * YC + r, ki_rb, 0));
-      }
-      const int s = (c - n_blk) * YC + r;
-      return s_idx ? *reinterpret_cast<const int*>(row_address(s_idx, s, si_rb, 0)) : s;
-    } else if (PASS == HA_BWD_DKV_BLOCK) {
-      const int t = attending_tile(c >> 1) & 0x3fffffff;
-      return *reinterpret_cast<const int*>(row_address(q_idx_head(gi), t * 128 + (c & 1) * YC + r, qi_rb, 0));
-    } else {
-      const int row = y_first + c * YC + r;
-      return row < n_y ? row : n_y - 1;
-    }
-  };
-
-  if (nc <= 0) {
-    // nothing attends (or is attended by) this tile: its gradient is zero
-    if (PASS != HA_BWD_DKV_SAMPLED && st_valid) {
-      const vec4 zero = {(T)0.f, (T)0.f, (T)0.f, (T)0.f};
-      unsigned char* const dqb = (unsigned char*)((T*)p.dq + b * p.dq_sb + h0 * p.dq_sh + q_row0 * p.dq_sn) + (int64_t)st_row * p.dq_sn * 2;
-      unsigned char* const dkb = (unsigned char*)((T*)p.dk + b * p.dk_sb + hk * p.dk_sh + k_row0 * p.dk_sn) + (int64_t)st_row * p.dk_sn * 2;
-      unsigned char* const dvb = (unsigned char*)((T*)p.dv + b * p.dv_sb + hk * p.dv_sh + k_row0 * p.dv_sn) + (int64_t)st_row * p.dv_sn * 2;
-#pragma unroll
-      for (int db = 0; db < DB; ++db)
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          const int dd = 32 * db + 8 * g + 4 * hi;
-          if (!KEY_ST) {
-            if (!p.accumulate) *reinterpret_cast<vec4*>(dqb + dd * 2) = zero;
-          } else if (!p.accumulate) {
-            *reinterpret_cast<vec4*>(dkb + dd * 2) = zero;
-            *reinterpret_cast<vec4*>(dvb + dd * 2) = zero;
-          }
-        }
-    }
-    return;
-  }
-
-  // ---- tile loads: HBM -> LDS, 16 bytes per lane, whole rows, swizzle applied on the source side ----
-  const int my_pp = lane % PR;  // physical piece of this lane's LDS slot
-  const int my_lr = lane / PR;  // row inside one tile load
-  int rows_next[LPW];           // source rows of this wave's loads of the next tile
-  int group_next = 0;           // the query head (within the group) those rows belong to
-  int stat_row_next = 0;        // dK/dV passes: source row of streamed row 16 * wave + lane % 16 of the next tile
-                                // (every wave fetches the statistics of 16 rows: no wave has more to do)
-  bool stat_past_end_next = false;
-  float stat_lse = 0.f, stat_delta = 0.f;
-  auto fetch_rows = [&](int c) {
-#pragma unroll
-    for (int j = 0; j < LPW; ++j) rows_next[j] = stream_row(c, (wave_s * LPW + j) * RPL + my_lr);
-    if (KEY_ST) {
-      stat_row_next = stream_row(c, wave_s * 16 + (lane & 15));
-      // sampled keys: a streamed query past the end of the workgroup's range gets L = +inf below, so that
-      // P = 2^(s - inf) = 0 and dS = 0 * finite = 0 with no mask in the chunk
-      if (PASS == HA_BWD_DKV_SAMPLED) {
-        const int cc = (c < nc ? c : nc - 1) - group_of(c) * nc_head;
-        stat_past_end_next = y_first + cc * YC + wave_s * 16 + (lane & 15) >= y_end;
-      }
-    }
-    group_next = group_of(c);
-  };
-  auto load_tile = [&](int buf) {  // the tile whose rows are in rows_next
-    const unsigned char* const y1b = KEY_ST ? q_head(group_next) : kb;
-    const unsigned char* const y2b = KEY_ST ? do_head(group_next) : vb;
-#pragma unroll
-    for (int j = 0; j < LPW; ++j) {
-      const int r = (wave_s * LPW + j) * RPL + my_lr;
-      const uint32_t piece = (uint32_t)((my_pp ^ bwd_swizzle<D>(r)) << 4);
-      unsigned char* const dst1 = lds_y1[buf] + (wave_s * LPW + j) * 1024;
-      unsigned char* const dst2 = lds_y2[buf] + (wave_s * LPW + j) * 1024;
-      global_to_lds_16(row_address(y1b, rows_next[j], y1_rb, piece), dst1);
-      global_to_lds_16(row_address(y2b, rows_next[j], y2_rb, piece), dst2);
-    }
-    if (KEY_ST) {
-      const f32x2 sd = stats_head(group_next)[stat_row_next];
-      stat_lse = stat_past_end_next ? __builtin_inff() : sd[0];
-      stat_delta = FOLD_D ? sd[1] : -sd[1] * p.scale;  // the word holds -D
-    }
-  };
-
-  // the row numbers of the first tile are asked for before the stationary rows, so that the two chains
-  // index -> rows run side by side
-  fetch_rows(0);
-  vec8 x1f[KSTEPS], x2f[KSTEPS];
-  float st_lse2 = 0.f, st_delta = 0.f;  // dQ passes: L (log2 units) and D * scale of the lane's query
-  f32x16 neg_d;  // dQ passes: -D in every element, what the dP accumulators of a chunk start from
-#pragma unroll
-  for (int i = 0; i < 16; ++i) neg_d[i] = 0.f;
-  vec8 of[KSTEPS];  // dQ passes: the lane's pieces of its query's output row
-  const unsigned char* const ob = (const unsigned char*)((const T*)p.out + b * p.o_sb + h0 * p.o_sh + q_row0 * p.o_sn);
-  const uint32_t o_rb = (uint32_t)p.o_sn * 2;
-  if (!KEY_ST) {
-    if (!STAGE_X) {
-#pragma unroll
-      for (int ks = 0; ks < KSTEPS; ++ks)
-        of[ks] = *reinterpret_cast<const vec8*>(row_address(ob, st_row, o_rb, (ks * 16 + hi * 8) * 2));
-    }
-  }
-  if (!STAGE_X) {
-#pragma unroll
-    for (int ks = 0; ks < KSTEPS; ++ks) {
-      x1f[ks] = *reinterpret_cast<const vec8*>(row_address(x1b, st_row, x1_rb, (ks * 16 + hi * 8) * 2));
-      x2f[ks] = *reinterpret_cast<const vec8*>(row_address(x2b, st_row, x2_rb, (ks * 16 + hi * 8) * 2));
-    }
+  if constexpr (!PAIRED) {
+    const int tile = slot;
+#include "attn_bwd_tile.inc"
   } else {
-    // The stationary rows come through LDS (dK/dV passes; dQ passes at d = 64, where the 32 KB fit beside
-    // two workgroups per CU): whole rows per 8 or 16 consecutive lanes (one 128- or 256-byte request per
-    // row) instead of one 16-byte piece of 64 different rows per instruction.  Each wave stages its own
-    // 32 rows, so only the wave itself has to wait.  The row numbers (stationary rows, first tile) are
-    // waited for first; then the stationary rows, the queries' output rows (dQ passes: into the second
-    // pair of tile buffers, which the loop fills only after its first barrier) and the first tile are all
-    // asked for together: two memory round trips before the first chunk instead of three or four.
-    constexpr int ROWS_PER_LOAD = 64 / PR;
-    const int row_in_load = lane / PR, phys_piece = lane % PR;
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the row numbers
-    unsigned char* const o_stage = (wave_s < 2 ? lds_y1[1] : lds_y2[1]) + (wave_s & 1) * 32 * D * 2;
-#pragma unroll
-    for (int j = 0; j < 32 / ROWS_PER_LOAD; ++j) {
-      const int r = j * ROWS_PER_LOAD + row_in_load;  // 0..31: a stationary row of this wave
-      const int row = __shfl(st_row, r);
-      const uint32_t piece = (uint32_t)((phys_piece ^ bwd_swizzle<D>(r)) << 4);
-      const int dst = (wave_s * 32 + j * ROWS_PER_LOAD) * D * 2;
-      global_to_lds_16(row_address(x1b, row, x1_rb, piece), lds_x1 + dst);
-      global_to_lds_16(row_address(x2b, row, x2_rb, piece), lds_x2 + dst);
-      if (!KEY_ST) global_to_lds_16(row_address(ob, row, o_rb, piece), o_stage + j * ROWS_PER_LOAD * D * 2);
+    const int t_long = PASS == HA_BWD_DQ_EXACT ? st_tiles - 1 - slot : slot;
+    const int t_short = st_tiles - 1 - t_long;
+    {
+      const int tile = t_long;
+#include "attn_bwd_tile.inc"
     }
-  }
-
-  if (!KEY_ST) st_lse2 = p.lse[b * p.lse_sb + h0 * p.lse_sh + q_row0 + st_row] * LOG2E;
-  load_tile(0);
-  fetch_rows(1);
-
-  if (STAGE_X) {
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the stationary rows (and the first tile) have landed
-#pragma unroll
-    for (int ks = 0; ks < KSTEPS; ++ks) {
-      const int off = bwd_tile_offset<D>(wave_s * 32 + col, ks * 2 + hi);
-      x1f[ks] = lds_read_k<T>(lds_x1, off);
-      x2f[ks] = lds_read_k<T>(lds_x2, off);
-      if (!KEY_ST) {
-        const unsigned char* const o_stage = (wave_s < 2 ? lds_y1[1] : lds_y2[1]) + (wave_s & 1) * 32 * D * 2;
-        of[ks] = lds_read_k<T>(o_stage, bwd_tile_offset<D>(col, ks * 2 + hi));
-      }
-    }
-  }
-  if (!KEY_ST) {
-    // D = sum_c dO * O of the lane's query: the two lanes of a column hold complementary pieces of the row.
-    // The dK/dV passes of the call read both statistics from the workspace.
-    float part = 0.f;
-#pragma unroll
-    for (int ks = 0; ks < KSTEPS; ++ks)
-#pragma unroll
-      for (int e = 0; e < 8; ++e) part = __builtin_fmaf((float)of[ks][e], (float)x2f[ks][e], part);
-    const float d_row = ha_sum_xor32(part);
-    st_delta = d_row * p.scale;
-#pragma unroll
-    for (int i = 0; i < 16; ++i) neg_d[i] = -d_row;
-    if (hi == 0 && st_valid) p.stats[((int64_t)(b * p.heads + h0) * p.segs + seg) * p.n_q + st_row] = f32x2{st_lse2, -d_row};
-  }
-
-  // per-lane LDS offsets of the operand reads
-  int off_rows[KSTEPS];  // piece of k-step ks of tile row lane%32, 16-byte read
-#pragma unroll
-  for (int ks = 0; ks < KSTEPS; ++ks) off_rows[ks] = bwd_tile_offset<D>(col, ks * 2 + hi);
-  // transposing read: lane s = 4j + w of a 16-lane group addresses streamed row j (+4 for the upper lane
-  // half), 8-byte word w of the 16 columns of its group; a second read takes the rows 8 further on
-  int off_tr_lo[DB], off_tr_hi[DB];
-  {
-    const int g = lane >> 4, sl = lane & 15;
-    const int key = (g >> 1) * 4 + (sl >> 2);
-    const int w = sl & 3;
-#pragma unroll
-    for (int db = 0; db < DB; ++db) {
-      off_tr_lo[db] = bwd_tile_offset<D>(key, db * 4 + (g & 1) * 2 + (w >> 1)) + (w & 1) * 8;
-      off_tr_hi[db] = bwd_tile_offset<D>(key + 8, db * 4 + (g & 1) * 2 + (w >> 1)) + (w & 1) * 8;
-    }
-  }
-
-  f32x16 acc1[DB], acc2[DB];  // dQ^T, or dK^T and dV^T: rows = head dim, column = the lane's stationary row
-#pragma unroll
-  for (int db = 0; db < DB; ++db)
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      acc1[db][i] = 0.f;
-      acc2[db][i] = 0.f;
-    }
-
-  for (int c = 0; c < nc; ++c) {
-    const int buf = c & 1;
-    if (KEY_ST && lane < 16) {
-      lds_lse[buf][wave_s * 16 + lane] = stat_lse;
-      lds_delta[buf][wave_s * 16 + lane] = stat_delta;
-    }
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's part of tile c has landed
-    __syncthreads();
-    if (c + 1 < nc) {
-      load_tile(buf ^ 1);
-      fetch_rows(c + 2);
-    }
-
-    // does this wave take part in the chunk at all (smoothed blocks: the window of a query tile can end
-    // between the two 64-key halves of the stationary tile)
-    const int cc = c - group_of(c) * nc_head;  // chunk number within its query head
-    bool wave_in = true;      // does the wave have any pair in this chunk
-    bool needs_mask = false;  // and are some of its pairs masked
-    const int y_lo = y_first + cc * YC, y_hi = y_lo + YC - 1;             // streamed rows of the chunk (exact, sampled)
-    const int st_lo = tile * ST_ROWS + wave_s * 32, st_hi = st_lo + 31;  // stationary positions of the wave
-    if (PASS == HA_BWD_DKV_BLOCK) {
-      wave_in = (attending_tile(cc >> 1) >> (30 + (wave_s >> 1))) & 1;
-    } else if (PASS == HA_BWD_DQ_EXACT) {
-      wave_in = !CAUSAL || y_lo <= st_hi;
-      needs_mask = y_hi >= p.n_k || (CAUSAL && y_hi > st_lo);
-    } else if (PASS == HA_BWD_DKV_EXACT) {
-      wave_in = !CAUSAL || y_hi >= st_lo;
-      needs_mask = y_hi >= p.n_q || (CAUSAL && y_lo < st_hi);
-    }
-
-    // One chunk of one wave as straight-line code, one copy with the mask and one without: the
-    // scheduler is free to mix the soft-max arithmetic of one 32-row half with the MFMAs of the other
-    // (forcing a particular interleave with scheduling groups made no difference).
-    auto chunk_body = [&](auto masked_tag) {
-      constexpr bool MASKED = decltype(masked_tag)::value;
-      const unsigned char* const y1 = lds_y1[buf];
-      const unsigned char* const y2 = lds_y2[buf];
-      f32x16 s[2], dp[2];
-#pragma unroll
-      for (int rb = 0; rb < 2; ++rb) {
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          s[rb][i] = 0.f;
-          dp[rb][i] = 0.f;
-        }
-        if (!KEY_ST) dp[rb] = neg_d;
-        if (FOLD_D) {
-          // dP' starts from -D of its streamed query (accumulator element 4g + e is row 8g + 4 hi + e of the
-          // 32-row block): the MFMAs then leave dP - D, and dS' = P' (dP - D) is one product; its factor
-          // `scale` is applied to the sums of dK at the end
-#pragma unroll
-          for (int g = 0; g < 4; ++g) {
-            const f32x4 nd = *reinterpret_cast<const f32x4*>(&lds_delta[buf][rb * 32 + g * 8 + hi * 4]);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) dp[rb][g * 4 + e] = nd[e];
-          }
-        }
-#pragma unroll
-        for (int ks = 0; ks < KSTEPS; ++ks) {
-          const vec8 a1 = lds_read_k<T>(y1, off_rows[ks] + rb * 32 * D * 2);
-          const vec8 a2 = lds_read_k<T>(y2, off_rows[ks] + rb * 32 * D * 2);
-          s[rb] = Mfma<T>::run(a1, x1f[ks], s[rb]);
-          dp[rb] = Mfma<T>::run(a2, x2f[ks], dp[rb]);
-        }
-      }
-
-      // P' and dS' of the lane's 32 (streamed row, stationary row) pairs, rounded to the input type.
-      // Only chunks that touch the diagonal or the end of the sequence pay for the mask.
-      vec8 pb[2][2], dsb[2][2];
-      {
-#pragma unroll
-        for (int rb = 0; rb < 2; ++rb)
-#pragma unroll
-          for (int g = 0; g < 4; ++g) {
-            const int r0 = rb * 32 + g * 8 + hi * 4;  // streamed rows r0..r0+3 of the chunk
-            f32x4 l4 = {st_lse2, st_lse2, st_lse2, st_lse2}, d4 = {st_delta, st_delta, st_delta, st_delta};
-            if (KEY_ST) l4 = *reinterpret_cast<const f32x4*>(&lds_lse[buf][r0]);
-            if (KEY_ST && !FOLD_D) d4 = *reinterpret_cast<const f32x4*>(&lds_delta[buf][r0]);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              const int i = g * 4 + e;
-              float pv = __builtin_amdgcn_exp2f(__builtin_fmaf(s[rb][i], p.scale_log2, -l4[e]));
-              if (MASKED) {
-                bool ok = true;
-                if (PASS == HA_BWD_DQ_EXACT) {
-                  const int key = cc * YC + r0 + e;
-                  ok = key < p.n_k && (!CAUSAL || key <= st_pos);
-                } else if (PASS == HA_BWD_DKV_EXACT) {
-                  const int query = y_first + cc * YC + r0 + e;
-                  ok = query < p.n_q && (!CAUSAL || st_pos <= query);
-                }
-                pv = ok ? pv : 0.f;
-              }
-              // d4 holds D * scale: dS = P (dP - D) scale in one FMA and one product; the gathered dK/dV passes
-              // hold dP - D in dp already
-              const float dsv = (FOLD_D || !KEY_ST) ? pv * dp[rb][i] : pv * __builtin_fmaf(dp[rb][i], p.scale, -d4[e]);
-              pb[rb][i >> 3][i & 7] = (T)pv;
-              dsb[rb][i >> 3][i & 7] = (T)dsv;
-            }
-          }
-      }
-
-      // the products that contract over the streamed rows
-#pragma unroll
-      for (int rb = 0; rb < 2; ++rb)
-#pragma unroll
-        for (int kk = 0; kk < 2; ++kk)
-#pragma unroll
-          for (int db = 0; db < DB; ++db) {
-            const int row_off = (rb * 32 + kk * 16) * D * 2;
-            const vec8 t1 = bwd_read_tr<T>(y1, off_tr_lo[db] + row_off, off_tr_hi[db] + row_off);
-            acc1[db] = Mfma<T>::run(t1, dsb[rb][kk], acc1[db]);
-            if (KEY_ST) {
-              const vec8 t2 = bwd_read_tr<T>(y2, off_tr_lo[db] + row_off, off_tr_hi[db] + row_off);
-              acc2[db] = Mfma<T>::run(t2, pb[rb][kk], acc2[db]);
-            }
-          }
-    };
-    // the passes whose pairs are masked one by one: the diagonal and the end of the sequence in exact
-    // attention (the sampled keys' pass handles the end of its query range through L)
-    constexpr bool CAN_MASK = PASS == HA_BWD_DQ_EXACT || PASS == HA_BWD_DKV_EXACT;
-    if (wave_in) {
-      if (CAN_MASK && needs_mask)
-        chunk_body(std::true_type{});
-      else
-        chunk_body(std::false_type{});
-    }
-  }
-
-  if (FOLD_D || !KEY_ST) {
-    // dK (dQ) was summed without the factor `scale` of dS
-#pragma unroll
-    for (int db = 0; db < DB; ++db)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) acc1[db][i] *= p.scale;
-  }
-
-  // ---- results -------------------------------------------------------------------------------
-  // A lane holds 4 consecutive elements of 16 pieces of ONE row.  In the gathered passes, whose rows lie
-  // all over the head, each wave turns its 32 x D results around in LDS (its quarter of the first tile
-  // buffer pair, free once every wave has left the loop), so that 8 or 16 consecutive lanes write one
-  // whole row, 16 bytes each, instead of every lane 8 bytes of its own row per instruction (3.5 %; the
-  // exact passes, whose rows are neighbours anyway, lose 1-3 % to the extra barrier and registers).
-  constexpr bool TURN_RESULTS = PASS == HA_BWD_DQ_BLOCK || PASS == HA_BWD_DKV_BLOCK;
-  if (TURN_RESULTS) {
-    constexpr int ROWS_PER_STORE = 64 / PR;
-    constexpr int NJ = 32 / ROWS_PER_STORE;
-    const int row_in_store = lane / PR, out_piece = lane % PR;
-    unsigned char* const base1 =
-        KEY_ST ? (unsigned char*)((T*)p.dk + b * p.dk_sb + hk * p.dk_sh + k_row0 * p.dk_sn)
-               : (unsigned char*)((T*)p.dq + b * p.dq_sb + h0 * p.dq_sh + q_row0 * p.dq_sn);
-    unsigned char* const base2 = (unsigned char*)((T*)p.dv + b * p.dv_sb + hk * p.dv_sh + k_row0 * p.dv_sn);
-    const int64_t stride1 = (KEY_ST ? p.dk_sn : p.dq_sn) * 2, stride2 = p.dv_sn * 2;
-    // the rows this lane writes (a piece of NJ rows of its wave), and, when the call adds to what is there,
-    // their present values: all asked for at once, ahead of the barrier and the turn through LDS (one
-    // memory round trip; fetched where each row is stored they were NJ round trips per tensor, one after
-    // the other, and a third of the block pass's time)
-    int rows_j[NJ];
-    bool valid_j[NJ];
-    vec8 old1[NJ], old2[NJ];
-#pragma unroll
-    for (int j = 0; j < NJ; ++j) {
-      const int r = j * ROWS_PER_STORE + row_in_store;
-      rows_j[j] = __shfl(st_row, r);  // lanes past the end hold the first row: a valid address
-      valid_j[j] = __shfl((int)st_valid, r) != 0;
-    }
-    if (p.accumulate) {
-#pragma unroll
-      for (int j = 0; j < NJ; ++j) {
-        old1[j] = *reinterpret_cast<const vec8*>(base1 + rows_j[j] * stride1 + out_piece * 16);
-        if (KEY_ST) old2[j] = *reinterpret_cast<const vec8*>(base2 + rows_j[j] * stride2 + out_piece * 16);
-      }
-    }
-    __syncthreads();
-    unsigned char* const turn = lds_y1[0] + wave_s * (32 * D * 2);
-    auto store_rows = [&](const f32x16 (&acc)[DB], unsigned char* base, int64_t row_stride_bytes, const vec8 (&old)[NJ]) {
-      // [row][D] in the output type, 16-byte pieces XOR-ed with the row number
-#pragma unroll
-      for (int db = 0; db < DB; ++db)
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          vec4 o;
-#pragma unroll
-          for (int e = 0; e < 4; ++e) o[e] = (T)acc[db][g * 4 + e];
-          const int piece = (4 * db + g) ^ (col & (PR - 1));
-          *reinterpret_cast<vec4*>(turn + col * (D * 2) + piece * 16 + hi * 8) = o;
-        }
-#pragma unroll
-      for (int j = 0; j < NJ; ++j) {
-        const int r = j * ROWS_PER_STORE + row_in_store;
-        vec8 o = *reinterpret_cast<const vec8*>(turn + r * (D * 2) + ((out_piece ^ (r & (PR - 1))) << 4));
-        if (p.accumulate) {
-#pragma unroll
-          for (int e = 0; e < 8; ++e) o[e] = (T)((float)o[e] + (float)old[j][e]);
-        }
-        if (valid_j[j]) *reinterpret_cast<vec8*>(base + rows_j[j] * row_stride_bytes + out_piece * 16) = o;
-      }
-    };
-    store_rows(acc1, base1, stride1, old1);
-    if (KEY_ST) store_rows(acc2, base2, stride2, old2);
-  }
-  if (!TURN_RESULTS && !KEY_ST && st_valid) {
-    unsigned char* const dqb = (unsigned char*)((T*)p.dq + b * p.dq_sb + h0 * p.dq_sh + q_row0 * p.dq_sn) + (int64_t)st_row * p.dq_sn * 2;
-#pragma unroll
-    for (int db = 0; db < DB; ++db)
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        vec4* const dst = reinterpret_cast<vec4*>(dqb + (32 * db + 8 * g + 4 * hi) * 2);
-        vec4 o;
-        if (p.accumulate) {
-          const vec4 old = *dst;
-#pragma unroll
-          for (int e = 0; e < 4; ++e) o[e] = (T)(acc1[db][g * 4 + e] + (float)old[e]);
-        } else {
-#pragma unroll
-          for (int e = 0; e < 4; ++e) o[e] = (T)acc1[db][g * 4 + e];
-        }
-        *dst = o;
-      }
-  } else if (!TURN_RESULTS && (PASS == HA_BWD_DKV_EXACT || PASS == HA_BWD_DKV_BLOCK) && st_valid) {
-    // complete sums (of the blocks: every key is in exactly one tile of the sorted order): straight to dk, dv
-    unsigned char* const dkb = (unsigned char*)((T*)p.dk + b * p.dk_sb + hk * p.dk_sh + k_row0 * p.dk_sn) + (int64_t)st_row * p.dk_sn * 2;
-    unsigned char* const dvb = (unsigned char*)((T*)p.dv + b * p.dv_sb + hk * p.dv_sh + k_row0 * p.dv_sn) + (int64_t)st_row * p.dv_sn * 2;
-#pragma unroll
-    for (int db = 0; db < DB; ++db)
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        vec4* const dst_k = reinterpret_cast<vec4*>(dkb + (32 * db + 8 * g + 4 * hi) * 2);
-        vec4* const dst_v = reinterpret_cast<vec4*>(dvb + (32 * db + 8 * g + 4 * hi) * 2);
-        vec4 ok_, ov_;
-        if (p.accumulate) {
-          const vec4 old_k = *dst_k, old_v = *dst_v;
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            ok_[e] = (T)(acc1[db][g * 4 + e] + (float)old_k[e]);
-            ov_[e] = (T)(acc2[db][g * 4 + e] + (float)old_v[e]);
-          }
-        } else {
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            ok_[e] = (T)acc1[db][g * 4 + e];
-            ov_[e] = (T)acc2[db][g * 4 + e];
-          }
-        }
-        *dst_k = ok_;
-        *dst_v = ov_;
-      }
-  }
-  if (PASS == HA_BWD_DKV_SAMPLED) {
-    // Sampled keys: partial sums over one range of queries of one query head, added with atomics to the
-    // fp32 row of the key's SLOT in the sample list (batch, kv_heads, sample_size, D).  Each wave turns its
-    // 32 x D results around in LDS (its quarter of the tile buffers, free once every wave has left the
-    // loop) so that one atomic instruction covers 64 consecutive floats of one row instead of one float of
-    // each of 64 rows.
-    __syncthreads();
-    float* const turn = reinterpret_cast<float*>(wave_s < 2 ? lds_y1[wave_s] : lds_y2[wave_s - 2]);
-    const int64_t head_base = ((int64_t)(b * kv_heads + hk) * p.segs + seg) * p.sample_size * D;
-#pragma unroll
-    for (int which = 0; which < 2; ++which) {
-      float* const dst = (which == 0 ? p.dk32 : p.dv32) + head_base;
-      // [key][D] fp32, the 16-byte pieces of a row XOR-ed with the key number: conflict-free both ways
-#pragma unroll
-      for (int db = 0; db < DB; ++db)
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          const f32x16& a = which == 0 ? acc1[db] : acc2[db];
-          const int piece = (8 * db + 2 * g + hi) ^ (col & 15);
-          *reinterpret_cast<f32x4*>(turn + col * D + piece * 4) = f32x4{a[g * 4], a[g * 4 + 1], a[g * 4 + 2], a[g * 4 + 3]};
-        }
-      for (int r = 0; r < 32; ++r) {
-        const int slot = tile * ST_ROWS + wave_s * 32 + r;  // < sample_size: a multiple of 128
-#pragma unroll
-        for (int part = 0; part < D / 64; ++part) {
-          const int dd = part * 64 + lane;
-          const float val = turn[r * D + (((dd >> 2) ^ (r & 15)) << 2) + (dd & 3)];
-          unsafeAtomicAdd(dst + (int64_t)slot * D + dd, val);
-        }
-      }
+    if (t_short != t_long) {  // an odd number of tiles: the middle one has no partner
+      // the first tile's last reads of the staging areas and the streamed tiles are behind every wave
+      __syncthreads();
+      const int tile = t_short;
+#include "attn_bwd_tile.inc"
     }
   }
 }
@@ -957,9 +399,10 @@ int run_flash_bwd(const ha_attn_operands& t, bool causal, const ha_attn_grads& g
   const int64_t bh = t.batch * t.heads * t.segs, bhk = t.batch * (t.heads / t.kv_group) * t.segs;
   const int64_t q_tiles = (t.n_q + ST_ROWS - 1) / ST_ROWS, k_tiles = (t.n_k + ST_ROWS - 1) / ST_ROWS;
   if (causal) {
-    st = launch_pass<T, D, HA_BWD_DQ_EXACT, true>(p, bh * q_tiles, stream, "ha_flash_attn_bwd: dq");
+    // one workgroup per pair of stationary tiles
+    st = launch_pass<T, D, HA_BWD_DQ_EXACT, true>(p, bh * ((q_tiles + 1) / 2), stream, "ha_flash_attn_bwd: dq");
     if (st != HA_OK) return st;
-    st = launch_pass<T, D, HA_BWD_DKV_EXACT, true>(p, bhk * k_tiles, stream, "ha_flash_attn_bwd: dk, dv");
+    st = launch_pass<T, D, HA_BWD_DKV_EXACT, true>(p, bhk * ((k_tiles + 1) / 2), stream, "ha_flash_attn_bwd: dk, dv");
   } else {
     st = launch_pass<T, D, HA_BWD_DQ_EXACT, false>(p, bh * q_tiles, stream, "ha_flash_attn_bwd: dq");
     if (st != HA_OK) return st;
