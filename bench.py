@@ -732,9 +732,16 @@ def main():
                 power = sustained(lambda: o.backward(do, retain_graph=True), 1.0, torch)
             return f, bw, power
 
+        torch.cuda.synchronize()
+        torch.cuda.reset_peak_memory_stats()
+        held = torch.cuda.memory_allocated()
         f_ms, b_ms, b_power = fwd_bwd_ms(lambda a, b_, c: m(a, b_, c, causal=w["causal"]), (q, k, v), 5,
                                          sustain=not args.no_sustained)
-        backward = {"fwd_autograd_ms": round(f_ms, 3), "bwd_ms": round(b_ms, 3), "fwd_bwd_ms": round(f_ms + b_ms, 3)}
+        backward = {"fwd_autograd_ms": round(f_ms, 3), "bwd_ms": round(b_ms, 3), "fwd_bwd_ms": round(f_ms + b_ms, 3),
+                    # device memory the forward + backward of the module took on top of what was held before
+                    # (inputs and the bench's own tensors), and the size of q, k, v together for comparison
+                    "peak_extra_memory_GB": round((torch.cuda.max_memory_allocated() - held) / 1e9, 3),
+                    "qkv_GB": round(sum(x.numel() * x.element_size() for x in (q, k, v)) / 1e9, 3)}
         if b_power:
             backward["sustained"] = b_power
         if not args.no_exact and hk == h:

@@ -80,6 +80,7 @@ class AttnOperands(ctypes.Structure):
         ("lse_stride_b", ctypes.c_int64), ("lse_stride_h", ctypes.c_int64),
         ("segs", ctypes.c_int64), ("seg_stride_rows", ctypes.c_int64),
         ("q_seg_offset", ctypes.c_int64), ("k_seg_offset", ctypes.c_int64),
+        ("o_seg_stride_rows", ctypes.c_int64), ("o_seg_offset", ctypes.c_int64),
         ("kv_group", ctypes.c_int64),
         ("scale", ctypes.c_float), ("dtype", ctypes.c_int),
     ]
@@ -168,7 +169,7 @@ def _declare(lib):
     lib.ha_forward.argtypes = [ctypes.POINTER(ForwardArgs), vp]
     lib.ha_lse_merge_levels.restype = ci
     lib.ha_lse_merge_levels.argtypes = [vp, vp, ctypes.POINTER(vp), ctypes.POINTER(vp), ctypes.POINTER(vp), vp, vp, vp,
-                                        ci, i64, i64, i64, ci, vp]
+                                        ci, i64, i64, i64, ci, ci, vp]
     lib.ha_power_probe.restype = ci
     lib.ha_power_probe.argtypes = [ci, i64, ci, vp, vp]
     lib.ha_forward_sort.restype = ci

@@ -88,6 +88,8 @@ void fill_params(const ha_attn_operands& t, ha_attn_kernel_params& p) {
   p.ki_sb = p.ki_sh = p.ki_sn = 0;
   p.si_sb = p.si_sh = 0;
   p.seg_stride = t.seg_stride_rows; p.q_seg_off = t.q_seg_offset; p.k_seg_off = t.k_seg_offset;
+  p.o_seg_stride = t.o_seg_stride_rows > 0 ? t.o_seg_stride_rows : t.seg_stride_rows;
+  p.o_seg_off = t.o_seg_stride_rows > 0 ? t.o_seg_offset : t.q_seg_offset;
   p.batch = (int)t.batch; p.heads = (int)t.heads; p.segs = (int)t.segs; p.kv_group = (int)t.kv_group;
   p.n_q = (int)t.n_q; p.n_k = (int)t.n_k;
   p.block_tiles = 1; p.sample_chunks = 0; p.smooth = 0; p.accumulate = 0; p.idx64 = 0;
@@ -286,6 +288,7 @@ int check_forward(const ha_forward_args& a) {
 
 // (batch, heads, n, d) operands of the whole forward pass: contiguous unless strides are given
 void forward_operands(const ha_forward_args& a, ha_attn_operands& t) {
+  t = ha_attn_operands{};  // segments as the callers set them; out and lse follow q (o_seg_stride_rows = 0)
   t.q = a.q; t.k = a.k; t.v = a.v; t.out = a.out; t.lse = a.lse;
   t.batch = a.batch; t.heads = a.heads; t.d = a.d; t.dv = a.dv;
   t.q_stride_b = a.heads * a.n * a.d; t.q_stride_h = a.n * a.d; t.q_stride_n = a.d;

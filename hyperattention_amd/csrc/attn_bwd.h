@@ -41,6 +41,7 @@ struct ha_attn_bwd_params {
   int batch, heads, kv_group;
   int segs;                                // segments per head, as in the forward
   int64_t seg_stride, q_seg_off, k_seg_off;  // rows
+  int64_t o_seg_stride, o_seg_off;           // the forward's out / lse (the query side's unless packed)
   int n_q, n_k;
   int block_tiles;  // ceil(block_size / 128)
   int sample_size;

@@ -143,6 +143,7 @@ __global__ __launch_bounds__(WG_THREADS, (D <= 64 || PASS == HA_BWD_DQ_BLOCK ? 2
   // first row of this segment in the query-side and in the key-side tensors
   const int64_t q_row0 = p.q_seg_off + (int64_t)seg * p.seg_stride;
   const int64_t k_row0 = p.k_seg_off + (int64_t)seg * p.seg_stride;
+  const int64_t o_row0 = p.o_seg_off + (int64_t)seg * p.o_seg_stride;  // in the forward's out and lse
 
   // query-side tensors of query head h0 + gi
   auto q_head = [&](int gi) { return (const unsigned char*)((const T*)p.q + b * p.q_sb + (h0 + gi) * p.q_sh + q_row0 * p.q_sn); };
@@ -327,6 +328,8 @@ void fill_bwd_params(const ha_attn_operands& t, const ha_attn_grads& g, const Wo
   p.si_sb = p.si_sh = 0;
   p.batch = (int)t.batch; p.heads = (int)t.heads; p.kv_group = (int)t.kv_group;
   p.segs = (int)t.segs; p.seg_stride = t.seg_stride_rows; p.q_seg_off = t.q_seg_offset; p.k_seg_off = t.k_seg_offset;
+  p.o_seg_stride = t.o_seg_stride_rows > 0 ? t.o_seg_stride_rows : t.seg_stride_rows;
+  p.o_seg_off = t.o_seg_stride_rows > 0 ? t.o_seg_offset : t.q_seg_offset;
   p.n_q = (int)t.n_q; p.n_k = (int)t.n_k;
   p.block_tiles = 1; p.sample_size = 0; p.smooth = 0; p.idx64 = 0;
   p.accumulate = g.accumulate != 0;

@@ -44,6 +44,9 @@ struct ha_attn_kernel_params {
   // past this number names a row that is not there (the zero row the causal recursion appends to an odd
   // length, hyper_attention.py:61-64); it is placed like any other row and its result is dropped.
   int n_q_last;
+  // first row of segment g in the out / lse tensors: o_seg_off + g * o_seg_stride (= the query side's unless
+  // the caller packs the rows a call writes)
+  int64_t o_seg_off, o_seg_stride;
   // Streaming gathered kernel: consecutive query tiles of one (virtual) head per workgroup (the last
   // workgroup of a head may have fewer); 1: the one-tile kernels
   int tiles_per_wg;

@@ -299,6 +299,7 @@ __global__ __launch_bounds__(WaveShape<D>::THREADS, 2) void ha_attn_fwd_kernel(c
   // ---- rows of this segment -----------------------------------------------------------------------
   int n_q = p.n_q, n_k = p.n_k;
   int64_t seg_q_row = p.q_seg_off + (int64_t)seg * p.seg_stride, seg_k_row = p.k_seg_off + (int64_t)seg * p.seg_stride;
+  int64_t seg_o_row = p.o_seg_off + (int64_t)seg * p.o_seg_stride;  // first row of the segment in out / lse
   if (!GATHER && p.rag_levels >= 0) {
     // walk down from the whole sequence: where the segment starts and how many of its rows exist
     int start = 0, real = p.rag_n;
@@ -321,6 +322,7 @@ __global__ __launch_bounds__(WaveShape<D>::THREADS, 2) void ha_attn_fwd_kernel(c
       seg_q_row = seg_k_row = start;
       n_q = n_k = real;
     }
+    seg_o_row = seg_q_row;
   }
   // gathered kernel: entries of the query order from this number on name a row that does not exist
   const int q_rows_exist = (GATHER && seg == p.segs - 1) ? p.n_q_last : n_q;

@@ -162,7 +162,7 @@ template <typename T, int MAXL>
 __global__ __launch_bounds__(256) void lse_merge_levels_kernel(const T* __restrict__ o_leaf, const float* __restrict__ lse_leaf,
                                                                T* __restrict__ out, float* __restrict__ lse_out,
                                                                float* __restrict__ leaf_shifted, MergeLevels lv,
-                                                               int64_t rows, int64_t n, int pieces) {
+                                                               int64_t rows, int64_t n, int pieces, int packed) {
   typedef typename ElemTraits<T>::vec8 vec8;
   const int64_t item = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   const int64_t row = item / pieces;
@@ -177,6 +177,15 @@ __global__ __launch_bounds__(256) void lse_merge_levels_kernel(const T* __restri
   vec8 r = *reinterpret_cast<const vec8*>(o_leaf + at);
   float c_of[MAXL], x_of[MAXL];
   vec8 v_of[MAXL];
+  // Row of the level-j arrays that holds this row's result.  Packed arrays keep only the rows a level writes,
+  // the second halves of its segments of n >> j rows one after the other: (batch * heads, n / 2) rows.
+  const int64_t seq = row / n;
+  const uint32_t r_in = (uint32_t)(row - seq * n);
+  auto level_row = [&](int j) -> int64_t {
+    if (!packed) return row;
+    const uint32_t len = (uint32_t)(n >> j), half = len >> 1;
+    return seq * (n >> 1) + (int64_t)(r_in / len) * half + (r_in % len - half);
+  };
   // every load first, so that they are all in flight before the chain of weights (each level's weight needs
   // the log-sum-exp the deeper levels left) starts
 #pragma unroll
@@ -184,8 +193,9 @@ __global__ __launch_bounds__(256) void lse_merge_levels_kernel(const T* __restri
     c_of[j] = 1.0f;
     x_of[j] = 0.0f;
     if (j < lv.levels && ((leaf_no >> (lv.levels - 1 - j)) & 1u)) {
-      x_of[j] = lv.lse_un[j][row];
-      v_of[j] = *reinterpret_cast<const vec8*>((const T*)lv.o_un[j] + at);
+      const int64_t lr = level_row(j);
+      x_of[j] = lv.lse_un[j][lr];
+      v_of[j] = *reinterpret_cast<const vec8*>((const T*)lv.o_un[j] + lr * pieces * 8 + piece * 8);
     }
   }
 #pragma unroll
@@ -206,7 +216,7 @@ __global__ __launch_bounds__(256) void lse_merge_levels_kernel(const T* __restri
 #pragma unroll
   for (int j = 0; j < MAXL; ++j) {
     if (j < lv.levels && ((leaf_no >> (lv.levels - 1 - j)) & 1u)) {
-      lv.shifted[j][row] = x_of[j] - log1pf(-c_of[j]) - log_w;
+      lv.shifted[j][level_row(j)] = x_of[j] - log1pf(-c_of[j]) - log_w;
       log_w += logf(c_of[j]);
     }
   }
@@ -218,7 +228,7 @@ __global__ __launch_bounds__(256) void lse_merge_levels_kernel(const T* __restri
 extern "C" int ha_lse_merge_levels(const void* o_leaf, const float* lse_leaf, const void* const* o_un,
                                    const float* const* lse_un, float* const* lse_shifted, float* leaf_shifted,
                                    void* out, float* lse_out, int levels, int64_t batch_heads, int64_t n, int64_t d,
-                                   int dtype, void* stream) {
+                                   int dtype, int packed, void* stream) {
   HA_REQUIRE(o_leaf && lse_leaf && out && lse_out && (levels == 0 || (o_un && lse_un)), HA_ERR_NULL,
              "ha_lse_merge_levels: null pointer");
   HA_REQUIRE(dtype == HA_F16 || dtype == HA_BF16, HA_ERR_DTYPE, "ha_lse_merge_levels: Only support fp16 and bf16");
@@ -252,7 +262,7 @@ extern "C" int ha_lse_merge_levels(const void* o_leaf, const float* lse_leaf, co
   hipStream_t s = (hipStream_t)stream;
 #define HA_MERGE_LEVELS(TT, LL)                                                                                  \
   hipLaunchKernelGGL((lse_merge_levels_kernel<TT, LL>), grid, dim3(256), 0, s, (const TT*)o_leaf, lse_leaf, (TT*)out, \
-                     lse_out, leaf_shifted, lv, rows, n, pieces)
+                     lse_out, leaf_shifted, lv, rows, n, pieces, packed)
   if (dtype == HA_F16) {
     if (levels <= 8) HA_MERGE_LEVELS(f16_t, 8); else HA_MERGE_LEVELS(f16_t, MERGE_MAX_LEVELS);
   } else {

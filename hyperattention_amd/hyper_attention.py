@@ -32,7 +32,7 @@ class _CausalRecursionFunc(torch.autograd.Function):
     gradient (src/hyper_attn_triton.py:922-945).  What differs is the bookkeeping.  All rows are hashed
     in one launch and ranked once for all levels (ha_forward_sort).  Every call reads and writes its
     segments of the whole (batch, heads, n, d) tensors through the C entry points; the result of level j
-    is kept in o_un[j] at the rows of the output it belongs to.  One pass merges the leaf and level
+    (the second halves of its segments: n/2 rows per head) is kept packed in o_un[j], (batch, heads, n/2, d).  One pass merges the leaf and level
     results of every row (ha_lse_merge_levels) and, on the way, turns the merge weights into the shifted
     log-sum-exps that the backward hands to each call in place of a weighted copy of the output gradient.
     In the backward the gradients of the calls are accumulated by the kernels (`accumulate`), so there
@@ -50,6 +50,8 @@ class _CausalRecursionFunc(torch.autograd.Function):
             half = lens[j + 1]
             t.n_q = t.n_k = half
             t.segs, t.seg_stride_rows, t.q_seg_offset, t.k_seg_offset = 1 << j, lens[j], half, 0
+            # out and lse hold the rows the call writes and nothing else: segment after segment
+            t.o_seg_stride_rows, t.o_seg_offset = half, 0
         return t
 
     @staticmethod
@@ -59,7 +61,7 @@ class _CausalRecursionFunc(torch.autograd.Function):
         hk, half, segs = key.shape[1], lens[j + 1], 1 << j
         a = _lib.BlockAttnArgs()
         a.t = _CausalRecursionFunc._segments(
-            ops._operands(query, key, value, out, lse, scale, layout_bnhd=False, lse_row_stride=n), lens, j)
+            ops._operands(query, key, value, out, lse, scale, layout_bnhd=False, lse_row_stride=n // 2), lens, j)
         a.q_idx, a.k_idx, a.idx_type = q_idx.data_ptr(), k_idx.data_ptr(), ops._idx_code(q_idx)
         a.q_idx_stride_b, a.q_idx_stride_h, a.q_idx_stride_n = h * segs * half, segs * half, 1
         a.k_idx_stride_b, a.k_idx_stride_h, a.k_idx_stride_n = hk * segs * half, segs * half, 1
@@ -93,7 +95,8 @@ class _CausalRecursionFunc(torch.autograd.Function):
         f32 = dict(device=dev, dtype=torch.float32)
         hashed = [not module.min_seq_len > lens[j + 1] for j in range(levels)]  # hyper_attention.py:109
         segments = _CausalRecursionFunc._segments
-        operands = lambda out, lse: ops._operands(query, key, value, out, lse, scale, layout_bnhd=False, lse_row_stride=n)
+        operands = lambda out, lse, rows=n: ops._operands(query, key, value, out, lse, scale, layout_bnhd=False,
+                                                           lse_row_stride=rows)
 
         q_idx = k_idx = [None] * levels
         if any(hashed):
@@ -101,9 +104,10 @@ class _CausalRecursionFunc(torch.autograd.Function):
                                             lsh_num_projs=module.lsh_num_projs, min_seq_len=module.min_seq_len)
         sampled = _CausalRecursionFunc._sampled(module, query, lens, hashed)
         o_leaf, lse_leaf = torch.empty_like(query), torch.empty((b, h, n), **f32)
-        o_un = torch.empty((levels, b, h, n, d), device=dev, dtype=query.dtype)
-        lse_un = torch.empty((levels, b, h, n), **f32)
-        lse_shifted, leaf_shifted = torch.empty((levels, b, h, n), **f32), torch.empty((b, h, n), **f32)
+        # level results, packed: a level writes the second halves of its segments, n/2 rows per head
+        o_un = torch.empty((levels, b, h, n // 2, d), device=dev, dtype=query.dtype)
+        lse_un = torch.empty((levels, b, h, n // 2), **f32)
+        lse_shifted, leaf_shifted = torch.empty((levels, b, h, n // 2), **f32), torch.empty((b, h, n), **f32)
         out, lse = torch.empty_like(query), torch.empty((b, h, n), **f32)
         with torch.cuda.device(dev):
             # leaves: exact causal attention on every segment of lens[levels] rows
@@ -115,13 +119,13 @@ class _CausalRecursionFunc(torch.autograd.Function):
                                                          q_idx[j], k_idx[j], sampled)
                     _lib.check(lib.ha_block_attn_fwd(ctypes.byref(a), stream))
                 else:
-                    t = segments(operands(o_un[j], lse_un[j]), lens, j)
+                    t = segments(operands(o_un[j], lse_un[j], n // 2), lens, j)
                     _lib.check(lib.ha_flash_attn_fwd(ctypes.byref(t), 0, stream))
             ptrs = lambda x: (ctypes.c_void_p * max(levels, 1))(*[x[j].data_ptr() for j in range(levels)])
             _lib.check(lib.ha_lse_merge_levels(
                 o_leaf.data_ptr(), lse_leaf.data_ptr(), ptrs(o_un), ptrs(lse_un), ptrs(lse_shifted),
                 leaf_shifted.data_ptr(), out.data_ptr(), lse.data_ptr(), levels, b * h, n, d, ops._dtype_code(query),
-                stream))
+                1, stream))
 
         tensors = [query, key, value, o_leaf, leaf_shifted, o_un, lse_shifted]
         if sampled is not None:
@@ -171,7 +175,7 @@ class _CausalRecursionFunc(torch.autograd.Function):
                     _lib.check(lib.ha_block_attn_bwd(ctypes.byref(a), ctypes.byref(g), stream))
                 else:
                     t = segments(ops._operands(query, key, value, o_un[j], lse_shifted[j], scale, layout_bnhd=False,
-                                               lse_row_stride=n), lens, j)
+                                               lse_row_stride=n // 2), lens, j)
                     g, ws = ops._attn_grads(t, dout, dq, dk, dv, layout_bnhd=False, accumulate=True)
                     _lib.check(lib.ha_flash_attn_bwd(ctypes.byref(t), 0, ctypes.byref(g), stream))
         return None, None, dq, dk, dv, None

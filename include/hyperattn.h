@@ -124,6 +124,10 @@ typedef struct {
   int64_t o_stride_b, o_stride_h, o_stride_n;
   int64_t lse_stride_b, lse_stride_h;
   int64_t segs, seg_stride_rows, q_seg_offset, k_seg_offset;
+  /* out and lse of segment g start at row o_seg_offset + g*o_seg_stride_rows of THEIR tensors when
+   * o_seg_stride_rows > 0 (a caller that keeps only the rows a call writes, e.g. the second halves of the
+   * segments of one level of the causal recursion, packed); 0: they follow q (the two fields above) */
+  int64_t o_seg_stride_rows, o_seg_offset;
   int64_t kv_group; /* grouped-query: q head h reads k/v (and k_idx) head h / kv_group; 1 = plain */
   float scale;    /* softmax scale; <= 0 or NaN is an error (callers resolve the default)  */
   int dtype;      /* ha_dtype                                                               */
@@ -259,7 +263,10 @@ int ha_lse_merge_segments(const void* attn1, const float* lse1, const void* attn
  * o_leaf, lse_leaf: exact causal attention of the leaves; o_un[j], lse_un[j] (j < levels, 0 = whole
  * sequence): result of the un-masked call of level j.  Every tensor has the layout of the whole
  * (batch_heads, n, d) / (batch_heads, n) contiguous tensors; level j only uses the rows in the second half
- * of each segment of n / 2^j rows.  out, lse_out: the merged result (not in place).
+ * of each segment of n / 2^j rows.  With packed != 0 the level arrays (o_un[j], lse_un[j], lse_shifted[j])
+ * hold those rows only, the second halves of the level's segments one after the other: (batch_heads, n/2, d)
+ * and (batch_heads, n/2) (what a call writes with o_seg_stride_rows = n / 2^(j+1), o_seg_offset = 0).
+ * out, lse_out: the merged result (not in place).
  * If leaf_shifted is not NULL, lse_shifted[j] (second halves) and leaf_shifted (all rows) receive
  * lse - log(w), w the total weight the merges give that call's result in `out`: handing a call's backward
  * this log-sum-exp together with the gradient of `out` equals handing it its own log-sum-exp and w times
@@ -268,7 +275,7 @@ int ha_lse_merge_segments(const void* attn1, const float* lse1, const void* attn
 int ha_lse_merge_levels(const void* o_leaf, const float* lse_leaf, const void* const* o_un,
                         const float* const* lse_un, float* const* lse_shifted, float* leaf_shifted,
                         void* out, float* lse_out, int levels, int64_t batch_heads, int64_t n, int64_t d,
-                        int dtype, void* stream);
+                        int dtype, int packed, void* stream);
 
 /* ---------------------------------------------------------------------------------------------
  * Whole forward pass of the module for (batch, heads, n, d) tensors, one call, no host

@@ -195,8 +195,8 @@ def test_merge_levels_argument_errors(lib):
     two = vp(512)
     arr = (vp * 1)(256)
     call = lambda levels, n, d, out=two, lse_out=two, dtype=0, o_un=arr: lib.ha_lse_merge_levels(
-        one, one, o_un, arr, arr, one, out, lse_out, levels, 4, n, d, dtype, None)
-    assert lib.ha_lse_merge_levels(None, None, None, None, None, None, None, None, 0, 1, 128, 64, 0, None) == -1
+        one, one, o_un, arr, arr, one, out, lse_out, levels, 4, n, d, dtype, 0, None)
+    assert lib.ha_lse_merge_levels(None, None, None, None, None, None, None, None, 0, 1, 128, 64, 0, 0, None) == -1
     assert call(1, 256, 64, dtype=3) == -2
     assert call(25, 1 << 25, 64) == -5            # more levels than the kernel is built for
     assert call(1, 256, 60) == -3                 # d % 8

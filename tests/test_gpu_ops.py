@@ -489,10 +489,12 @@ def test_add_self_attentions_is_the_same_with_and_without_grad(ha, dtype):
     assert torch.equal(c_kernel, c_ref.expand_as(c_kernel))
 
 
+@pytest.mark.parametrize("packed", [False, True])
 @pytest.mark.parametrize("dtype,levels", [(torch.float16, 3), (torch.bfloat16, 2), (torch.float16, 0)])
-def test_merge_levels_equals_the_chain_of_segment_merges(ha, dtype, levels):
+def test_merge_levels_equals_the_chain_of_segment_merges(ha, dtype, levels, packed):
     """ha_lse_merge_levels against the per-level in-place merges it stands for (bit for bit), and its shifted
-    log-sum-exps against lse - log(weight) from the weights those merges write."""
+    log-sum-exps against lse - log(weight) from the weights those merges write.  packed: the level arrays hold
+    only the second halves of the level's segments, one after the other."""
     import ctypes
     from hyperattention_amd import _lib
     b, h, d, leaf = 2, 3, 64, 40
@@ -525,9 +527,22 @@ def test_merge_levels_equals_the_chain_of_segment_merges(ha, dtype, levels):
     shifted = torch.full((max(levels, 1), b, h, n), float("nan"), dtype=torch.float32, **dev)
     leaf_shifted = torch.empty_like(lse_leaf)
     ptrs = lambda x: (ctypes.c_void_p * max(levels, 1))(*[x[j].data_ptr() for j in range(levels)])
-    _lib.check(lib.ha_lse_merge_levels(o_leaf.data_ptr(), lse_leaf.data_ptr(), ptrs(o_un), ptrs(lse_un), ptrs(shifted),
-                                       leaf_shifted.data_ptr(), got.data_ptr(), got_lse.data_ptr(), levels, b * h, n, d,
-                                       code, stream))
+    if packed:
+        # (levels, b, h, n/2[, d]): the second halves of the segments of n >> j rows, one after the other
+        second = lambda x, j, tail: x[j].reshape(b, h, 1 << j, 2, n >> (j + 1), *tail)[:, :, :, 1].reshape(b, h, n // 2, *tail)
+        o_pk = torch.stack([second(o_un, j, (d,)) for j in range(levels)]) if levels else o_un[:, :, :, : n // 2]
+        l_pk = torch.stack([second(lse_un, j, ()) for j in range(levels)]) if levels else lse_un[:, :, :, : n // 2]
+        o_pk, l_pk = o_pk.contiguous(), l_pk.contiguous()
+        s_pk = torch.full((max(levels, 1), b, h, n // 2), float("nan"), dtype=torch.float32, **dev)
+        _lib.check(lib.ha_lse_merge_levels(o_leaf.data_ptr(), lse_leaf.data_ptr(), ptrs(o_pk), ptrs(l_pk), ptrs(s_pk),
+                                           leaf_shifted.data_ptr(), got.data_ptr(), got_lse.data_ptr(), levels, b * h, n, d,
+                                           code, 1, stream))
+        for j in range(levels):
+            shifted[j].view(b, h, 1 << j, 2, n >> (j + 1))[:, :, :, 1] = s_pk[j].view(b, h, 1 << j, n >> (j + 1))
+    else:
+        _lib.check(lib.ha_lse_merge_levels(o_leaf.data_ptr(), lse_leaf.data_ptr(), ptrs(o_un), ptrs(lse_un), ptrs(shifted),
+                                           leaf_shifted.data_ptr(), got.data_ptr(), got_lse.data_ptr(), levels, b * h, n, d,
+                                           code, 0, stream))
     torch.cuda.synchronize()
     assert torch.equal(got, out) and torch.equal(got_lse, lse)
     log_w = torch.zeros((b, h, n), dtype=torch.float64, **dev)
