@@ -29,6 +29,12 @@ def get_arguments(argv=None):
     parser.add_argument("--min_log2_seq", type=int, default=10, help="first sequence length of the sweep (2^k)")
     parser.add_argument("--max_log2_seq", type=int, default=17, help="last sequence length of the sweep (2^k)")
     parser.add_argument("--rep", type=int, default=100)
+    # beyond the reference's command line (its shapes are the defaults): other workloads of the same sweep
+    parser.add_argument("--batch_size", type=int, default=1)
+    parser.add_argument("--head_size", type=int, default=24, help="number of heads")
+    parser.add_argument("--dim", type=int, default=64, help="head dim")
+    parser.add_argument("--block_size", type=int, default=256)
+    parser.add_argument("--sample_size", type=int, default=256)
     return parser.parse_args(argv)
 
 
@@ -64,10 +70,11 @@ def run_flash_attn(batch_size, head_size, seq_len, dim, causal, mode="fwd", warm
     return time_mode(lambda: flash_attn_func(q, k, v, None, causal, None)[0], mode, warmup, rep)
 
 
-def run_hyper_attn(batch_size, head_size, seq_len, dim, causal, smooth_block, mode="fwd", warmup=20, rep=100):
+def run_hyper_attn(batch_size, head_size, seq_len, dim, causal, smooth_block, mode="fwd", warmup=20, rep=100,
+                   block_size=256, sample_size=256):
     q, k, v = (torch.randn((batch_size, head_size, seq_len, dim), dtype=torch.bfloat16, device="cuda",
                            requires_grad=mode != "fwd") for _ in range(3))
-    attn = HyperAttention(input_dim=dim, block_size=256, sample_size=256, smooth_block=smooth_block).to(
+    attn = HyperAttention(input_dim=dim, block_size=block_size, sample_size=sample_size, smooth_block=smooth_block).to(
         device="cuda", dtype=q.dtype)
     return time_mode(lambda: attn(q, k, v, causal=causal), mode, warmup, rep)
 
@@ -80,14 +87,15 @@ def main(argv=None):
         sys.exit("flash-cuda is a CUDA package; use --attn_method flash for this library's exact attention")
 
     seq_lens = [2 ** i for i in range(args.min_log2_seq, args.max_log2_seq + 1)]
-    batch_size, head_size, dim = 1, 24, 64
+    batch_size, head_size, dim = args.batch_size, args.head_size, args.dim
     print(f"mode: {args.mode}, attn_method: {args.attn_method}, batch_size: {batch_size}, head_size: {head_size}, dim: {dim}")
     causal = not args.no_causal
     for seq_len in seq_lens:
         if args.attn_method == "flash":
             ms = run_flash_attn(batch_size, head_size, seq_len, dim, causal, args.mode, rep=args.rep)
         else:
-            ms = run_hyper_attn(batch_size, head_size, seq_len, dim, causal, args.smooth_block, args.mode, rep=args.rep)
+            ms = run_hyper_attn(batch_size, head_size, seq_len, dim, causal, args.smooth_block, args.mode, rep=args.rep,
+                                block_size=args.block_size, sample_size=args.sample_size)
         print(f"[{args.mode:<8}], {args.attn_method}, seq_len: {seq_len:<8}, causal: {causal}, "
               f"ms: {ms[0]:.5f} ({ms[1]:.5f}, {ms[2]:.5f}) | ", flush=True)
 

@@ -183,8 +183,9 @@ __global__ __launch_bounds__(256) void lse_merge_levels_kernel(const T* __restri
   const uint32_t r_in = (uint32_t)(row - seq * n);
   auto level_row = [&](int j) -> int64_t {
     if (!packed) return row;
-    const uint32_t len = (uint32_t)(n >> j), half = len >> 1;
-    return seq * (n >> 1) + (int64_t)(r_in / len) * half + (r_in % len - half);
+    // the segment number from the leaf number: shifts only (the leaf length need not be a power of two)
+    const uint32_t len = (uint32_t)(n >> j), half = len >> 1, sg = leaf_no >> (lv.levels - j);
+    return seq * (n >> 1) + (int64_t)sg * half + (r_in - sg * len - half);
   };
   // every load first, so that they are all in flight before the chain of weights (each level's weight needs
   // the log-sum-exp the deeper levels left) starts
