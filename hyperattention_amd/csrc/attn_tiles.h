@@ -77,15 +77,18 @@ __device__ __forceinline__ const unsigned char* row_address(const unsigned char*
 }
 
 // 16-byte piece `piece` of row `row` of a row-major [rows][D] 2-byte tile, XOR-swizzled; byte offset.
-// Q and K tiles (read 16 bytes per lane, 8 consecutive rows at a time) move a piece by the row number
-// mod 8.  V tiles are read by the transposing loads, 16 lanes at a time: 4 consecutive rows x 32
-// bytes; they move a PAIR of pieces by the row number mod 4, so that the four rows fall into four
-// different 32-byte bank groups.
-__device__ __forceinline__ int k_swizzle(int row) { return row & 7; }
+// Q and K tiles are read 16 bytes per lane, 16 lanes (16 consecutive rows, the same piece of each) at a time
+// over the 64 banks: they move a piece by the row number modulo the pieces of a row (8 at D = 64, where rows
+// r and r + 8 still share a bank group: a row is half a bank window; 16 at D = 128, where the 16 rows then
+// fall into 16 different groups).  V tiles are read by the transposing loads, 16 lanes at a time: 4
+// consecutive rows x 32 bytes; they move a PAIR of pieces by the row number mod 4, so that the four rows fall
+// into four different 32-byte bank groups.
+template <int D>
+__device__ __forceinline__ int k_swizzle(int row) { return row & (D / 8 - 1) & 15; }
 __device__ __forceinline__ int v_swizzle(int row) { return (row & 3) << 1; }
 template <int D>
 __device__ __forceinline__ int tile_offset(int row, int piece) {
-  return row * D * 2 + ((piece ^ k_swizzle(row)) << 4);
+  return row * D * 2 + ((piece ^ k_swizzle<D>(row)) << 4);
 }
 template <int D>
 __device__ __forceinline__ int v_tile_offset(int row, int piece) {
