@@ -128,6 +128,27 @@ def test_causal_odd_lengths(ha, monkeypatch, n, msl, block):
     assert_close(lse, rl, "lse")
 
 
+@pytest.mark.parametrize("d,dtype,kv_heads", [(128, torch.bfloat16, 1), (64, torch.float16, 2), (128, torch.float16, 2)])
+def test_one_call_forward_is_the_same_with_streaming_workgroups(ha, monkeypatch, d, dtype, kv_heads):
+    """The whole causal forward with the gathered levels run by workgroups that stream runs of query tiles
+    (forced by the library's measurement switch) equals the forward with one tile per workgroup bit for bit:
+    an odd length (the last query of the last segment of every hashed level is the appended row, which the
+    stream kernel has to drop), resumed partial results at every level, grouped-query heads."""
+    n, msl = 9215, 2304   # -> 9216 -> halves of 4608 and 2304: two hashed levels of 18 and 9 tiles per segment
+    q = _randn((1, 2, n, d), 160, dtype).cuda()
+    k, v = (_randn((1, kv_heads, n, d), s, dtype).cuda() for s in (161, 162))
+    m, _ = _module(ha, d, dtype, 163, block_size=256, sample_size=256, min_seq_len=msl)
+    _no_composed_path(m, monkeypatch)
+    out = {}
+    for tiles in (1, 4):
+        monkeypatch.setenv("HA_STREAM_TILES", str(tiles))
+        attn, lse = m(q, k, v, causal=True, return_lse=True)
+        torch.cuda.synchronize()
+        out[tiles] = (attn.clone(), lse.clone())
+    assert torch.isfinite(out[1][0].float()).all()
+    assert torch.equal(out[1][0], out[4][0]) and torch.equal(out[1][1], out[4][1])
+
+
 def test_causal_odd_length_sort_places_the_appended_row(ha):
     """The query order of every hashed level of an odd length is the stable bucket sort of the segment's rows
     with the appended zero row (bucket of the zero vector: 0) as its last row."""
