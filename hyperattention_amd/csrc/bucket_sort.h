@@ -25,6 +25,7 @@ struct ha_sort_jobs {
   int num_jobs;
   int shift;   // bit offset of the 8-bit digit sorted in this pass
   int idx64;   // output width of this pass
+  int scanned; // set by ha_sort_launch: the histograms hold first output slots (scan launch) rather than counts
 };
 
 int ha_sort_launch(const ha_sort_jobs& jobs, int total_blocks, int total_segments, bool any_multi_chunk,

@@ -6,8 +6,10 @@
 // A segment is cut into chunks of SORT_CHUNK keys, one workgroup each.  Ranking inside a wave
 // uses ballot matching (8 ballots give every lane the set of lanes holding the same 8-bit digit),
 // so skewed key distributions cost the same as uniform ones and no LDS atomics are needed for the
-// order-sensitive part.  Segments longer than one chunk use three launches (per-chunk histograms,
-// per-segment scan, scatter); shorter ones a single launch.  Keys above 255 take one extra
+// order-sensitive part.  Segments longer than one chunk use two launches (per-chunk histograms, then a
+// scatter in which every workgroup adds up the histograms of its segment for itself), and beyond
+// SORT_DIRECT_CHUNKS chunks per segment a third one between them (per-segment scan); shorter ones a single
+// launch.  Keys above 255 take one extra
 // least-significant-digit pass per byte.  Several jobs (for instance all recursion levels of a
 // causal forward) share one launch through a small by-value job table.
 #include "ha_common.h"
@@ -20,6 +22,9 @@ namespace {
 constexpr int SORT_THREADS = 256;
 constexpr int SORT_WAVES = SORT_THREADS / HA_WAVE;
 constexpr int SORT_STEPS = HA_SORT_CHUNK / SORT_THREADS;  // 64-key steps per wave per chunk
+// up to this many chunks per segment a scatter workgroup reads the histograms of all chunks of its segment
+// (256 counters each, from L2) rather than wait for a scan launch that has one workgroup per segment
+constexpr int SORT_DIRECT_CHUNKS = 64;
 
 struct BlockRef {
   int job, seg, chunk;
@@ -180,7 +185,24 @@ __global__ __launch_bounds__(SORT_THREADS) void sort_scatter_kernel(ha_sort_jobs
   for (int w = 0; w < SORT_WAVES; ++w) total += wave_hist[w][tid];
   const uint32_t local_base = block_exclusive_scan(total, wave_totals);
   uint32_t global_base = local_base;
-  if (job.chunks_per_seg > 1) global_base = job.hist[((int64_t)br.seg * job.chunks_per_seg + br.chunk) * 256 + tid];
+  if (job.chunks_per_seg > 1 && jobs.scanned) {
+    global_base = job.hist[((int64_t)br.seg * job.chunks_per_seg + br.chunk) * 256 + tid];
+  } else if (job.chunks_per_seg > 1) {
+    // raw counts: keys tid of the whole segment and of the chunks before this one, eight loads in flight
+    const uint32_t* h = job.hist + (int64_t)br.seg * job.chunks_per_seg * 256 + tid;
+    uint32_t tot = 0, before = 0;
+    for (int c0 = 0; c0 < job.chunks_per_seg; c0 += 8) {
+      uint32_t c[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) c[i] = c0 + i < job.chunks_per_seg ? h[(int64_t)(c0 + i) * 256] : 0u;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        before += c0 + i < br.chunk ? c[i] : 0u;
+        tot += c[i];
+      }
+    }
+    global_base = block_exclusive_scan(tot, wave_totals) + before;
+  }
   to_global[tid] = (int32_t)(global_base - local_base);
   // turn the per-wave counts into per-wave chunk-local first slots
   uint32_t run = local_base;
@@ -375,11 +397,15 @@ int ha_place_units(const ha_place_jobs& jobs, int total_blocks, hipStream_t stre
   return ha_launch_status("ha_forward (place)");
 }
 
-int ha_sort_launch(const ha_sort_jobs& jobs, int total_blocks, int total_segments, bool any_multi_chunk,
+int ha_sort_launch(const ha_sort_jobs& jobs_in, int total_blocks, int total_segments, bool any_multi_chunk,
                    hipStream_t stream) {
+  ha_sort_jobs jobs = jobs_in;
+  int most_chunks = 1;
+  for (int j = 0; j < jobs.num_jobs; ++j) most_chunks = jobs.job[j].chunks_per_seg > most_chunks ? jobs.job[j].chunks_per_seg : most_chunks;
+  jobs.scanned = most_chunks > SORT_DIRECT_CHUNKS;
   if (any_multi_chunk) {
     hipLaunchKernelGGL(sort_hist_kernel, dim3(total_blocks), dim3(SORT_THREADS), 0, stream, jobs);
-    hipLaunchKernelGGL(sort_scan_kernel, dim3(total_segments), dim3(SORT_THREADS), 0, stream, jobs);
+    if (jobs.scanned) hipLaunchKernelGGL(sort_scan_kernel, dim3(total_segments), dim3(SORT_THREADS), 0, stream, jobs);
   }
   hipLaunchKernelGGL(sort_scatter_kernel, dim3(total_blocks), dim3(SORT_THREADS), 0, stream, jobs);
   return ha_launch_status("ha_bucket_argsort");

@@ -80,6 +80,8 @@ def test_hash_golden_vectors(ha):
     (6, 100, 256, "uniform"), (4, 2048, 256, "uniform"), (3, 4096, 256, "skew"), (2, 5000, 64, "uniform"),
     (64, 32768, 256, "uniform"), (2, 65536 + 17, 256, "skew"), (3, 4097, 256, "same"), (2, 3000, 4096, "uniform"),
     (1, 20000, 65536, "uniform"),
+    # 64 chunks per segment: every scatter workgroup adds up its segment's histograms; 65: the scan launch does
+    (2, 64 * 4096, 256, "uniform"), (1, 64 * 4096 + 5, 256, "skew"), (1, 300000, 4096, "uniform"),
 ])
 def test_sort_bit_exact(ha, segs, n, num_keys, kind):
     g = np.random.default_rng(7)
