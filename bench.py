@@ -687,6 +687,34 @@ def main():
         if pf:
             kernels["flash leaves (exact causal)"].update(pf)
 
+        if w["causal"] and not args.no_exact:
+            # what a workgroup of the exact causal kernel costs beyond its key chunks: the same rows cut into
+            # segments of other lengths (a workgroup takes a pair of 256-query tiles (s, T-1-s): 4 (T + 1) chunks
+            # of 64 keys), per-workgroup time = launch time / rounds of workgroups per CU slot, fitted as
+            # a * chunks + c.  c is the fixed cost of a pair of tiles (query rows, first tiles, two epilogues),
+            # which is what separates the leaves from the same kernel on one long sequence
+            slots = 256 * (2 if d == 64 else 1)
+            pts, by_len = [], {}
+            for seg_len in (1024, 2048, 4096, 8192, 16384):
+                if seg_len > n or n % seg_len:
+                    continue
+                t_seg = wl.operands(seg_len, n // seg_len, seg_len, 0)
+                st_seg = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+                ms_seg = time_events(lambda: _lib.check(L.ha_flash_attn_fwd(ctypes.byref(t_seg), 1, st_seg)), 3, torch)
+                tiles = seg_len // 256
+                wgs = b * h * (n // seg_len) * ((tiles + 1) // 2)
+                chunks = 4 * (tiles + 1)
+                pts.append((chunks, ms_seg * 1e3 / (wgs / slots)))
+                seg_flops = b * h * (n // seg_len) * seg_len * seg_len // 2 * 4 * d
+                by_len[str(seg_len)] = {"ms": round(ms_seg, 4), "chunks_per_workgroup": chunks,
+                                        "frac": round(seg_flops / ms_seg / 1e9 / MFMA_PEAK_TFLOPS, 4)}
+            if len(pts) >= 3:
+                mx, my = sum(x for x, _ in pts) / len(pts), sum(y for _, y in pts) / len(pts)
+                slope = sum((x - mx) * (y - my) for x, y in pts) / sum((x - mx) ** 2 for x, _ in pts)
+                kernels["flash leaves (exact causal)"]["by_segment_length"] = {
+                    "segments": by_len, "us_per_chunk": round(slope, 3), "us_per_pair_of_tiles": round(my - slope * mx, 2),
+                    "note": "least-squares line through (chunks per workgroup, launch time / workgroup rounds per CU slot)"}
+
     # the operator-level kernels that the one-call forward does not launch (row gather of the reference's
     # `indexing`, merge of two partial attentions), at this workload's tensor size
     perm = torch.argsort(bq.view(b, h, n), dim=2)
