@@ -356,6 +356,29 @@ def test_module_backward_twice_and_retain_graph(ha):
         assert ((a.double() - b_.double()).norm() / a.double().norm()).item() < 1e-3
 
 
+def test_gradients_of_heads_far_into_large_tensors_equal_those_of_the_heads_alone(ha):
+    """2^20 rows, 24 heads: the last heads start more than 2^31 bytes into q, k, v and the gradients.  A head's
+    gradients inside the big call equal those of the same head in a call of its own (the sampled keys' sums are
+    accumulated with atomics, so to rounding)."""
+    dtype, h, n, d = torch.bfloat16, 24, 1 << 20, 64
+    g = torch.Generator(device="cuda").manual_seed(240)
+    q, k, v = (torch.randn((1, h, n, d), generator=g, device="cuda", dtype=dtype).requires_grad_() for _ in range(3))
+    dout = torch.randn((1, h, n, d), generator=g, device="cuda", dtype=dtype)
+    assert q[0, h - 1].data_ptr() - q.data_ptr() > 1 << 31
+    m = ha.HyperAttention(input_dim=d, block_size=256, sample_size=256, min_seq_len=4096,
+                          rng=torch.Generator().manual_seed(241)).to(device="cuda", dtype=dtype)
+    for causal in (True, False):
+        grads = torch.autograd.grad(m(q, k, v, causal=causal), (q, k, v), dout)
+        for head in (0, h - 1):
+            sl = slice(head, head + 1)
+            q1, k1, v1 = (x[:, sl].detach().clone().requires_grad_() for x in (q, k, v))
+            alone = torch.autograd.grad(m(q1, k1, v1, causal=causal), (q1, k1, v1), dout[:, sl].contiguous())
+            for big, one, what in zip(grads, alone, ("dq", "dk", "dv")):
+                assert torch.isfinite(one.float()).all()
+                rel = (big[:, sl].double() - one.double()).norm() / one.double().norm()
+                assert float(rel) < 1e-3, (causal, head, what, float(rel))
+
+
 def test_module_backward_on_views_agrees_with_operator_by_operator_at_length_32768(ha):
     # two routes to the same gradient at a length the CPU oracle does not reach: the recursion on views
     # with accumulated gradients, and the reference's recursion operator by operator under torch autograd

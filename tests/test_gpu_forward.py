@@ -538,6 +538,24 @@ def test_full_size_c5_properties(ha):
         assert_close(lse[:, sl], rl, f"lse head {head}")
 
 
+@pytest.mark.parametrize("n,h,d,causal,dtype", [(1 << 20, 24, 64, True, torch.bfloat16),
+                                                (1 << 19, 20, 128, False, torch.float16)])
+def test_heads_far_into_large_tensors_equal_the_heads_computed_alone(ha, n, h, d, causal, dtype):
+    """Sequences of 2^20 and 2^19 rows: the last heads of q, k, v start more than 2^31 bytes into their tensors
+    (row numbers and byte offsets beyond 32 bits).  A head's result inside the big call equals, bit for bit, the
+    result of the same head in a call of its own."""
+    g = torch.Generator(device="cuda").manual_seed(230)
+    q, k, v = (torch.randn((1, h, n, d), generator=g, device="cuda", dtype=dtype) for _ in range(3))
+    assert q[0, h - 1].data_ptr() - q.data_ptr() > 1 << 31
+    m, _ = _module(ha, d, dtype, 231, min_seq_len=4096)
+    out, lse = m(q, k, v, causal=causal, return_lse=True)
+    for head in (0, h // 2, h - 1):
+        sl = slice(head, head + 1)
+        o1, l1 = m(q[:, sl].contiguous(), k[:, sl].contiguous(), v[:, sl].contiguous(), causal=causal, return_lse=True)
+        assert torch.isfinite(o1.float()).all()
+        assert torch.equal(out[:, sl], o1) and torch.equal(lse[:, sl], l1), head
+
+
 def test_grouped_query_heads(ha):
     """benchmark configuration c5 shape family (32 query heads on 2 KV heads, d 128, bf16, causal, clustered
     keys) at reduced length: the expanded-KV module call matches the oracle, and the native grouped
