@@ -82,6 +82,9 @@ def test_hash_golden_vectors(ha):
     (1, 20000, 65536, "uniform"),
     # 64 chunks per segment: every scatter workgroup adds up its segment's histograms; 65: the scan launch does
     (2, 64 * 4096, 256, "uniform"), (1, 64 * 4096 + 5, 256, "skew"), (1, 300000, 4096, "uniform"),
+    # beyond 2^24 keys per segment a row number no longer fits beside its digit in the word a chunk is staged
+    # in: the scatter writes each row where it belongs instead
+    (1, (1 << 24) + 3, 256, "uniform"),
 ])
 def test_sort_bit_exact(ha, segs, n, num_keys, kind):
     g = np.random.default_rng(7)
